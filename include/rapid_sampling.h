@@ -1,0 +1,148 @@
+/*
+ * C ABI of the MI355X token sampler (librapid_sampling_hip.so).
+ *
+ * The reference exposes this path only as three ATen functions bound with
+ * pybind11 (/root/reference/sampling.cpp:2-8); it has no C interface.  The
+ * entry points below are what those three functions need from the device
+ * side, with plain pointers and sizes, so that any host (the pybind module in
+ * rapid_sampling_amd/csrc/sampling.cpp, ctypes, cgo, JNI ...) can bind them.
+ *
+ * Conventions: every pointer named *device* is device memory owned by the
+ * caller; `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ * calls enqueue work on `stream` and return without synchronising; the return
+ * value is RS_OK or a negative RS_ERR_* code; nothing throws, and only the
+ * calls that say so allocate.
+ */
+#ifndef RAPID_SAMPLING_H
+#define RAPID_SAMPLING_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RS_OK               0
+#define RS_ERR_VOCAB       -1   /* V <= 0, V > 1048576 or V % 4 != 0   (sampling.cu:461,986)  */
+#define RS_ERR_BATCH       -2   /* B <= 0 or T <= 0                    (sampling.cu:467,992)  */
+#define RS_ERR_TEMPERATURE -3   /* outside [0.001, 1000]               (sampling.cu:474,999)  */
+#define RS_ERR_NULL        -4   /* a required pointer is NULL                                 */
+#define RS_ERR_WORKSPACE   -5   /* workspace too small or misaligned                          */
+#define RS_ERR_ALIGN       -6   /* a row of logits/penalties is not 16-byte aligned           */
+#define RS_ERR_ARG         -7   /* top_k / top_p not normalised (use rs_normalize_args)       */
+#define RS_ERR_LAUNCH      -8   /* the HIP runtime refused the launch                         */
+#define RS_ERR_DEVICE      -9   /* a kernel gave up waiting for its peer workgroups           */
+
+/* Bytes of RNG state per row.  Same size as the reference's
+ * curandStatePhilox4_32_10_t record (sampling.cu:9,141) so that the opaque
+ * tensor returned by setup_rand keeps its shape. */
+#define RS_STATE_BYTES_PER_ROW 64
+
+/* Optional per-row diagnostics (device memory, B records). */
+typedef struct rs_row_diag {
+    float    xmax;        /* row maximum of the scaled logits                 */
+    uint32_t emin_bits;   /* bit pattern of the smallest e in the row         */
+    uint64_t D;           /* sum of the fixed-point weights q over the row    */
+    uint64_t P;           /* ceil(top_p * D)                                  */
+    uint32_t left_bits;   /* lower end of the search interval at loop exit    */
+    uint32_t thr_bits;    /* bit pattern of the smallest kept e               */
+    uint32_t rounds;      /* passes of the threshold search                   */
+    uint32_t n_gt;        /* tokens with e >  threshold                       */
+    uint32_t n_eq;        /* tokens with e == threshold                       */
+    int32_t  index;       /* sampled token                                    */
+    uint64_t G;           /* sum of q over e > threshold                      */
+    uint64_t w_tie;       /* weight of each token with e == threshold         */
+    uint64_t S;           /* G + n_eq * w_tie                                 */
+    uint64_t r;           /* target of the inverse CDF, 1 <= r <= S           */
+} rs_row_diag;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int rs_version(void);
+
+/* Static text for an RS_ERR_* code. */
+const char *rs_error_string(int code);
+
+/*
+ * Host-side argument normalisation of both reference wrappers
+ * (sampling.cu:461-486 and :986-1011): range checks, top_k<=0||top_k>V -> V,
+ * top_p<0||top_p>1 -> 1, top_p==0 -> greedy (top_k=1, top_p=1), and
+ * log2e_inv_temp = (float)(log2(e) / temperature).  No device work.
+ */
+int rs_normalize_args(double temperature, int64_t top_k, double top_p,
+                      int64_t B, int64_t T, int64_t V,
+                      float *log2e_inv_temp, int32_t *top_k_out, float *top_p_out);
+
+/*
+ * Size of the workspace rs_sample needs for a batch of B rows of V tokens.
+ * Replaces the reference's per-call `probs` scratch tensor
+ * (sampling.cu:488,1014); it does not grow with T.
+ */
+int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes);
+
+/*
+ * Zero a freshly allocated workspace (device memory, 256-byte aligned).  Call
+ * once after allocation, and again after a call reported RS_ERR_DEVICE;
+ * rs_sample leaves the workspace ready for the next call on the same stream.
+ */
+int rs_workspace_init(void *workspace_device, size_t bytes, void *stream);
+
+/*
+ * Read back the sticky device error word of a workspace (synchronises
+ * `stream`).  *status is RS_OK or RS_ERR_DEVICE.
+ */
+int rs_workspace_status(const void *workspace_device, int32_t *status, void *stream);
+
+/*
+ * setup_rand (sampling.cu:136-144): initialise B records of RNG state for
+ * Philox4x32-10 with key = seed and subsequence = row, draw counter 0.
+ * state_device: B * RS_STATE_BYTES_PER_ROW bytes.  Runs on `stream` (the
+ * reference uses the null stream).
+ */
+int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
+
+/*
+ * One sampling call; replaces the kernel launches at sampling.cu:500,
+ * :1025 and :1033.
+ *
+ *   logits_device     first sampled row; row b starts b*row_stride floats on.
+ *                     For a (B,T,V) tensor pass base + (T-1)*V and
+ *                     row_stride = T*V (sampling.cu:176,202).
+ *   penalties_device  (B,V) contiguous, updated in place, or NULL for the
+ *                     plain path (sampling.cu:427-437).
+ *   out_device        (B,) int32 sampled token ids.
+ *   rng_state_device  from rs_philox_init; each row's draw counter advances
+ *                     by one.  Ignored (may be NULL) when injected_u is given.
+ *   injected_u_device (B,) floats in (0,1] used instead of the RNG, or NULL.
+ *   top_k, top_p, log2e_inv_temp   as produced by rs_normalize_args:
+ *                     1 <= top_k <= V, 0 < top_p <= 1.
+ *   workspace_device  rs_workspace_bytes(B,V) bytes, initialised once.
+ *   diag_device       B rs_row_diag records, or NULL.
+ *   e_bits_device     (B,V) uint32: bit patterns of e = exp2(x - max) per
+ *                     token, or NULL.  Together with diag.thr_bits this is
+ *                     the kept set {e >= thr}.
+ *
+ * Calls that share a workspace must be ordered on one stream.
+ */
+int rs_sample(const float *logits_device, int64_t row_stride,
+              float *penalties_device, int32_t *out_device,
+              void *rng_state_device, const float *injected_u_device,
+              int32_t B, int32_t V,
+              float presence_penalty, float repetition_penalty, float penalty_decay,
+              float log2e_inv_temp, int32_t top_k, float top_p,
+              void *workspace_device, size_t workspace_bytes,
+              rs_row_diag *diag_device, uint32_t *e_bits_device,
+              void *stream);
+
+/*
+ * Launch-plus-one-read floor: a kernel with rs_sample's grid for (B,V) that
+ * reads every logit once and writes one int per row.  Measurement aid for the
+ * B=1 latency bound; no counterpart in the reference.
+ */
+int rs_floor_read(const float *logits_device, int64_t row_stride, int32_t *out_device,
+                  int32_t B, int32_t V, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

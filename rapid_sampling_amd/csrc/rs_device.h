@@ -1,0 +1,151 @@
+// Device-side building blocks of the MI355X token sampler: canonical
+// element-wise arithmetic, wave64/workgroup reductions and scans, Philox.
+//
+// Arithmetic contract (shared with the CPU oracle used by the tests): every
+// floating-point step is a single IEEE fp32 operation (compile with
+// -ffp-contract=off; fused multiply-adds are explicit), and everything summed
+// across tokens is an integer, so no result depends on how tokens are spread
+// over lanes, waves or workgroups.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rs {
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- scalars --
+
+// NaN -> 0, +-Inf -> +-FLT_MAX            (reference: sampling.cu:131-134)
+__device__ __forceinline__ float sf(float x)
+{
+    float y = (x != x) ? 0.0f : x;
+    return fminf(fmaxf(y, -3.402823466e+38f), 3.402823466e+38f);
+}
+
+// exp2 for d <= 0: floor/fraction split, degree-5 Horner with positive
+// coefficients on the fraction (monotone), exact scale by 2^floor(d), flush to
+// +0 below 2^-64.                          (reference: exp2f at sampling.cu:235)
+__device__ __forceinline__ float exp2c(float d)
+{
+    const float n = __builtin_floorf(d);
+    const float f = d - n;
+    float p = 0x1.e974fap-10f;
+    p = __builtin_fmaf(p, f, 0x1.277856p-7f);
+    p = __builtin_fmaf(p, f, 0x1.c91ce6p-5f);
+    p = __builtin_fmaf(p, f, 0x1.ebdb56p-3f);
+    p = __builtin_fmaf(p, f, 0x1.62e4bap-1f);
+    p = __builtin_fmaf(p, f, 1.0f);
+    const float e = __builtin_ldexpf(p, (int)n);
+    return (n >= -64.0f) ? e : 0.0f;
+}
+
+// Fixed-point weight of a token from the bit pattern of e (0 or 2^-64..1):
+// q = max(1, floor(e * 2^40)).
+__device__ __forceinline__ uint64_t q_of_bits(uint32_t b)
+{
+    const int      ex = (int)(b >> 23);                    // biased exponent, <= 127
+    const uint32_t m  = (b & 0x7FFFFFu) | 0x800000u;       // 24-bit significand
+    const int      sh = ex - 110;                          // e*2^40 = m * 2^sh
+    uint64_t q;
+    if (sh >= 0) q = (uint64_t)m << sh;
+    else         q = (uint64_t)(m >> (sh < -31 ? 31 : -sh));
+    return q ? q : 1;
+}
+
+// ceil(f * s) for a float 0 < f <= 1, exact, clamped to [1, s].
+__device__ inline uint64_t ceil_mul(float f, uint64_t s)
+{
+    if (!(f > 0.0f)) return 1;
+    if (f >= 1.0f) return s;
+    const uint32_t b = __float_as_uint(f);
+    int ex = (int)(b >> 23);
+    uint64_t m = b & 0x7FFFFFu;
+    if (ex == 0) ex = 1; else m |= 0x800000u;
+    const int sh = 150 - ex;                                // f = m * 2^-sh, sh >= 24
+    uint64_t r;
+    if (sh >= 96) r = 1;
+    else {
+        // 128-bit (hi:lo) = m*s + 2^sh - 1, then >> sh
+        uint64_t lo = m * s;
+        uint64_t hi = __umul64hi(m, s);
+        uint64_t add_lo = (sh < 64) ? ((1ull << sh) - 1) : ~0ull;
+        uint64_t add_hi = (sh < 64) ? 0ull : ((1ull << (sh - 64)) - 1);
+        uint64_t lo2 = lo + add_lo;
+        hi += add_hi + (lo2 < lo ? 1 : 0);
+        r = (sh < 64) ? ((lo2 >> sh) | (hi << (64 - sh))) : (hi >> (sh - 64));
+    }
+    if (r < 1) r = 1;
+    if (r > s) r = s;
+    return r;
+}
+
+// 64 random bits -> r in [1, S]
+__device__ __forceinline__ uint64_t r_from_bits(uint64_t u64, uint64_t S)
+{
+    return __umul64hi(u64, S) + 1;
+}
+
+// order-preserving map float -> uint32 (for atomicMax on floats)
+__device__ __forceinline__ uint32_t fkey(float x)
+{
+    const uint32_t b = __float_as_uint(x);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float fkey_inv(uint32_t k)
+{
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
+}
+
+// ---------------------------------------------------------- Philox4x32-10 --
+// Counter-based generator of Salmon et al.; same stream layout as the
+// reference's curand_init(seed, row, 0) (sampling.cu:137): key = seed,
+// counter = (draw_lo, draw_hi, row_lo, row_hi).
+__device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                     uint32_t k0, uint32_t k1, uint32_t out[4])
+{
+#pragma unroll
+    for (int i = 0; i < 10; ++i) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// ------------------------------------------------------ wave64 primitives --
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) { uint32_t o = __shfl_xor(v, off, kWave); v = o > v ? o : v; }
+    return v;
+}
+
+// Inclusive scan over the 64 lanes, ladder 32,16,8,4,2,1 (descending, the
+// order the reference requires of its 16..1 ladder, sampling.cu:48-58; on
+// integers any order is exact).
+__device__ __forceinline__ uint64_t wave_inclusive_scan_u64(uint64_t v, int lane)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint64_t n = __shfl_up(v, off, kWave);
+        if (lane >= off) v += n;
+    }
+    return v;
+}
+
+}  // namespace rs

@@ -1,0 +1,117 @@
+"""ctypes binding of the C ABI in include/rapid_sampling.h, used by the tests to
+call the HIP library directly (torch only provides device memory)."""
+import ctypes as C
+import os
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(ROOT, "rapid_sampling_amd", "librapid_sampling_hip.so")
+HEADER = os.path.join(ROOT, "include", "rapid_sampling.h")
+
+DIAG_DTYPE = np.dtype([
+    ("xmax", "<f4"), ("emin_bits", "<u4"), ("D", "<u8"), ("P", "<u8"),
+    ("left_bits", "<u4"), ("thr_bits", "<u4"), ("rounds", "<u4"), ("n_gt", "<u4"),
+    ("n_eq", "<u4"), ("index", "<i4"), ("G", "<u8"), ("w_tie", "<u8"),
+    ("S", "<u8"), ("r", "<u8"),
+])
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("HIP library not built: run python rapid_sampling_amd/build.py")
+        L = C.CDLL(LIB_PATH)
+        vp, i32, i64, f32, sz = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_size_t
+        L.rs_version.restype = C.c_int
+        L.rs_error_string.restype = C.c_char_p
+        L.rs_error_string.argtypes = [C.c_int]
+        L.rs_normalize_args.restype = C.c_int
+        L.rs_normalize_args.argtypes = [C.c_double, i64, C.c_double, i64, i64, i64,
+                                        C.POINTER(f32), C.POINTER(i32), C.POINTER(f32)]
+        L.rs_workspace_bytes.restype = C.c_int
+        L.rs_workspace_bytes.argtypes = [i32, i32, C.POINTER(sz)]
+        L.rs_workspace_init.restype = C.c_int
+        L.rs_workspace_init.argtypes = [vp, sz, vp]
+        L.rs_workspace_status.restype = C.c_int
+        L.rs_workspace_status.argtypes = [vp, C.POINTER(i32), vp]
+        L.rs_philox_init.restype = C.c_int
+        L.rs_philox_init.argtypes = [vp, C.c_uint64, i32, vp]
+        L.rs_sample.restype = C.c_int
+        L.rs_sample.argtypes = [vp, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
+                                vp, sz, vp, vp, vp]
+        L.rs_floor_read.restype = C.c_int
+        L.rs_floor_read.argtypes = [vp, i64, vp, i32, i32, vp]
+        _lib = L
+    return _lib
+
+
+def normalize(temperature, top_k, top_p, V, B=1, T=1):
+    c, k, p = C.c_float(), C.c_int32(), C.c_float()
+    rc = lib().rs_normalize_args(temperature, top_k, top_p, B, T, V, C.byref(c), C.byref(k), C.byref(p))
+    return rc, c.value, k.value, p.value
+
+
+def workspace_bytes(B, V):
+    n = C.c_size_t()
+    rc = lib().rs_workspace_bytes(B, V, C.byref(n))
+    return rc, n.value
+
+
+class Sampler:
+    """Holds a workspace on the current torch device and calls rs_sample on the
+    current torch stream."""
+
+    def __init__(self, B, V):
+        import torch
+        self.torch = torch
+        rc, n = workspace_bytes(B, V)
+        assert rc == 0
+        self.ws = torch.zeros(n, dtype=torch.int8, device="cuda")
+        self.B, self.V = B, V
+
+    def stream(self):
+        return C.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def status(self):
+        st = C.c_int32(-100)
+        rc = lib().rs_workspace_status(self.ws.data_ptr(), C.byref(st), self.stream())
+        assert rc == 0
+        return st.value
+
+    def sample(self, logits, c, top_k, top_p, *, rng=None, uniforms=None, penalties=None,
+               presence=0.0, repetition=0.0, decay=1.0, want_diag=True, want_e=False):
+        """logits: (B,V) or (B,T,V) float32 cuda tensor.  Returns dict of cpu numpy results."""
+        torch = self.torch
+        if logits.dim() == 3:
+            B, T, V = logits.shape
+            ptr = logits.data_ptr() + 4 * (T - 1) * logits.stride(1)
+            stride = logits.stride(0)
+        else:
+            B, V = logits.shape
+            ptr, stride = logits.data_ptr(), logits.stride(0)
+        if penalties is not None:
+            B = penalties.shape[0]
+        out = torch.full((B,), -7, dtype=torch.int32, device="cuda")
+        diag = torch.zeros((B, DIAG_DTYPE.itemsize), dtype=torch.uint8, device="cuda") if want_diag else None
+        eb = torch.empty((B, V), dtype=torch.int32, device="cuda") if want_e else None
+        rc = lib().rs_sample(ptr, stride, penalties.data_ptr() if penalties is not None else None,
+                             out.data_ptr(), rng.data_ptr() if rng is not None else None,
+                             uniforms.data_ptr() if uniforms is not None else None,
+                             B, V, presence, repetition, decay, c, top_k, top_p,
+                             self.ws.data_ptr(), self.ws.numel(),
+                             diag.data_ptr() if diag is not None else None,
+                             eb.data_ptr() if eb is not None else None, self.stream())
+        res = {"rc": rc}
+        if rc != 0:
+            return res
+        torch.cuda.synchronize()
+        res["out"] = out.cpu().numpy()
+        if want_diag:
+            res["diag"] = diag.cpu().numpy().view(DIAG_DTYPE).reshape(B)
+        if want_e:
+            res["e_bits"] = eb.cpu().numpy().view(np.uint32)
+        return res

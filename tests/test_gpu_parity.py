@@ -1,0 +1,246 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU oracle
+on the same seeded inputs.  Bar: everything here is integer / bit-pattern work,
+so every compared field must be EQUAL (sampled index, threshold, kept set as
+{e >= thr} from bit-identical e, counts, integer masses); updated penalties are
+compared bit for bit as well (the stated bar is 1e-6 relative)."""
+import os
+
+import numpy as np
+import pytest
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+FIELDS = ["xmax", "emin_bits", "D", "P", "left_bits", "thr_bits", "rounds", "n_gt", "n_eq",
+          "index", "G", "w_tie", "S", "r"]
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch
+
+
+def _check(res, ref_out, ref_diag, what):
+    assert res["rc"] == 0, what
+    for f in FIELDS:
+        got, exp = res["diag"][f], ref_diag[f]
+        assert np.array_equal(got, exp), "%s: field %s differs, rows %s" % (what, f, np.nonzero(got != exp)[0][:8])
+    assert np.array_equal(res["out"], ref_out), what
+
+
+def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_np=None, u_np=None,
+              presence=0.0, repetition=0.0, decay=1.0, force_r=None, what=""):
+    if logits_np.ndim == 3:
+        B, T, V = logits_np.shape
+    else:
+        (B, V), T = logits_np.shape, 1
+    rc, c, k, p = capi.normalize(temperature, top_k, top_p, V, B, T)
+    assert rc == 0
+    oc, ok, op = oracle.normalize(temperature, top_k, top_p, V, B, T)
+    assert (c, k, p) == (oc, ok, op)
+    pen_ref = None if pen_np is None else pen_np.copy()
+    ref_out, ref_diag = oracle.sample_batch(logits_np, c, k, p, injected_u=u_np, penalties=pen_ref,
+                                            presence=presence, repetition=repetition, decay=decay)
+    if force_r is None:
+        os.environ.pop("RS_FORCE_R", None)
+    else:
+        os.environ["RS_FORCE_R"] = str(force_r)
+    try:
+        smp = capi.Sampler(B, V)
+        lg = torch.from_numpy(logits_np).cuda()
+        pen = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
+        u = torch.from_numpy(u_np).cuda()
+        print("case", what, "B", B, "T", T, "V", V, "k", k, "p", p, "R", force_r, flush=True)
+        res = smp.sample(lg, c, k, p, uniforms=u, penalties=pen, presence=presence, repetition=repetition,
+                         decay=decay, want_e=True)
+        _check(res, ref_out, ref_diag, what)
+        assert smp.status() == 0
+        if pen is not None:
+            assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32)), what + ": penalties"
+        # second call on the same workspace: it must have been left clean
+        pen2 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
+        res2 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen2, presence=presence, repetition=repetition,
+                          decay=decay)
+        _check(res2, ref_out, ref_diag, what + " (second call)")
+        return res, ref_diag
+    finally:
+        os.environ.pop("RS_FORCE_R", None)
+
+
+def test_c1_uniform_logits_top_p(torch_cuda, oracle):
+    """BASELINE config 1: B=1, V=131072, U[0,1), T=1, top_k=-1, top_p=0.5, one uniform per row."""
+    from tests import capi
+    lg = H.logits_uniform(1, 131072, seed=0)
+    res, ref = _run_case(torch_cuda, oracle, capi, lg, 1.0, -1, 0.5, u_np=H.uniforms(1), what="C1")
+    # kept set = {e >= thr}: e bit-identical and thr identical => identical set
+    row = oracle.sample_row(lg[0], *oracle.normalize(1.0, -1, 0.5, 131072), u=float(H.uniforms(1)[0]), want_e=True)
+    assert np.array_equal(res["e_bits"][0], row["e_bits"])
+    kept_gpu = np.nonzero(res["e_bits"][0] >= res["diag"]["thr_bits"][0])[0]
+    kept_ref = np.nonzero(row["e_bits"] >= row["thr_bits"])[0]
+    assert np.array_equal(kept_gpu, kept_ref) and len(kept_ref) == ref["n_gt"][0] + ref["n_eq"][0]
+
+
+def test_c2_single_row_split(torch_cuda, oracle):
+    """BASELINE config 2: B=1, V=262144, N(0,1)*3, top_p=0.3."""
+    from tests import capi
+    _run_case(torch_cuda, oracle, capi, H.logits_normal(1, 262144, 3.0, seed=3), 1.0, -1, 0.3,
+              u_np=H.uniforms(1, 5), what="C2")
+
+
+def test_c3_mixed_topk_topp(torch_cuda, oracle):
+    """BASELINE config 3: B=64, V=152064, N(0,2) + 10 on 16 ids, T=0.8, top_k=50, top_p=0.9."""
+    from tests import capi
+    _run_case(torch_cuda, oracle, capi, H.logits_spiked(64, 152064, seed=4), 0.8, 50, 0.9,
+              u_np=H.uniforms(64, 6), what="C3")
+
+
+def test_c5_shape_btv_reduced(torch_cuda, oracle):
+    """BASELINE config 5 at reduced B: (B,T,V)=(6,4,1048576), top_k=1024, top_p=0.95; only t=T-1 is read."""
+    from tests import capi
+    lg = H.logits_normal(6 * 4, 1048576, 1.5, seed=7).reshape(6, 4, 1048576)
+    _run_case(torch_cuda, oracle, capi, lg, 1.0, 1024, 0.95, u_np=H.uniforms(6, 8), what="C5r")
+
+
+@pytest.mark.parametrize("R", [1, 2, 4, 8, 16, 32])
+def test_every_slice_length(torch_cuda, oracle, R):
+    """Same rows through every tokens-per-thread variant: identical results."""
+    from tests import capi
+    V = 50304                      # not a multiple of the slice: ragged last workgroup
+    lg = H.logits_normal(5, V, 2.0, seed=10 + R)
+    _run_case(torch_cuda, oracle, capi, lg, 0.7, 100, 0.8, u_np=H.uniforms(5, 11), force_r=R, what="R%d" % R)
+
+
+@pytest.mark.parametrize("V,top_k,top_p,temp", [
+    (4, -1, 1.0, 1.0), (4, 1, 1.0, 1.0), (256, 10, 0.3, 1.0), (1028, -1, 0.999, 2.0),
+    (32768, 1000, 1.0, 0.5), (65536, -1, 0.1, 1.0), (100256, 10000, 0.7, 1.3), (151936, -1, 0.0, 1.0),
+    (1048576, -1, 0.9, 1.0), (1048576, 1048576, 1.0, 1.0),
+])
+def test_grid_of_shapes(torch_cuda, oracle, V, top_k, top_p, temp):
+    from tests import capi
+    B = 3
+    lg = H.logits_normal(B, V, 2.5, seed=V % 97)
+    _run_case(torch_cuda, oracle, capi, lg, temp, top_k, top_p, u_np=H.uniforms(B, V % 13),
+              what="grid V=%d" % V)
+
+
+def test_degenerate_rows(torch_cuda, oracle):
+    """All-equal logits (every token ties), NaN/Inf entries, one dominant token."""
+    from tests import capi
+    V = 4096
+    lg = np.zeros((6, V), dtype=np.float32)
+    lg[1] = 1.5
+    lg[2] = H.logits_normal(1, V, 1.0, seed=1)[0]; lg[2, 7] = np.inf; lg[2, 9] = -np.inf; lg[2, 11] = np.nan
+    lg[3] = H.logits_normal(1, V, 1.0, seed=2)[0]; lg[3, 100] = 300.0
+    lg[4] = -np.inf
+    lg[5] = H.logits_normal(1, V, 1.0, seed=3)[0]; lg[5, :2000] = lg[5, 2000]
+    for (k, p) in [(10, 0.5), (-1, 1.0), (1, 1.0), (-1, 1e-30), (V, 0.9)]:
+        _run_case(torch_cuda, oracle, capi, lg, 1.0, k, p, u_np=H.uniforms(6, 17), what="degenerate k=%s p=%s" % (k, p))
+
+
+def test_uniform_extremes(torch_cuda, oracle):
+    """u -> 0+ picks the first kept token, u = 1 the last one."""
+    from tests import capi
+    V = 8192
+    lg = H.logits_normal(4, V, 2.0, seed=21)
+    u = np.array([1.0, np.nextafter(np.float32(0), np.float32(1)), 1e-30, 0.5], dtype=np.float32)
+    res, ref = _run_case(torch_cuda, oracle, capi, lg, 1.0, 20, 0.9, u_np=u, what="u extremes")
+    e, thr = res["e_bits"], res["diag"]["thr_bits"]
+    kept0 = np.nonzero(e[0] >= thr[0])[0]
+    kept1 = np.nonzero(e[1] >= thr[1])[0]
+    assert res["out"][0] == kept0[-1] and res["out"][1] == kept1[0]
+
+
+def test_penalty_path_single_step(torch_cuda, oracle):
+    from tests import capi
+    B, V = 8, 32768
+    lg = H.logits_normal(B, V, 1.5, seed=30)
+    pen = H.penalties_sparse(B, V, seed=31)
+    pen[0, :64] = np.inf            # masked tokens (penalty +inf)
+    _run_case(torch_cuda, oracle, capi, lg, 0.8, 50, 0.9, pen_np=pen, u_np=H.uniforms(B, 32),
+              presence=0.1, repetition=0.1, decay=0.95, what="penalty step")
+    for R in (1, 4, 16):
+        _run_case(torch_cuda, oracle, capi, lg, 0.8, 50, 0.9, pen_np=pen, u_np=H.uniforms(B, 32),
+                  presence=0.25, repetition=0.1, decay=0.95, force_r=R, what="penalty step R%d" % R)
+
+
+def test_c4_penalty_chain(torch_cuda, oracle):
+    """BASELINE config 4 (B=32, V=131072, 2 % Exp(1) penalties, presence=repetition=0.1, decay=0.95,
+    T=0.8, top_k=50, top_p=0.9) for 24 chained steps on fixed logits; penalties evolve in place on both sides."""
+    torch = torch_cuda
+    from tests import capi
+    B, V, steps = 32, 131072, 24
+    lg_np = H.logits_normal(B, V, 1.5, seed=40)
+    pen_ref = H.penalties_sparse(B, V, seed=41)
+    rc, c, k, p = capi.normalize(0.8, 50, 0.9, V, B, 1)
+    smp = capi.Sampler(B, V)
+    lg = torch.from_numpy(lg_np).cuda()
+    pen = torch.from_numpy(pen_ref.copy()).cuda()
+    for step in range(steps):
+        u_np = H.uniforms(B, 100 + step)
+        ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np, penalties=pen_ref,
+                                                presence=0.1, repetition=0.1, decay=0.95)
+        print("chain step", step, flush=True)
+        res = smp.sample(lg, c, k, p, uniforms=torch.from_numpy(u_np).cuda(), penalties=pen,
+                         presence=0.1, repetition=0.1, decay=0.95)
+        _check(res, ref_out, ref_diag, "chain step %d" % step)
+    got = pen.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), pen_ref.view(np.uint32))
+    rel = np.abs(got - pen_ref) / np.maximum(np.abs(pen_ref), 1e-30)
+    assert rel.max() <= 1e-6
+    assert smp.status() == 0
+
+
+def test_philox_stream_matches_oracle(torch_cuda, oracle):
+    """Without injected uniforms: rs_philox_init + the in-kernel Philox draw give the oracle's indices,
+    call after call (the draw counter advances by one per call)."""
+    torch = torch_cuda
+    from tests import capi
+    import ctypes as C
+    B, V = 16, 16384
+    lg_np = H.logits_normal(B, V, 2.0, seed=50)
+    rc, c, k, p = capi.normalize(1.0, -1, 0.9, V, B, 1)
+    smp = capi.Sampler(B, V)
+    lg = torch.from_numpy(lg_np).cuda()
+    st = torch.empty(B * 64, dtype=torch.int8, device="cuda")
+    assert capi.lib().rs_philox_init(st.data_ptr(), 1234567890123, B, smp.stream()) == 0
+    rng_ref = oracle.rng_init(1234567890123, B)
+    torch.cuda.synchronize()
+    assert np.array_equal(st.cpu().numpy().view(np.uint32).reshape(B, 16), rng_ref)
+    for call in range(4):
+        ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref)
+        res = smp.sample(lg, c, k, p, rng=st)
+        _check(res, ref_out, ref_diag, "philox call %d" % call)
+    assert np.array_equal(st.cpu().numpy().view(np.uint32).reshape(B, 16), rng_ref)
+
+
+def test_chi_square_one_million_draws(torch_cuda, oracle):
+    """1,048,576 Philox-driven draws of one row against the exact renormalised weights w_i / S."""
+    torch = torch_cuda
+    from scipy import stats
+    from tests import capi
+    B, V, calls = 8192, 1024, 128
+    row = H.logits_normal(1, V, 1.5, seed=60)
+    rc, c, k, p = capi.normalize(1.0, 40, 0.9, V, B, 1)
+    d = oracle.sample_row(row[0], c, k, p, u=0.5, want_e=True)
+    e, thr = d["e_bits"], d["thr_bits"]
+    w = np.where(e > thr, oracle.q_of(e.view(np.float32)).astype(np.float64), 0.0)
+    w[e == thr] = float(d["w_tie"])
+    assert abs(w.sum() - float(d["S"])) <= 1e-6 * float(d["S"])
+    lg = torch.from_numpy(np.repeat(row, B, axis=0)).cuda()
+    smp = capi.Sampler(B, V)
+    st = torch.empty(B * 64, dtype=torch.int8, device="cuda")
+    assert capi.lib().rs_philox_init(st.data_ptr(), 7, B, smp.stream()) == 0
+    counts = np.zeros(V, dtype=np.int64)
+    for _ in range(calls):
+        res = smp.sample(lg, c, k, p, rng=st, want_diag=False)
+        assert res["rc"] == 0
+        counts += np.bincount(res["out"], minlength=V)
+    n = B * calls
+    assert counts[w == 0].sum() == 0, "a dropped token was sampled"
+    keep = w > 0
+    chi2, pval = stats.chisquare(counts[keep], n * w[keep] / w.sum())
+    print("chi2", chi2, "dof", keep.sum() - 1, "p", pval)
+    assert pval > 0.01
