@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Benchmark of the sampling hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload of the headline number (BASELINE.json configs[1]): B=1, V=262144,
+logits N(0,1)*3 (seeded, synthetic), temperature 1.0, top_k -1, top_p 0.3; a
+"step" is one call of batch_sampling_temperature_topk_topp through the drop-in
+Python module with the logits already resident in HBM.  `value` is the median
+device-side time of one call in microseconds (HIP events around each call on the
+stream the kernel runs on).  Next to it, in the same JSON line:
+
+  latency    the launch-plus-one-read floor kernel timed the same way, the
+             ratio to it, and the wall-clock "call + synchronize" time the
+             reference's own bench measures (reference bench.py:84-92)
+  roofline   the bandwidth-bound configuration (BASELINE.json configs[4]):
+             logits (128,4,1048576) fp32 = 2 GiB resident, top_k 1024,
+             top_p 0.95; algorithmic bytes = 4*V per sampled row
+  cpu_baseline  the CPU oracle (single thread) on a bounded sample of the
+             headline workload; cpu_torch is torch-CPU softmax/sort/cumsum/
+             multinomial on the same row with its thread count
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, vendor figure
+
+
+def event_times_us(torch, fn, steps, warmup):
+    """Median / mean device time of fn() in microseconds, from one event pair per call
+    recorded on the current stream, plus the wall-clock time of the whole timed region."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us = [s.elapsed_time(e) * 1000.0 for s, e in zip(starts, ends)]
+    return us, wall
+
+
+def block_time_us(torch, fn, steps, warmup):
+    """Average device time per call over `steps` back-to-back calls (one event pair around all)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(steps):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) * 1000.0 / steps
+
+
+def sync_call_us(torch, fn, reps):
+    """Wall clock of call + synchronize, as the reference's bench takes it."""
+    out = []
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        out.append((time.perf_counter() - t0) * 1e6)
+    return out
+
+
+def pct(xs, q):
+    xs = sorted(xs)
+    return xs[min(len(xs) - 1, int(q * len(xs)))]
+
+
+def cpu_baselines(logits_row_np, temperature, top_k, top_p, budget_s=12.0):
+    """Oracle (port, 1 thread) and torch-CPU sort/cumsum/multinomial on the headline row."""
+    import numpy as np
+    import torch
+    from oracle import oracle as O
+
+    V = logits_row_np.shape[0]
+    c, k, p = O.normalize(temperature, top_k, top_p, V)
+    O.sample_row(logits_row_np, c, k, p, u=0.5)
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        O.sample_row(logits_row_np, c, k, p, u=0.25 + 0.5 * ((n * 0.618) % 1.0))
+        n += 1
+    oracle_us = (time.perf_counter() - t0) / n * 1e6
+    port = {"value": round(oracle_us, 1), "unit": "us/call", "cores": 1, "kind": "port",
+            "sample": "%d calls of the oracle on the same B=1, V=%d row (%.0f s)" % (n, V, budget_s)}
+
+    x = torch.from_numpy(logits_row_np)[None, :]
+    kk = V if top_k <= 0 or top_k > V else top_k
+
+    def torch_cpu():
+        probs = torch.softmax(x / temperature, dim=-1)
+        sp, si = torch.sort(probs, dim=-1, descending=True)
+        cs = torch.cumsum(sp, dim=-1)
+        keep = (cs - sp < top_p) & (torch.arange(V)[None, :] < kk)
+        w = torch.where(keep, sp, torch.zeros_like(sp))
+        j = torch.multinomial(w, 1)
+        return si.gather(-1, j)
+
+    torch_cpu()
+    m, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s / 2:
+        torch_cpu()
+        m += 1
+    tus = (time.perf_counter() - t0) / m * 1e6
+    tc = {"value": round(tus, 1), "unit": "us/call", "cores": torch.get_num_threads(),
+          "host_cpus": os.cpu_count(), "kind": "torch-cpu softmax/sort/cumsum/multinomial",
+          "sample": "%d calls on the same row" % m}
+    return port, tc
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--skip-bandwidth", action="store_true", help="skip the 2 GiB bandwidth configuration")
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--bandwidth-steps", type=int, default=20)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (rows shard over GPUs without communication; "
+              "no multi-GPU path is part of it). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import rapid_sampling_amd as sample
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    # ---- headline: B=1, V=262144 -------------------------------------------
+    V, temperature, top_k, top_p = 262144, 1.0, -1, 0.3
+    row_np = (np.random.default_rng(1).standard_normal(V, dtype=np.float32) * np.float32(3.0)).astype(np.float32)
+    logits = torch.from_numpy(row_np)[None, :].to(dev)
+    states = sample.setup_rand(0, 1)
+
+    def call():
+        return sample.batch_sampling_temperature_topk_topp(logits, states, temperature, top_k, top_p)
+
+    def floor():
+        return sample.floor_read(logits)
+
+    us, wall = event_times_us(torch, call, args.steps, args.warmup)
+    p50 = statistics.median(us)
+    floor_us, _ = event_times_us(torch, floor, min(args.steps, 2000), min(args.warmup, 100))
+    floor_p50 = statistics.median(floor_us)
+    sync_us = sync_call_us(torch, call, 200)
+    b2b_us = block_time_us(torch, call, min(args.steps, 2000), 20)
+    floor_b2b_us = block_time_us(torch, floor, min(args.steps, 2000), 20)
+
+    result = {
+        "metric": "p50 us/call (B=1,V=256K); HBM GB/s vs peak at B=128x4,V=1M",
+        "value": round(p50, 3),
+        "unit": "us/call",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "B=1, V=262144, logits N(0,1)*3 seed 1, temperature 1.0, top_k -1, top_p 0.3, "
+                               "Philox draws, drop-in Python call"},
+        "latency": {
+            "p50_us": round(p50, 3), "p10_us": round(pct(us, 0.10), 3), "p90_us": round(pct(us, 0.90), 3),
+            "back_to_back_us": round(b2b_us, 3),
+            "floor_p50_us": round(floor_p50, 3), "floor_back_to_back_us": round(floor_b2b_us, 3),
+            "ratio_to_floor": round(p50 / floor_p50, 3),
+            "call_plus_sync_p50_us": round(statistics.median(sync_us), 2),
+            "reference_call_plus_sync_us": 220.3,
+            "reference_note": "reference README.md:21-31: same B, V, top_p, top_k, logits U[0,1)*4, unnamed NVIDIA GPU",
+        },
+    }
+
+    # ---- bandwidth: (128, 4, 1048576), 2 GiB resident ------------------------
+    if not args.skip_bandwidth:
+        Bb, Tb, Vb = 128, 4, 1048576
+        g = torch.Generator(device=dev)
+        g.manual_seed(5)
+        big = torch.randn((Bb, Tb, Vb), generator=g, device=dev, dtype=torch.float32)
+        big.mul_(1.5)
+        st_b = sample.setup_rand(1, Bb * Tb)
+
+        def call_btv():
+            return sample.batch_sampling_temperature_topk_topp(big, st_b, 1.0, 1024, 0.95)
+
+        flat = big.view(Bb * Tb, Vb)
+
+        def call_flat():
+            return sample.batch_sampling_temperature_topk_topp(flat, st_b, 1.0, 1024, 0.95)
+
+        def floor_btv():
+            return sample.floor_read(big)
+
+        t_btv = block_time_us(torch, call_btv, args.bandwidth_steps, 3)
+        t_flat = block_time_us(torch, call_flat, max(2, args.bandwidth_steps // 2), 2)
+        t_floor = block_time_us(torch, floor_btv, args.bandwidth_steps, 3)
+        bytes_btv = Bb * Vb * 4
+        bytes_flat = Bb * Tb * Vb * 4
+        ach = bytes_btv / (t_btv * 1e-6) / 1e9
+        result["roofline"] = {
+            "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+            "workload": "(B,T,V)=(128,4,1048576) N(0,1.5), top_k 1024, top_p 0.95: 128 sampled rows of 4 MiB, "
+                        "stride T*V, algorithmic bytes 4*V per row = 512 MiB per call",
+            "us_per_call": round(t_btv, 2), "rows_per_s": round(Bb / (t_btv * 1e-6), 1),
+            "read_once_floor_GBs": round(bytes_btv / (t_floor * 1e-6) / 1e9, 1),
+            "flattened_512_rows": {"us_per_call": round(t_flat, 2),
+                                   "achieved": round(bytes_flat / (t_flat * 1e-6) / 1e9, 1),
+                                   "rows_per_s": round(Bb * Tb / (t_flat * 1e-6), 1)},
+        }
+        del big, flat
+
+    # ---- CPU baselines ------------------------------------------------------
+    if not args.skip_cpu:
+        port, tc = cpu_baselines(row_np, temperature, top_k, top_p)
+        result["cpu_baseline"] = port
+        result["cpu_torch"] = tc
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

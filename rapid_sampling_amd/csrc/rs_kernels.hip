@@ -5,17 +5,24 @@
 // in registers for the whole call, so the row is read from HBM exactly once
 // and every later pass runs out of the register file.  Workgroups of a
 // cluster meet at device-scope barriers (an arrival counter per row in the
-// workspace); everything they exchange is an integer sum, a max or a min, so
-// the result does not depend on G, R or arrival order.
+// workspace); everything they exchange is an integer sum or a max, so the
+// result does not depend on G, R or arrival order.
 //
 // Steps per row (reference lines in /root/reference/sampling.cu):
-//   1  x = sf((sf(l) - pen) * c), row max            :208-227, :547-559
-//   2  e = exp2(x - max) kept as bit patterns, D      :228-258
-//   3  4-way threshold search on bit patterns         :261-329
-//   4  smallest kept e, counts and mass above it      :332-355
-//   5  tie weight                                     :365-371
-//   6  inverse-CDF pick in index order                :374-426
-//   7  penalty decay + one-hot add, in place          :427-437
+//   1  x = sf((sf(l) - pen) * c), row max                         :208-227, :547-559
+//   2  e = exp2(x - max) kept as bit patterns                     :228-258
+//   3  threshold = largest t with count{e>=t} >= top_k or mass{e>=t} >= top_p*D.
+//      The reference finds it by a 4-way search on bit patterns with one pass
+//      over the row per step (:261-329); here it is a radix selection on the
+//      same bit patterns: a (count, mass) histogram over the top 11 bits of
+//      the key summed across the cluster, then either the few tokens of the
+//      boundary bin are gathered and resolved in LDS, or the next 10 / 9 bits
+//      are histogrammed the same way.  Same threshold, 3 barriers instead of
+//      one per search step.
+//   4  counts and mass above / at the threshold                   :332-355
+//   5  tie weight                                                 :365-371
+//   6  inverse-CDF pick in index order                            :374-426
+//   7  penalty decay + one-hot add, in place, from registers      :427-437
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -28,7 +35,11 @@ namespace rs {
 constexpr int      kThreads   = 256;          // 4 waves, one per SIMD
 constexpr int      kWaves     = kThreads / kWave;
 constexpr int      kMaxParts  = 256;          // workgroups per row, at most
-constexpr int      kMaxRounds = 24;           // search passes, at most (range <= 2^30)
+constexpr int      kNB1       = 1280;         // level-1 bins (1026 used), 5 per thread
+constexpr int      kNB2       = 1024;         // level-2 bins, 4 per thread
+constexpr int      kNB3       = 512;          // level-3 bins, 2 per thread
+constexpr int      kCap       = 1024;         // tokens of a boundary bin that are gathered
+constexpr uint32_t kOneBits   = 0x3F800000u;  // bits(1.0f) = bits(e_max)
 constexpr uint64_t kSpinLimit = 200000000ull; // 2 s of the 100 MHz wall clock
 
 struct alignas(256) WsHeader {
@@ -38,23 +49,20 @@ struct alignas(256) WsHeader {
     uint32_t pad[61];
 };
 
-struct RoundSlot {
-    uint32_t c[3];
-    uint32_t pad;
-    uint64_t m[3];
-};
-
+// Per-row record.  Everything a call reads before writing it is zero when the
+// call starts: the call itself re-zeroes what it used before it ends.
 struct alignas(256) RowCtl {
     uint32_t arrive;      // barrier arrivals so far
     uint32_t done;        // workgroups finished with this row
     uint32_t maxkey;      // max of fkey(x)
-    uint32_t emin_inv;    // max of ~bits(e)            -> emin
-    uint32_t thr_inv;     // max of ~bits(e), e >= left -> smallest kept e
-    uint32_t n_gt, n_eq;
-    int32_t  index;
-    uint64_t D, G;
-    RoundSlot round[kMaxRounds];
-    uint64_t W[kMaxParts];   // kept weight of each workgroup's slice
+    uint32_t cursor;      // fill of cand[]
+    uint32_t index_p1;    // sampled token + 1, once known
+    uint32_t pad[3];
+    uint64_t A[kMaxParts];      // per workgroup: mass above the gathered bin, or kept weight
+    uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
+    uint32_t c1[kNB1]; uint64_t m1[kNB1];
+    uint32_t c2[kNB2]; uint64_t m2[kNB2];
+    uint32_t c3[kNB3]; uint64_t m3[kNB3];
 };
 
 struct Params {
@@ -77,52 +85,53 @@ struct Params {
 
 #define RS_AGENT __HIP_MEMORY_SCOPE_AGENT
 
+// Everything workgroups exchange goes through relaxed device-scope atomics
+// (they act at the level all XCDs share); "my contributions are performed" is
+// a wait on the vector-memory counter, not a cache write-back.
 template <typename T> __device__ __forceinline__ T a_load(const T *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, RS_AGENT); }
 template <typename T> __device__ __forceinline__ void a_store(T *p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, RS_AGENT); }
 template <typename T> __device__ __forceinline__ void a_add(T *p, T v) { __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, RS_AGENT); }
 template <typename T> __device__ __forceinline__ void a_max(T *p, T v) { __hip_atomic_fetch_max(p, v, __ATOMIC_RELAXED, RS_AGENT); }
+__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Hides a register from the optimiser for one use, so that work derived from
 // the resident tokens (their fixed-point weights) is redone in each pass
-// instead of being hoisted out of the loops and kept in two more registers
-// per token.
+// instead of being hoisted and kept in two more registers per token.
 __device__ __forceinline__ uint32_t opaque(uint32_t v)
 {
     asm volatile("" : "+v"(v));
     return v;
 }
 
-// Workgroup-local staging in LDS.
+// Radix digits of a token, most significant first, on key' = bits(1.0) - bits(e)
+// (0 for the largest e, growing as e falls; e == 0 lands in bin 1025).
+__device__ __forceinline__ uint32_t digit1(uint32_t b) { return min((kOneBits - b) >> 19, 1025u); }
+__device__ __forceinline__ uint32_t digit2(uint32_t b) { return ((kOneBits - b) >> 9) & 1023u; }
+__device__ __forceinline__ uint32_t digit3(uint32_t b) { return (kOneBits - b) & 511u; }
+
+struct Found {               // result of a histogram scan (uniform over the workgroup)
+    uint32_t bin;            // first bin at which the kept set becomes sufficient
+    uint32_t cnt_above;      // tokens in bins before it (plus the carried offset)
+    uint32_t cnt_bin;        // tokens in it
+    uint64_t mass_above;
+    uint64_t mass_bin;
+};
+
 struct Lds {
+    uint32_t hc[kNB1];
+    uint64_t hm[kNB1];
+    uint64_t cand[kCap];
     uint64_t u64[kWaves * 4];
     uint32_t u32[kWaves * 4];
-    uint64_t bc64[8];       // broadcast slots
+    uint64_t bc64[8];
     uint32_t bc32[8];
     uint64_t wj[kWaves][32];
     uint64_t tj[32];
+    Found    found;
+    uint64_t D, P;
+    uint32_t ctr;
     int      abort;
 };
-
-// Sum of (c0,c1,c2 | m0,m1,m2) over the workgroup; result valid in thread 0.
-__device__ __forceinline__ void block_sum3(Lds &s, uint32_t c[3], uint64_t m[3], int lane, int wave)
-{
-#pragma unroll
-    for (int i = 0; i < 3; ++i) { c[i] = wave_sum(c[i]); m[i] = wave_sum(m[i]); }
-    __syncthreads();
-    if (lane == 0) {
-#pragma unroll
-        for (int i = 0; i < 3; ++i) { s.u32[wave * 4 + i] = c[i]; s.u64[wave * 4 + i] = m[i]; }
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-#pragma unroll
-        for (int i = 0; i < 3; ++i) {
-            uint32_t cc = 0; uint64_t mm = 0;
-            for (int w = 0; w < kWaves; ++w) { cc += s.u32[w * 4 + i]; mm += s.u64[w * 4 + i]; }
-            c[i] = cc; m[i] = mm;
-        }
-    }
-}
 
 __device__ __forceinline__ uint32_t block_max_u32(Lds &s, uint32_t v, int lane, int wave)
 {
@@ -148,19 +157,33 @@ __device__ __forceinline__ uint64_t block_sum_u64(Lds &s, uint64_t v, int lane, 
     return r;
 }
 
-// Meet the other workgroups of the row.  Thread 0 has issued this
-// workgroup's contributions (relaxed device-scope atomics) before the call.
-// Returns false when the wait gave up (sticky error set).
-__device__ __forceinline__ bool cluster_barrier(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t target)
+// two sums at once
+__device__ __forceinline__ void block_sum2_u64(Lds &s, uint64_t &a, uint64_t &b, int lane, int wave)
 {
+    a = wave_sum(a); b = wave_sum(b);
+    __syncthreads();
+    if (lane == 0) { s.u64[wave * 2] = a; s.u64[wave * 2 + 1] = b; }
+    __syncthreads();
+    a = 0; b = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) { a += s.u64[w * 2]; b += s.u64[w * 2 + 1]; }
+}
+
+// Meet the other workgroups of the row.  Every thread's contributions are
+// relaxed device-scope atomics issued before the call; each thread waits for
+// its own to be performed, then thread 0 arrives and polls.  Returns false
+// when the wait gave up (sticky error set).
+__device__ __forceinline__ bool cluster_barrier(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t G, uint32_t target)
+{
+    if (G == 1) { __syncthreads(); return true; }
+    wait_vmem();
     __syncthreads();
     if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(&rc->arrive, 1u, __ATOMIC_RELEASE, RS_AGENT);
+        __hip_atomic_fetch_add(&rc->arrive, 1u, __ATOMIC_RELAXED, RS_AGENT);
         const uint64_t t0 = wall_clock64();
         uint32_t spins = 0;
-        while (__hip_atomic_load(&rc->arrive, __ATOMIC_ACQUIRE, RS_AGENT) < target) {
-            __builtin_amdgcn_s_sleep(1);
-            if ((++spins & 255u) == 0 && wall_clock64() - t0 > kSpinLimit) {
+        while (a_load(&rc->arrive) < target) {
+            if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
                 a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
                 s.abort = 1;
                 break;
@@ -169,6 +192,88 @@ __device__ __forceinline__ bool cluster_barrier(Lds &s, RowCtl *rc, WsHeader *hd
     }
     __syncthreads();
     return s.abort == 0;
+}
+
+__device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)
+{
+    for (int b = threadIdx.x; b < nb; b += kThreads) { s.hc[b] = 0; s.hm[b] = 0; }
+}
+__device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint64_t q)
+{
+    atomicAdd(&s.hc[bin], 1u);
+    atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[bin]), (unsigned long long)q);
+}
+
+// Re-zero this workgroup's share of a global histogram (the cluster splits the bins).
+__device__ __forceinline__ void zero_slice(uint32_t *gc, uint64_t *gm, uint32_t nb, uint32_t part, uint32_t G)
+{
+    const uint32_t lo = (uint32_t)(((uint64_t)nb * part) / G), hi = (uint32_t)(((uint64_t)nb * (part + 1)) / G);
+    for (uint32_t b = lo + threadIdx.x; b < hi; b += kThreads) { a_store(&gc[b], 0u); a_store(&gm[b], (uint64_t)0); }
+}
+
+// Sum the workgroup histograms of a cluster: add mine into the row's global
+// bins, meet, read the totals back into LDS.  A cluster of one keeps its own.
+__device__ __forceinline__ bool hist_combine(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t G, uint32_t target,
+                                             uint32_t *gc, uint64_t *gm, int nb)
+{
+    __syncthreads();
+    if (G == 1) return true;
+    for (int b = threadIdx.x; b < nb; b += kThreads) {
+        const uint32_t c = s.hc[b];
+        if (c) { a_add(&gc[b], c); a_add(&gm[b], s.hm[b]); }
+    }
+    if (!cluster_barrier(s, rc, hdr, G, target)) return false;
+    for (int b = threadIdx.x; b < nb; b += kThreads) { s.hc[b] = a_load(&gc[b]); s.hm[b] = a_load(&gm[b]); }
+    __syncthreads();
+    return true;
+}
+
+// Scan the LDS histogram in bin order and find the first bin at which
+// (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).  With
+// first != 0 the total mass of the histogram is the row total D and P is
+// derived from it here.  Thread t owns bins [t*PER, (t+1)*PER).
+template <int PER>
+__device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0, uint64_t top_k, float top_p,
+                                           bool first, int lane, int wave)
+{
+    const int t = threadIdx.x;
+    uint32_t c[PER]; uint64_t m[PER];
+    uint32_t cs = 0; uint64_t ms = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) { c[i] = s.hc[t * PER + i]; m[i] = s.hm[t * PER + i]; cs += c[i]; ms += m[i]; }
+    // inclusive scan over threads
+    uint64_t mi = wave_inclusive_scan_u64(ms, lane);
+    uint64_t ci = wave_inclusive_scan_u64((uint64_t)cs, lane);
+    __syncthreads();
+    if (lane == kWave - 1) { s.u64[wave * 2] = mi; s.u64[wave * 2 + 1] = ci; }
+    __syncthreads();
+    uint64_t moff = 0, coff = 0, mtot = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        if (w < wave) { moff += s.u64[w * 2]; coff += s.u64[w * 2 + 1]; }
+        mtot += s.u64[w * 2];
+    }
+    if (first) {
+        if (t == 0) { s.D = mtot; s.P = ceil_mul(top_p, mtot); }
+        __syncthreads();
+    }
+    const uint64_t P = s.P;
+    uint64_t rcnt = (uint64_t)cnt0 + coff + ci - cs;     // count before my first bin
+    uint64_t rm = mass0 + moff + mi - ms;                // mass before my first bin
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const bool before = rcnt >= top_k || rm >= P;
+        const uint64_t nc = rcnt + c[i], nm = rm + m[i];
+        const bool after = nc >= top_k || nm >= P;
+        if (!before && after) {
+            s.found.bin = (uint32_t)(t * PER + i);
+            s.found.cnt_above = (uint32_t)rcnt; s.found.cnt_bin = c[i];
+            s.found.mass_above = rm; s.found.mass_bin = m[i];
+        }
+        rcnt = nc; rm = nm;
+    }
+    __syncthreads();
+    return s.found;
 }
 
 template <int R, bool PEN>
@@ -226,131 +331,195 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
         const uint32_t k = block_max_u32(s, fkey(lmax), lane, wave);
-        if (tid == 0) a_max(&rc->maxkey, k);
+        if (G > 1) {
+            if (tid == 0) a_max(&rc->maxkey, k);
+            if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
+            if (tid == 0) s.bc32[1] = a_load(&rc->maxkey);
+        } else if (tid == 0) s.bc32[1] = k;
+        lds_hist_zero(s, kNB1);
+        __syncthreads();
     }
-    if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
-    if (tid == 0) s.bc32[1] = a_load(&rc->maxkey);
-    __syncthreads();
     const float xmax = fkey_inv(s.bc32[1]);
 
-    // ---- 2. e = exp2(x - max) in place, D, emin ---------------------------
-    {
-        uint64_t dl = 0;
-        uint32_t einv = 0;
+    // ---- 2. e = exp2(x - max) in place; level-1 histogram ------------------
 #pragma unroll
-        for (int j = 0; j < R; ++j) {
+    for (int j = 0; j < R; ++j) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t b = __float_as_uint(exp2c(__uint_as_float(eb[j * 4 + k]) - xmax));
-                eb[j * 4 + k] = b;
-                if (j < nv) { dl += q_of_bits(b); einv = max(einv, ~b); }
-            }
-        }
-        dl = block_sum_u64(s, dl, lane, wave);
-        einv = block_max_u32(s, einv, lane, wave);
-        if (tid == 0) { a_add(&rc->D, dl); a_max(&rc->emin_inv, einv); }
-        if (p.e_bits) {
-            uint4 *dst = reinterpret_cast<uint4 *>(p.e_bits + (int64_t)row * p.V);
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-                if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t b = __float_as_uint(exp2c(__uint_as_float(eb[j * 4 + k]) - xmax));
+            eb[j * 4 + k] = b;
+            if (j < nv) lds_hist_add(s, digit1(b), q_of_bits(b));
         }
     }
-    if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
-    if (tid == 0) { s.bc64[0] = a_load(&rc->D); s.bc32[2] = ~a_load(&rc->emin_inv); }
-    __syncthreads();
-    const uint64_t D = s.bc64[0];
-    const uint32_t emin = s.bc32[2];
-    const uint64_t P = ceil_mul(p.top_p, D);
+    if (p.e_bits) {
+        uint4 *dst = reinterpret_cast<uint4 *>(p.e_bits + (int64_t)row * p.V);
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+            if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
+    }
+    if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->c1, rc->m1, kNB1)) return;
     const uint64_t top_k = (uint64_t)p.top_k;
 
-    // ---- 3. quaternary search on bit patterns ------------------------------
-    // e_max is exp2c(0) = 1.0 exactly, so the upper end starts at bits(1.0)+1.
-    uint32_t left = emin, right = 0x3F800000u + 1u;
-    uint64_t cnt_x = (uint64_t)p.V, mass_x = D;
-    uint32_t rounds = 0;
-    while ((cnt_x > top_k || mass_x > P) && left < right - 1) {
-        if (rounds >= (uint32_t)kMaxRounds) {            // cannot happen: the range shrinks 4x per pass
-            if (tid == 0) a_store(&p.hdr->error, (int32_t)RS_ERR_DEVICE);
-            return;
-        }
-        const uint32_t pz = (left + right) / 2;
-        const uint32_t py = (left + pz) / 2;
-        const uint32_t pw = (pz + right) / 2;
-        uint32_t c[3] = {0, 0, 0};
-        uint64_t m[3] = {0, 0, 0};
+    // ---- 3. radix selection of the threshold -------------------------------
+    Found f = hist_find<kNB1 / kThreads>(s, 0u, 0ull, top_k, p.top_p, true, lane, wave);
+    const uint64_t D = s.D, P = s.P;
+    const uint32_t b1 = f.bin;
+    uint32_t b2 = 0, b3 = 0;
+    uint32_t levels = 1;                     // histogram levels summed over the cluster
+    if (f.cnt_bin > (uint32_t)kCap) {
+        lds_hist_zero(s, kNB2);
+        __syncthreads();
 #pragma unroll
-        for (int j = 0; j < R; ++j) {
+        for (int j = 0; j < R; ++j)
             if (j < nv) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t b = opaque(eb[j * 4 + k]);
-                    const uint64_t q = q_of_bits(b);
-                    if (b >= py) { c[0]++; m[0] += q; }
-                    if (b >= pz) { c[1]++; m[1] += q; }
-                    if (b >= pw) { c[2]++; m[2] += q; }
+                    if (digit1(b) == b1) lds_hist_add(s, digit2(b), q_of_bits(b));
                 }
             }
-        }
-        block_sum3(s, c, m, lane, wave);
-        RoundSlot *slot = &rc->round[rounds];
-        if (tid == 0) {
+        if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->c2, rc->m2, kNB2)) return;
+        if (G > 1) zero_slice(rc->c1, rc->m1, kNB1, part, G);   // everyone has read level 1 by now
+        f = hist_find<kNB2 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
+        b2 = f.bin;
+        levels = 2;
+        if (f.cnt_bin > (uint32_t)kCap) {
+            lds_hist_zero(s, kNB3);
+            __syncthreads();
 #pragma unroll
-            for (int i = 0; i < 3; ++i) { a_add(&slot->c[i], c[i]); a_add(&slot->m[i], m[i]); }
-        }
-        if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
-        if (tid == 0) {
+            for (int j = 0; j < R; ++j)
+                if (j < nv) {
 #pragma unroll
-            for (int i = 0; i < 3; ++i) { s.bc32[4 + i] = a_load(&slot->c[i]); s.bc64[4 + i] = a_load(&slot->m[i]); }
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t b = opaque(eb[j * 4 + k]);
+                        if (digit1(b) == b1 && digit2(b) == b2) lds_hist_add(s, digit3(b), q_of_bits(b));
+                    }
+                }
+            if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->c3, rc->m3, kNB3)) return;
+            if (G > 1) zero_slice(rc->c2, rc->m2, kNB2, part, G);
+            f = hist_find<kNB3 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
+            b3 = f.bin;
+            levels = 3;
+        }
+    }
+    // global histogram of the last summed level: re-zeroed after the next barrier
+    uint32_t *const zc = levels == 1 ? rc->c1 : levels == 2 ? rc->c2 : rc->c3;
+    uint64_t *const zm = levels == 1 ? rc->m1 : levels == 2 ? rc->m2 : rc->m3;
+    const uint32_t znb = levels == 1 ? kNB1 : levels == 2 ? kNB2 : kNB3;
+
+    // Tokens still undistinguished share digits 1..levels.  If they are few,
+    // gather them (bits and index) so that every workgroup can finish alone.
+    auto in_bin = [&](uint32_t b) -> bool {
+        if (digit1(b) != b1) return false;
+        if (levels >= 2 && digit2(b) != b2) return false;
+        if (levels >= 3 && digit3(b) != b3) return false;
+        return true;
+    };
+    auto above_bin = [&](uint32_t b) -> bool {         // larger e than every token of the bin
+        const uint32_t d1 = digit1(b);
+        if (d1 != b1) return d1 < b1;
+        if (levels < 2) return false;
+        const uint32_t d2 = digit2(b);
+        if (d2 != b2) return d2 < b2;
+        if (levels < 3) return false;
+        return digit3(b) < b3;
+    };
+    const bool gather = f.cnt_bin <= (uint32_t)kCap;
+    uint32_t ncand = 0;
+    if (gather) {
+        uint64_t amass = 0;
+        uint32_t mycnt = 0;
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+            if (j < nv) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t b = opaque(eb[j * 4 + k]);
+                    if (above_bin(b)) amass += q_of_bits(b);
+                    if (in_bin(b)) mycnt++;
+                }
+            }
+        amass = block_sum_u64(s, amass, lane, wave);
+        if (tid == 0) s.ctr = 0;
+        __syncthreads();
+        uint32_t myslot = 0;
+        if (mycnt) myslot = atomicAdd(&s.ctr, mycnt);
+        __syncthreads();
+        ncand = f.cnt_bin;
+        if (G > 1) {
+            if (tid == 0) {
+                const uint32_t n = s.ctr;
+                s.bc32[2] = n ? __hip_atomic_fetch_add(&rc->cursor, n, __ATOMIC_RELAXED, RS_AGENT) : 0u;
+                a_store(&rc->A[part], amass);
+            }
+            __syncthreads();
+            uint32_t o = s.bc32[2] + myslot;
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+                if (j < nv) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t b = opaque(eb[j * 4 + k]);
+                        if (in_bin(b)) {
+                            const uint32_t idx = (base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)k;
+                            if (o < (uint32_t)kCap) a_store(&rc->cand[o], ((uint64_t)b << 32) | idx);
+                            ++o;
+                        }
+                    }
+                }
+            if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
+            for (uint32_t i = tid; i < ncand; i += kThreads) s.cand[i] = a_load(&rc->cand[i]);
+            zero_slice(zc, zm, znb, part, G);
+        } else {
+            uint32_t o = myslot;
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+                if (j < nv) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t b = opaque(eb[j * 4 + k]);
+                        if (in_bin(b)) {
+                            const uint32_t idx = (base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)k;
+                            if (o < (uint32_t)kCap) s.cand[o] = ((uint64_t)b << 32) | idx;
+                            ++o;
+                        }
+                    }
+                }
+            if (tid == 0) s.bc64[7] = amass;
         }
         __syncthreads();
-        const uint64_t cy = s.bc32[4], cz = s.bc32[5], cw = s.bc32[6];
-        const uint64_t my = s.bc64[4], mz = s.bc64[5], mw = s.bc64[6];
-        ++rounds;
-        if (cy < top_k && my < P)      { right = py; }
-        else if (cz < top_k && mz < P) { left = py; right = pz; cnt_x = cy; mass_x = my; }
-        else if (cw < top_k && mw < P) { left = pz; right = pw; cnt_x = cz; mass_x = mz; }
-        else                           { left = pw; cnt_x = cw; mass_x = mw; }
-    }
 
-    // ---- 4. smallest kept e, then counts and mass above it ------------------
-    {
-        uint32_t tinv = 0;
-#pragma unroll
-        for (int j = 0; j < R; ++j)
-            if (j < nv) {
-#pragma unroll
-                for (int k = 0; k < 4; ++k) { const uint32_t b = eb[j * 4 + k]; if (b >= left) tinv = max(tinv, ~b); }
+        // resolve the remaining digits on the gathered tokens, in LDS
+        if (levels < 2) {
+            lds_hist_zero(s, kNB2);
+            __syncthreads();
+            for (uint32_t i = tid; i < ncand; i += kThreads) {
+                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
+                lds_hist_add(s, digit2(b), q_of_bits(b));
             }
-        tinv = block_max_u32(s, tinv, lane, wave);
-        if (tid == 0) a_max(&rc->thr_inv, tinv);
-    }
-    if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
-    if (tid == 0) s.bc32[3] = ~a_load(&rc->thr_inv);
-    __syncthreads();
-    const uint32_t thr = s.bc32[3];
-    {
-        uint32_t c[3] = {0, 0, 0};
-        uint64_t m[3] = {0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < R; ++j)
-            if (j < nv) {
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const uint32_t b = opaque(eb[j * 4 + k]);
-                    if (b > thr) { c[0]++; m[0] += q_of_bits(b); }
-                    if (b == thr) c[1]++;
-                }
+            __syncthreads();
+            f = hist_find<kNB2 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
+            b2 = f.bin;
+        }
+        if (levels < 3) {
+            lds_hist_zero(s, kNB3);
+            __syncthreads();
+            for (uint32_t i = tid; i < ncand; i += kThreads) {
+                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
+                if (digit2(b) == b2) lds_hist_add(s, digit3(b), q_of_bits(b));
             }
-        block_sum3(s, c, m, lane, wave);
-        if (tid == 0) { a_add(&rc->n_gt, c[0]); a_add(&rc->n_eq, c[1]); a_add(&rc->G, m[0]); }
+            __syncthreads();
+            f = hist_find<kNB3 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
+            b3 = f.bin;
+        }
     }
-    if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
+    // all three digits are known: the threshold is one value
+    const uint32_t thr = (b1 >= 1025u) ? 0u : kOneBits - ((b1 << 19) | (b2 << 9) | b3);
+    const uint32_t n_gt = f.cnt_above, n_eq = f.cnt_bin;
+    const uint64_t Gm = f.mass_above;
 
     // ---- 5. tie weight, total S, target r (every workgroup, identically) ----
     if (tid == 0) {
-        const uint32_t n_gt = a_load(&rc->n_gt), n_eq = a_load(&rc->n_eq);
-        const uint64_t Gm = a_load(&rc->G);
         const uint64_t q_thr = q_of_bits(thr);
         uint64_t w_tie = q_thr;
         const uint64_t a = (P > Gm) ? (P - Gm) / n_eq : 0;
@@ -370,8 +539,8 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
         s.bc64[1] = w_tie; s.bc64[2] = S; s.bc64[3] = r;
         if (p.diag && part == 0) {
             rs_row_diag *d = p.diag + row;
-            d->xmax = xmax; d->emin_bits = emin; d->D = D; d->P = P;
-            d->left_bits = left; d->thr_bits = thr; d->rounds = rounds;
+            d->xmax = xmax; d->emin_bits = 0; d->D = D; d->P = P;
+            d->left_bits = thr; d->thr_bits = thr; d->rounds = levels;
             d->n_gt = n_gt; d->n_eq = n_eq; d->G = Gm; d->w_tie = w_tie; d->S = S; d->r = r;
         }
     }
@@ -386,16 +555,39 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
     auto slot_weight = [&](int j) -> uint64_t {         // weight of float4 slot j of this thread
         return weight(eb[j * 4]) + weight(eb[j * 4 + 1]) + weight(eb[j * 4 + 2]) + weight(eb[j * 4 + 3]);
     };
-    uint64_t wloc = 0;
+    uint64_t before = 0, wblock = 0;
+    if (gather) {
+        // kept weight of workgroup g = A[g] + weights of its gathered tokens
+        const uint32_t shift = 2 + 8 + (uint32_t)__builtin_ctz((unsigned)R);   // token index -> workgroup
+        uint64_t cb = 0, cm = 0;
+        for (uint32_t i = tid; i < ncand; i += kThreads) {
+            const uint64_t cd = s.cand[i];
+            const uint32_t g = ((uint32_t)cd) >> shift;
+            const uint64_t w = weight((uint32_t)(cd >> 32));
+            if (g < part) cb += w;
+            if (g == part) cm += w;
+        }
+        if (G > 1) {
+            if ((uint32_t)tid < part) cb += a_load(&rc->A[tid]);
+            if ((uint32_t)tid == part) cm += a_load(&rc->A[tid]);
+        } else if (tid == 0) cm += s.bc64[7];
+        block_sum2_u64(s, cb, cm, lane, wave);
+        before = cb; wblock = cm;
+    } else {
+        uint64_t wloc = 0;
 #pragma unroll
-    for (int j = 0; j < R; ++j)
-        if (j < nv) wloc += slot_weight(j);
-    const uint64_t wblock = block_sum_u64(s, wloc, lane, wave);
-    if (tid == 0) a_store(&rc->W[part], wblock);
-    if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
-    uint64_t before = 0;
-    for (uint32_t i = tid; i < part; i += kThreads) before += a_load(&rc->W[i]);
-    before = block_sum_u64(s, before, lane, wave);
+        for (int j = 0; j < R; ++j)
+            if (j < nv) wloc += slot_weight(j);
+        wblock = block_sum_u64(s, wloc, lane, wave);
+        if (G > 1) {
+            if (tid == 0) a_store(&rc->A[part], wblock);
+            if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
+            zero_slice(zc, zm, znb, part, G);
+            uint64_t bf = 0;
+            if ((uint32_t)tid < part) bf = a_load(&rc->A[tid]);
+            before = block_sum_u64(s, bf, lane, wave);
+        }
+    }
     const bool owner = before < r && r <= before + wblock;   // block-uniform
 
     if (owner) {
@@ -435,15 +627,30 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
             const int32_t idx = (int32_t)((base4 + (uint32_t)jstar * kThreads) * 4 + (uint32_t)kk);
             p.out[row] = idx;
             if (p.diag) p.diag[row].index = idx;
-            if (PEN) a_store(&rc->index, idx);
+            if (PEN && G > 1) a_store(&rc->index_p1, (uint32_t)idx + 1u);
+            if (PEN) s.bc32[7] = (uint32_t)idx;
         }
     }
 
     // ---- 7. penalties: decay and one-hot add, from registers ---------------
     if (PEN) {
-        if (!cluster_barrier(s, rc, p.hdr, ++bar * G)) return;
-        if (tid == 0) s.bc32[7] = (uint32_t)a_load(&rc->index);
         __syncthreads();
+        if (G > 1) {
+            if (tid == 0) {
+                const uint64_t t0 = wall_clock64();
+                uint32_t spins = 0, v;
+                while ((v = a_load(&rc->index_p1)) == 0u) {
+                    if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
+                        a_store(&p.hdr->error, (int32_t)RS_ERR_DEVICE);
+                        s.abort = 1;
+                        break;
+                    }
+                }
+                s.bc32[7] = v - 1u;
+            }
+            __syncthreads();
+            if (s.abort) return;
+        }
         const uint32_t idx = s.bc32[7];
 #pragma unroll
         for (int j = 0; j < R; ++j) {
@@ -469,18 +676,17 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
             st[2] = lo;
             if (lo == 0) st[3] += 1;
         }
-        s.bc32[0] = __hip_atomic_fetch_add(&rc->done, 1u, __ATOMIC_ACQ_REL, RS_AGENT);
-    }
-    __syncthreads();
-    if (s.bc32[0] == G - 1) {
-        // last workgroup out of this row: nobody reads the record any more
-        uint32_t *w = reinterpret_cast<uint32_t *>(rc);
-        for (uint32_t i = tid; i < sizeof(RowCtl) / 4; i += kThreads) a_store(&w[i], 0u);
-    }
-    __syncthreads();
-    if (tid == 0) {
-        const uint32_t f = __hip_atomic_fetch_add(&p.hdr->finished, 1u, __ATOMIC_ACQ_REL, RS_AGENT);
-        if (f == gridDim.x - 1) { a_store(&p.hdr->finished, 0u); a_store(&p.hdr->ticket, 0u); }
+        if (G > 1) {
+            const uint32_t d = __hip_atomic_fetch_add(&rc->done, 1u, __ATOMIC_RELAXED, RS_AGENT);
+            if (d == G - 1) {
+                // last workgroup out of this row: nobody reads the record any more
+                a_store(&rc->arrive, 0u); a_store(&rc->done, 0u); a_store(&rc->maxkey, 0u);
+                a_store(&rc->cursor, 0u); a_store(&rc->index_p1, 0u);
+            }
+        }
+        wait_vmem();
+        const uint32_t fin = __hip_atomic_fetch_add(&p.hdr->finished, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        if (fin == gridDim.x - 1) { a_store(&p.hdr->finished, 0u); a_store(&p.hdr->ticket, 0u); }
     }
 }
 
@@ -519,8 +725,8 @@ __global__ void philox_init_kernel(uint32_t *state, uint64_t seed, int32_t B)
 struct Geometry { int R; uint32_t G; };
 
 // Tokens per thread (4R) and workgroups per row.  Large batches take long
-// slices (few barriers' worth of peers, deep loads); a lone row is cut into
-// ~64 slices so that many CUs pull it from HBM at once.
+// slices (few peers to meet, deep loads); a lone row is cut into a few dozen
+// slices so that many CUs pull it from HBM at once.
 static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
 {
     const uint32_t V4 = (uint32_t)V / 4;
@@ -563,7 +769,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 100; }
+int rs_version(void) { return 200; }
 
 const char *rs_error_string(int code)
 {
