@@ -14,11 +14,11 @@
 //   3  threshold = largest t with count{e>=t} >= top_k or mass{e>=t} >= top_p*D.
 //      The reference finds it by a 4-way search on bit patterns with one pass
 //      over the row per step (:261-329); here it is a radix selection on the
-//      same bit patterns: a (count, mass) histogram over the top 11 bits of
-//      the key summed across the cluster, then either the few tokens of the
-//      boundary bin are gathered and resolved in LDS, or the next 10 / 9 bits
-//      are histogrammed the same way.  Same threshold, 3 barriers instead of
-//      one per search step.
+//      same bit patterns: a (count, mass) histogram over the top 10 bits
+//      summed across the cluster, then either the few tokens of the boundary
+//      bin are gathered and resolved in LDS, or the next 7 bits are
+//      histogrammed the same way (up to 4 levels).  Same threshold, usually 3
+//      barriers instead of one per search step.
 //   4  counts and mass above / at the threshold                   :332-355
 //   5  tie weight                                                 :365-371
 //   6  inverse-CDF pick in index order                            :374-426
@@ -35,11 +35,9 @@ namespace rs {
 constexpr int      kThreads   = 256;          // 4 waves, one per SIMD
 constexpr int      kWaves     = kThreads / kWave;
 constexpr int      kMaxParts  = 256;          // workgroups per row, at most
-constexpr int      kNB1       = 1280;         // level-1 bins (1026 used), 5 per thread
-constexpr int      kNB2       = 1024;         // level-2 bins, 4 per thread
-constexpr int      kNB3       = 512;          // level-3 bins, 2 per thread
+constexpr int      kNB        = 512;          // bins per histogram: level 1 uses 258, deeper levels 128
+constexpr int      kLevels    = 4;            // 10 + 7 + 7 + 7 bits
 constexpr int      kCap       = 1024;         // tokens of a boundary bin that are gathered
-constexpr uint32_t kOneBits   = 0x3F800000u;  // bits(1.0f) = bits(e_max)
 constexpr uint64_t kSpinLimit = 200000000ull; // 2 s of the 100 MHz wall clock
 
 struct alignas(256) WsHeader {
@@ -60,9 +58,7 @@ struct alignas(256) RowCtl {
     uint32_t pad[3];
     uint64_t A[kMaxParts];      // per workgroup: mass above the gathered bin, or kept weight
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
-    uint32_t c1[kNB1]; uint64_t m1[kNB1];
-    uint32_t c2[kNB2]; uint64_t m2[kNB2];
-    uint32_t c3[kNB3]; uint64_t m3[kNB3];
+    uint64_t h[kLevels][kNB];   // cluster histograms, packed (see pack_value)
 };
 
 struct Params {
@@ -95,19 +91,46 @@ template <typename T> __device__ __forceinline__ void a_max(T *p, T v) { __hip_a
 __device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Hides a register from the optimiser for one use, so that work derived from
-// the resident tokens (their fixed-point weights) is redone in each pass
-// instead of being hoisted and kept in two more registers per token.
+// the resident tokens is redone in each pass instead of being hoisted and kept
+// in more registers per token.
 __device__ __forceinline__ uint32_t opaque(uint32_t v)
 {
     asm volatile("" : "+v"(v));
     return v;
 }
 
-// Radix digits of a token, most significant first, on key' = bits(1.0) - bits(e)
-// (0 for the largest e, growing as e falls; e == 0 lands in bin 1025).
-__device__ __forceinline__ uint32_t digit1(uint32_t b) { return min((kOneBits - b) >> 19, 1025u); }
-__device__ __forceinline__ uint32_t digit2(uint32_t b) { return ((kOneBits - b) >> 9) & 1023u; }
-__device__ __forceinline__ uint32_t digit3(uint32_t b) { return (kOneBits - b) & 511u; }
+// ---- radix digits and histogram packing ----------------------------------
+// Digits are taken from the bit pattern of e in DESCENDING order (digit 0 =
+// largest e).  Level 1 = bits [30:21] counted down from bits(1.0) >> 21 = 508:
+// 4 bins per octave, aligned with the octaves, so every token of a bin has the
+// same exponent; e == 2^-64 is bin 256 and e == 0 bin 257.  Levels 2..4 take 7
+// more bits each (shifts 14, 7, 0).
+__device__ __forceinline__ uint32_t digit1(uint32_t b) { return min(508u - (b >> 21), 257u); }
+__device__ __forceinline__ uint32_t digit_at(uint32_t b, uint32_t sh) { return 127u - ((b >> sh) & 127u); }
+__device__ __forceinline__ uint32_t level_shift(uint32_t level) { return 21u - 7u * (level - 1u); }   // level >= 2
+__device__ __forceinline__ int      bin1_exponent(uint32_t d1) { return d1 <= 256u ? (int)((508u - d1) >> 2) : 0; }
+
+// A bin is one 64-bit word: count << 43 | sum of per-token values.  The value
+// of a token is its 23 fraction bits when its exponent is >= 110 (q = (2^23 +
+// fraction) << (exponent - 110), exact), else q itself (the significand
+// shifted right, at least 1).  Counts stay below 2^21 and sums below 2^43 for
+// any row of at most 2^20 tokens, so one atomic add carries both.
+constexpr uint64_t kPackOne  = 1ull << 43;
+constexpr uint64_t kPackMask = kPackOne - 1;
+__device__ __forceinline__ uint32_t pack_value(uint32_t b)
+{
+    const int ex = (int)(b >> 23);
+    const uint32_t frac = b & 0x7FFFFFu;
+    const uint32_t low = max((frac | 0x800000u) >> min(max(110 - ex, 0), 31), 1u);
+    return ex >= 110 ? frac : low;
+}
+__device__ __forceinline__ uint32_t pack_count(uint64_t w) { return (uint32_t)(w >> 43); }
+// mass (sum of q) of a bin whose tokens have biased exponent ex
+__device__ __forceinline__ uint64_t pack_mass(uint64_t w, int ex)
+{
+    const uint64_t sv = w & kPackMask;
+    return ex >= 110 ? ((sv + ((w >> 43) << 23)) << (ex - 110)) : sv;
+}
 
 struct Found {               // result of a histogram scan (uniform over the workgroup)
     uint32_t bin;            // first bin at which the kept set becomes sufficient
@@ -118,8 +141,8 @@ struct Found {               // result of a histogram scan (uniform over the wor
 };
 
 struct Lds {
-    uint32_t hc[kNB1];
-    uint64_t hm[kNB1];
+    uint64_t hm[kNB];        // this workgroup's histogram
+    uint64_t g[kNB];         // the cluster's histogram
     uint64_t cand[kCap];
     uint64_t u64[kWaves * 4];
     uint32_t u32[kWaves * 4];
@@ -194,53 +217,63 @@ __device__ __forceinline__ bool cluster_barrier(Lds &s, RowCtl *rc, WsHeader *hd
     return s.abort == 0;
 }
 
-__device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)
+__device__ __forceinline__ void lds_hist_zero(Lds &s)
 {
-    for (int b = threadIdx.x; b < nb; b += kThreads) { s.hc[b] = 0; s.hm[b] = 0; }
+    for (int b = threadIdx.x; b < kNB; b += kThreads) s.hm[b] = 0;
 }
-__device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint64_t q)
+// one LDS atomic per token: count and value together
+__device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint32_t value)
 {
-    atomicAdd(&s.hc[bin], 1u);
-    atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[bin]), (unsigned long long)q);
+    atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[bin]), (unsigned long long)(kPackOne | value));
 }
 
 // Re-zero this workgroup's share of a global histogram (the cluster splits the bins).
-__device__ __forceinline__ void zero_slice(uint32_t *gc, uint64_t *gm, uint32_t nb, uint32_t part, uint32_t G)
+__device__ __forceinline__ void zero_slice(uint64_t *gh, uint32_t part, uint32_t G)
 {
-    const uint32_t lo = (uint32_t)(((uint64_t)nb * part) / G), hi = (uint32_t)(((uint64_t)nb * (part + 1)) / G);
-    for (uint32_t b = lo + threadIdx.x; b < hi; b += kThreads) { a_store(&gc[b], 0u); a_store(&gm[b], (uint64_t)0); }
+    const uint32_t lo = (uint32_t)(((uint64_t)kNB * part) / G), hi = (uint32_t)(((uint64_t)kNB * (part + 1)) / G);
+    for (uint32_t b = lo + threadIdx.x; b < hi; b += kThreads) a_store(&gh[b], (uint64_t)0);
 }
 
-// Sum the workgroup histograms of a cluster: add mine into the row's global
-// bins, meet, read the totals back into LDS.  A cluster of one keeps its own.
-__device__ __forceinline__ bool hist_combine(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t G, uint32_t target,
-                                             uint32_t *gc, uint64_t *gm, int nb)
+// Sum the workgroup histograms of a cluster: add mine (s.hm, kept) into the
+// row's global bins, meet, read the totals into s.g.  A cluster of one copies
+// its own.
+__device__ __forceinline__ bool hist_combine(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t G, uint32_t target, uint64_t *gh)
 {
     __syncthreads();
-    if (G == 1) return true;
-    for (int b = threadIdx.x; b < nb; b += kThreads) {
-        const uint32_t c = s.hc[b];
-        if (c) { a_add(&gc[b], c); a_add(&gm[b], s.hm[b]); }
+    if (G == 1) {
+        for (int b = threadIdx.x; b < kNB; b += kThreads) s.g[b] = s.hm[b];
+        __syncthreads();
+        return true;
+    }
+    for (int b = threadIdx.x; b < kNB; b += kThreads) {
+        const uint64_t v = s.hm[b];
+        if (v) a_add(&gh[b], v);
     }
     if (!cluster_barrier(s, rc, hdr, G, target)) return false;
-    for (int b = threadIdx.x; b < nb; b += kThreads) { s.hc[b] = a_load(&gc[b]); s.hm[b] = a_load(&gm[b]); }
+    for (int b = threadIdx.x; b < kNB; b += kThreads) s.g[b] = a_load(&gh[b]);
     __syncthreads();
     return true;
 }
 
-// Scan the LDS histogram in bin order and find the first bin at which
-// (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).  With
-// first != 0 the total mass of the histogram is the row total D and P is
-// derived from it here.  Thread t owns bins [t*PER, (t+1)*PER).
-template <int PER>
+// Scan s.g in bin order and find the first bin at which
+// (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).  With first
+// the total mass of the histogram is the row total D and P is derived from it
+// here.  Thread t owns bins 2t and 2t+1; ex(bin) is the exponent of a bin.
+template <typename ExFn>
 __device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0, uint64_t top_k, float top_p,
-                                           bool first, int lane, int wave)
+                                           bool first, int lane, int wave, ExFn ex)
 {
+    constexpr int PER = kNB / kThreads;
     const int t = threadIdx.x;
     uint32_t c[PER]; uint64_t m[PER];
     uint32_t cs = 0; uint64_t ms = 0;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) { c[i] = s.hc[t * PER + i]; m[i] = s.hm[t * PER + i]; cs += c[i]; ms += m[i]; }
+    for (int i = 0; i < PER; ++i) {
+        const uint64_t w = s.g[t * PER + i];
+        c[i] = pack_count(w);
+        m[i] = pack_mass(w, ex((uint32_t)(t * PER + i)));
+        cs += c[i]; ms += m[i];
+    }
     // inclusive scan over threads
     uint64_t mi = wave_inclusive_scan_u64(ms, lane);
     uint64_t ci = wave_inclusive_scan_u64((uint64_t)cs, lane);
@@ -276,8 +309,26 @@ __device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0
     return s.found;
 }
 
+// Mass of this workgroup's own tokens in the bins before `bin` (from s.hm),
+// summed over the workgroup.
+template <typename ExFn>
+__device__ __forceinline__ uint64_t local_mass_before(Lds &s, uint32_t bin, int lane, int wave, ExFn ex)
+{
+    uint64_t a = 0;
+    for (uint32_t b = threadIdx.x; b < bin; b += kThreads) a += pack_mass(s.hm[b], ex(b));
+    return block_sum_u64(s, a, lane, wave);
+}
+
+// Waves per SIMD the register allocation must leave room for: the resident
+// tokens take 4R registers (8R with penalties), the rest is working set.
+template <int R, bool PEN> constexpr int min_waves()
+{
+    constexpr int data = (PEN ? 8 : 4) * R;
+    return data <= 32 ? 4 : data <= 64 ? 3 : 2;
+}
+
 template <int R, bool PEN>
-__global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
+__global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
 {
     __shared__ Lds s;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
@@ -301,34 +352,56 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
     const float4 *lg = reinterpret_cast<const float4 *>(p.logits + (int64_t)row * p.row_stride);
     float4 *pn4 = PEN ? reinterpret_cast<float4 *>(p.penalties + (int64_t)row * p.V) : nullptr;
 
-    uint32_t eb[R * 4];                                 // x, then bits(e)
+    uint32_t eb[R * 4];                                 // l, then x, then bits(e)
     float4 pen[PEN ? R : 1];
 
     // ---- 1. load once, scale, local max ---------------------------------
     {
-        float4 l[R];
 #pragma unroll
         for (int j = 0; j < R; ++j) {
             const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
-            l[j] = lg[i4];
+            const float4 l = lg[i4];
+            eb[j * 4 + 0] = __float_as_uint(l.x); eb[j * 4 + 1] = __float_as_uint(l.y);
+            eb[j * 4 + 2] = __float_as_uint(l.z); eb[j * 4 + 3] = __float_as_uint(l.w);
             if (PEN) pen[j] = pn4[i4];
         }
+        // Fast path: x = (l - pen) * c with no clean-up.  A NaN or Inf anywhere
+        // in l, pen or the product shows as a NaN or Inf x, and only then do the
+        // sf() calls of the definition change anything.
+        constexpr int kSpecial = 0x207;                 // sNaN | qNaN | -Inf | +Inf
+        bool special = false;
         float lmax = -3.402823466e+38f;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            float x0, x1, x2, x3;
-            if (PEN) {
-                x0 = sf((sf(l[j].x) - pen[j].x) * p.c);
-                x1 = sf((sf(l[j].y) - pen[j].y) * p.c);
-                x2 = sf((sf(l[j].z) - pen[j].z) * p.c);
-                x3 = sf((sf(l[j].w) - pen[j].w) * p.c);
-            } else {
-                x0 = sf(l[j].x * p.c); x1 = sf(l[j].y * p.c);
-                x2 = sf(l[j].z * p.c); x3 = sf(l[j].w * p.c);
+            float x[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float l = __uint_as_float(eb[j * 4 + k]);
+                const float pk = PEN ? (k == 0 ? pen[j].x : k == 1 ? pen[j].y : k == 2 ? pen[j].z : pen[j].w) : 0.0f;
+                x[k] = PEN ? (l - pk) * p.c : l * p.c;
+                special |= __builtin_amdgcn_classf(x[k], kSpecial);
+                eb[j * 4 + k] = __float_as_uint(x[k]);
             }
-            if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
-            eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
-            eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
+            if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
+        }
+        if (special) {
+            // rare: fetch the logits again and apply the definition with its clean-ups
+            lmax = -3.402823466e+38f;
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
+                const float4 l = lg[i4];
+                float x0, x1, x2, x3;
+                if (PEN) {
+                    x0 = sf((sf(l.x) - pen[j].x) * p.c); x1 = sf((sf(l.y) - pen[j].y) * p.c);
+                    x2 = sf((sf(l.z) - pen[j].z) * p.c); x3 = sf((sf(l.w) - pen[j].w) * p.c);
+                } else {
+                    x0 = sf(l.x * p.c); x1 = sf(l.y * p.c); x2 = sf(l.z * p.c); x3 = sf(l.w * p.c);
+                }
+                if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
+                eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
+                eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
+            }
         }
         const uint32_t k = block_max_u32(s, fkey(lmax), lane, wave);
         if (G > 1) {
@@ -336,7 +409,7 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
             if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
             if (tid == 0) s.bc32[1] = a_load(&rc->maxkey);
         } else if (tid == 0) s.bc32[1] = k;
-        lds_hist_zero(s, kNB1);
+        lds_hist_zero(s);
         __syncthreads();
     }
     const float xmax = fkey_inv(s.bc32[1]);
@@ -348,7 +421,7 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
         for (int k = 0; k < 4; ++k) {
             const uint32_t b = __float_as_uint(exp2c(__uint_as_float(eb[j * 4 + k]) - xmax));
             eb[j * 4 + k] = b;
-            if (j < nv) lds_hist_add(s, digit1(b), q_of_bits(b));
+            if (j < nv) lds_hist_add(s, digit1(b), pack_value(b));
         }
     }
     if (p.e_bits) {
@@ -357,17 +430,27 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
         for (int j = 0; j < R; ++j)
             if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
     }
-    if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->c1, rc->m1, kNB1)) return;
+    if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->h[0])) return;
     const uint64_t top_k = (uint64_t)p.top_k;
 
     // ---- 3. radix selection of the threshold -------------------------------
-    Found f = hist_find<kNB1 / kThreads>(s, 0u, 0ull, top_k, p.top_p, true, lane, wave);
+    auto ex1 = [](uint32_t bin) -> int { return bin1_exponent(bin); };
+    Found f = hist_find(s, 0u, 0ull, top_k, p.top_p, true, lane, wave, ex1);
     const uint64_t D = s.D, P = s.P;
-    const uint32_t b1 = f.bin;
-    uint32_t b2 = 0, b3 = 0;
-    uint32_t levels = 1;                     // histogram levels summed over the cluster
-    if (f.cnt_bin > (uint32_t)kCap) {
-        lds_hist_zero(s, kNB2);
+    const int exb = bin1_exponent(f.bin);                // exponent of every token still in play
+    auto exc = [exb](uint32_t) -> int { return exb; };
+    // my own tokens: mass in the bins before the boundary, count in the boundary bin
+    uint64_t amass = local_mass_before(s, f.bin, lane, wave, ex1);
+    uint32_t mycnt = pack_count(s.hm[f.bin]);
+    // bit patterns of the tokens still undistinguished: [lo, lo + span]
+    uint32_t lo = f.bin <= 256u ? (508u - f.bin) << 21 : 0u;
+    uint32_t span = f.bin <= 256u ? (1u << 21) - 1u : 0u;
+    uint32_t levels = 1;                                 // histogram levels summed over the cluster
+    while (f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
+        ++levels;
+        const uint32_t dsh = level_shift(levels);
+        __syncthreads();
+        lds_hist_zero(s);
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; ++j)
@@ -375,146 +458,75 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t b = opaque(eb[j * 4 + k]);
-                    if (digit1(b) == b1) lds_hist_add(s, digit2(b), q_of_bits(b));
+                    if (b - lo <= span) lds_hist_add(s, digit_at(b, dsh), pack_value(b));
                 }
             }
-        if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->c2, rc->m2, kNB2)) return;
-        if (G > 1) zero_slice(rc->c1, rc->m1, kNB1, part, G);   // everyone has read level 1 by now
-        f = hist_find<kNB2 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
-        b2 = f.bin;
-        levels = 2;
-        if (f.cnt_bin > (uint32_t)kCap) {
-            lds_hist_zero(s, kNB3);
-            __syncthreads();
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-                if (j < nv) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint32_t b = opaque(eb[j * 4 + k]);
-                        if (digit1(b) == b1 && digit2(b) == b2) lds_hist_add(s, digit3(b), q_of_bits(b));
-                    }
-                }
-            if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->c3, rc->m3, kNB3)) return;
-            if (G > 1) zero_slice(rc->c2, rc->m2, kNB2, part, G);
-            f = hist_find<kNB3 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
-            b3 = f.bin;
-            levels = 3;
-        }
+        if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->h[levels - 1])) return;
+        if (G > 1) zero_slice(rc->h[levels - 2], part, G);      // everyone has read the level above by now
+        f = hist_find(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
+        amass += local_mass_before(s, f.bin, lane, wave, exc);
+        mycnt = pack_count(s.hm[f.bin]);
+        lo |= (127u - f.bin) << dsh;
+        span = (1u << dsh) - 1u;
     }
-    // global histogram of the last summed level: re-zeroed after the next barrier
-    uint32_t *const zc = levels == 1 ? rc->c1 : levels == 2 ? rc->c2 : rc->c3;
-    uint64_t *const zm = levels == 1 ? rc->m1 : levels == 2 ? rc->m2 : rc->m3;
-    const uint32_t znb = levels == 1 ? kNB1 : levels == 2 ? kNB2 : kNB3;
 
-    // Tokens still undistinguished share digits 1..levels.  If they are few,
-    // gather them (bits and index) so that every workgroup can finish alone.
-    auto in_bin = [&](uint32_t b) -> bool {
-        if (digit1(b) != b1) return false;
-        if (levels >= 2 && digit2(b) != b2) return false;
-        if (levels >= 3 && digit3(b) != b3) return false;
-        return true;
-    };
-    auto above_bin = [&](uint32_t b) -> bool {         // larger e than every token of the bin
-        const uint32_t d1 = digit1(b);
-        if (d1 != b1) return d1 < b1;
-        if (levels < 2) return false;
-        const uint32_t d2 = digit2(b);
-        if (d2 != b2) return d2 < b2;
-        if (levels < 3) return false;
-        return digit3(b) < b3;
-    };
+    // If the undistinguished tokens are few, gather them (bits and index) so
+    // that every workgroup can finish alone.
     const bool gather = f.cnt_bin <= (uint32_t)kCap;
     uint32_t ncand = 0;
     if (gather) {
-        uint64_t amass = 0;
-        uint32_t mycnt = 0;
+        ncand = f.cnt_bin;
+        __syncthreads();
+        if (tid == 0) {
+            s.ctr = 0;
+            if (G > 1) {
+                s.bc32[2] = mycnt ? __hip_atomic_fetch_add(&rc->cursor, mycnt, __ATOMIC_RELAXED, RS_AGENT) : 0u;
+                a_store(&rc->A[part], amass);
+            } else s.bc64[7] = amass;
+        }
+        __syncthreads();
+        const uint32_t gbase = G > 1 ? s.bc32[2] : 0u;
 #pragma unroll
         for (int j = 0; j < R; ++j)
             if (j < nv) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t b = opaque(eb[j * 4 + k]);
-                    if (above_bin(b)) amass += q_of_bits(b);
-                    if (in_bin(b)) mycnt++;
-                }
-            }
-        amass = block_sum_u64(s, amass, lane, wave);
-        if (tid == 0) s.ctr = 0;
-        __syncthreads();
-        uint32_t myslot = 0;
-        if (mycnt) myslot = atomicAdd(&s.ctr, mycnt);
-        __syncthreads();
-        ncand = f.cnt_bin;
-        if (G > 1) {
-            if (tid == 0) {
-                const uint32_t n = s.ctr;
-                s.bc32[2] = n ? __hip_atomic_fetch_add(&rc->cursor, n, __ATOMIC_RELAXED, RS_AGENT) : 0u;
-                a_store(&rc->A[part], amass);
-            }
-            __syncthreads();
-            uint32_t o = s.bc32[2] + myslot;
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-                if (j < nv) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint32_t b = opaque(eb[j * 4 + k]);
-                        if (in_bin(b)) {
-                            const uint32_t idx = (base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)k;
-                            if (o < (uint32_t)kCap) a_store(&rc->cand[o], ((uint64_t)b << 32) | idx);
-                            ++o;
-                        }
+                    if (b - lo <= span) {
+                        const uint32_t o = gbase + atomicAdd(&s.ctr, 1u);
+                        const uint32_t idx = (base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)k;
+                        const uint64_t cd = ((uint64_t)b << 32) | idx;
+                        if (o < (uint32_t)kCap) { if (G > 1) a_store(&rc->cand[o], cd); else s.cand[o] = cd; }
                     }
                 }
+            }
+        if (G > 1) {
             if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
             for (uint32_t i = tid; i < ncand; i += kThreads) s.cand[i] = a_load(&rc->cand[i]);
-            zero_slice(zc, zm, znb, part, G);
-        } else {
-            uint32_t o = myslot;
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-                if (j < nv) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint32_t b = opaque(eb[j * 4 + k]);
-                        if (in_bin(b)) {
-                            const uint32_t idx = (base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)k;
-                            if (o < (uint32_t)kCap) s.cand[o] = ((uint64_t)b << 32) | idx;
-                            ++o;
-                        }
-                    }
-                }
-            if (tid == 0) s.bc64[7] = amass;
+            zero_slice(rc->h[levels - 1], part, G);
         }
         __syncthreads();
 
         // resolve the remaining digits on the gathered tokens, in LDS
-        if (levels < 2) {
-            lds_hist_zero(s, kNB2);
+        for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels; ++lv) {
+            const uint32_t dsh = level_shift(lv);
+            __syncthreads();
+            lds_hist_zero(s);
             __syncthreads();
             for (uint32_t i = tid; i < ncand; i += kThreads) {
                 const uint32_t b = (uint32_t)(s.cand[i] >> 32);
-                lds_hist_add(s, digit2(b), q_of_bits(b));
+                if (b - lo <= span) lds_hist_add(s, digit_at(b, dsh), pack_value(b));
             }
             __syncthreads();
-            f = hist_find<kNB2 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
-            b2 = f.bin;
-        }
-        if (levels < 3) {
-            lds_hist_zero(s, kNB3);
+            for (int b = tid; b < kNB; b += kThreads) s.g[b] = s.hm[b];
             __syncthreads();
-            for (uint32_t i = tid; i < ncand; i += kThreads) {
-                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
-                if (digit2(b) == b2) lds_hist_add(s, digit3(b), q_of_bits(b));
-            }
-            __syncthreads();
-            f = hist_find<kNB3 / kThreads>(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave);
-            b3 = f.bin;
+            f = hist_find(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
+            lo |= (127u - f.bin) << dsh;
+            span = (1u << dsh) - 1u;
         }
     }
-    // all three digits are known: the threshold is one value
-    const uint32_t thr = (b1 >= 1025u) ? 0u : kOneBits - ((b1 << 19) | (b2 << 9) | b3);
+    // every digit is known: the threshold is the one value left in [lo, lo + span]
+    const uint32_t thr = lo;
     const uint32_t n_gt = f.cnt_above, n_eq = f.cnt_bin;
     const uint64_t Gm = f.mass_above;
 
@@ -582,7 +594,7 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
         if (G > 1) {
             if (tid == 0) a_store(&rc->A[part], wblock);
             if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
-            zero_slice(zc, zm, znb, part, G);
+            zero_slice(rc->h[levels - 1], part, G);
             uint64_t bf = 0;
             if ((uint32_t)tid < part) bf = a_load(&rc->A[tid]);
             before = block_sum_u64(s, bf, lane, wave);
@@ -620,9 +632,9 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
         uint64_t woff = 0;
         for (int w = 0; w < wave; ++w) woff += s.u64[w];
         inc += woff;
-        const uint64_t exc = inc - mine;
-        if (exc < rl && rl <= inc) {                      // exactly one thread
-            const uint64_t rr = rl - exc;                 // 1 <= rr <= mine
+        const uint64_t exc_ = inc - mine;
+        if (exc_ < rl && rl <= inc) {                     // exactly one thread
+            const uint64_t rr = rl - exc_;                // 1 <= rr <= mine
             const int kk = (rr <= w0) ? 0 : (rr <= w0 + w1) ? 1 : (rr <= w0 + w1 + w2) ? 2 : 3;
             const int32_t idx = (int32_t)((base4 + (uint32_t)jstar * kThreads) * 4 + (uint32_t)kk);
             p.out[row] = idx;
@@ -672,9 +684,9 @@ __global__ void __launch_bounds__(kThreads) sample_kernel(const Params p)
     if (tid == 0) {
         if (part == 0 && !p.inj_u) {
             uint32_t *st = p.rng + (size_t)row * 16;
-            const uint32_t lo = st[2] + 1;
-            st[2] = lo;
-            if (lo == 0) st[3] += 1;
+            const uint32_t lo32 = st[2] + 1;
+            st[2] = lo32;
+            if (lo32 == 0) st[3] += 1;
         }
         if (G > 1) {
             const uint32_t d = __hip_atomic_fetch_add(&rc->done, 1u, __ATOMIC_RELAXED, RS_AGENT);
