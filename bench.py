@@ -134,6 +134,9 @@ def main():
     ap.add_argument("--skip-bandwidth", action="store_true", help="skip the 2 GiB bandwidth configuration")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--bandwidth-steps", type=int, default=20)
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run one plain device copy of 512 MiB (read 512 MiB + write 512 MiB), the known-size "
+                         "kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (rows shard over GPUs without communication; "
@@ -232,6 +235,12 @@ def main():
                                    "achieved": round(bytes_flat / (t_flat * 1e-6) / 1e9, 1),
                                    "rows_per_s": round(Bb * Tb / (t_flat * 1e-6), 1)},
         }
+        if args.traffic_probe:
+            src = big.view(-1)[: Bb * Vb]
+            dst = torch.empty_like(src)
+            dst.copy_(src)
+            torch.cuda.synchronize()
+            del dst
         del big, flat
 
     # ---- CPU baselines ------------------------------------------------------
