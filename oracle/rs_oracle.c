@@ -13,7 +13,8 @@
  *   penalty decay with one-hot add           :427-437
  * What is restated so that the result is independent of summation order:
  *   - exp2 is a fixed degree-5 Horner polynomial on the fractional part
- *     (hardware/libm exp2f are not bit-identical across machines);
+ *     (hardware/libm exp2f are not bit-identical across machines), with
+ *     the argument clamped at -64 so that every e is a normal float;
  *   - the probability of token i is carried as the integer
  *         q_i = max(1, floor(e_i * 2^40)),    e_max = 1 exactly,
  *     the row total D = sum q_i replaces the float denominator, and "mass
@@ -55,11 +56,13 @@ float rs_oracle_scale(float logit, float penalty, int has_penalty, float c)
 }
 
 /*
- * exp2 for d <= 0 (d = x - max, sampling.cu:235).  n = floor(d), f = d - n is
- * exact and lies in [0,1]; 2^f is a degree-5 minimax polynomial (relative
- * error 8.3e-8) evaluated by Horner with fmaf; the result is scaled by 2^n
- * exactly.  All coefficients are positive, so the polynomial is monotone in
- * f, and poly(1) <= 2 = 2*poly(0), so exp2c is monotone in d.
+ * exp2 for d <= 0 (d = x - max, sampling.cu:235), d clamped to >= -64 first
+ * (tokens further down all get e = 2^-64, whose weight q is the minimum 1).
+ * n = floor(d), f = d - n is exact and lies in [0,1]; 2^f is a degree-5
+ * minimax polynomial (relative error 8.3e-8) evaluated by Horner with fmaf;
+ * the result is scaled by 2^n exactly.  All coefficients are positive, so the
+ * polynomial is monotone in f, and poly(1) <= 2 = 2*poly(0), so exp2c is
+ * monotone in d.
  */
 static const float RS_C1 = 0x1.62e4bap-1f;
 static const float RS_C2 = 0x1.ebdb56p-3f;
@@ -69,8 +72,8 @@ static const float RS_C5 = 0x1.e974fap-10f;
 
 float rs_oracle_exp2c(float d)
 {
+    d = fmaxf(d, (float)RS_EXP_CLAMP);
     float n = floorf(d);
-    if (!(n >= (float)RS_EXP_FLUSH)) return 0.0f;
     float f = d - n;
     float p = RS_C5;
     p = fmaf(p, f, RS_C4);

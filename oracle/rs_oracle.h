@@ -36,8 +36,8 @@ extern "C" {
 
 /* Fractional bits of the fixed-point weight q = max(1, floor(e * 2^RS_QBITS)). */
 #define RS_QBITS 40
-/* exp2c(d) is flushed to +0 when floor(d) < RS_EXP_FLUSH. */
-#define RS_EXP_FLUSH (-64)
+/* exp2c clamps its argument: exp2c(d) = exp2c(max(d, RS_EXP_CLAMP)) >= 2^-64. */
+#define RS_EXP_CLAMP (-64)
 
 /* Per-row diagnostics; mirrors rs_row_diag of include/rapid_sampling.h. */
 typedef struct {

@@ -1,5 +1,6 @@
 // Device-side building blocks of the MI355X token sampler: canonical
-// element-wise arithmetic, wave64/workgroup reductions and scans, Philox.
+// element-wise arithmetic, wave64 reductions and scans on the DPP data path,
+// Philox.
 //
 // Arithmetic contract (shared with the CPU oracle used by the tests): every
 // floating-point step is a single IEEE fp32 operation (compile with
@@ -24,11 +25,13 @@ __device__ __forceinline__ float sf(float x)
     return fminf(fmaxf(y, -3.402823466e+38f), 3.402823466e+38f);
 }
 
-// exp2 for d <= 0: floor/fraction split, degree-5 Horner with positive
-// coefficients on the fraction (monotone), exact scale by 2^floor(d), flush to
-// +0 below 2^-64.                          (reference: exp2f at sampling.cu:235)
-__device__ __forceinline__ float exp2c(float d)
+// exp2 for d <= 0, argument clamped at -64 (so the result is a normal float in
+// [2^-64, 1]): floor/fraction split, degree-5 Horner with positive
+// coefficients on the fraction (monotone), exact scale by 2^floor(d).
+// Returns the bit pattern.                 (reference: exp2f at sampling.cu:235)
+__device__ __forceinline__ uint32_t exp2c_bits(float d)
 {
+    d = fmaxf(d, -64.0f);
     const float n = __builtin_floorf(d);
     const float f = d - n;
     float p = 0x1.e974fap-10f;
@@ -37,15 +40,15 @@ __device__ __forceinline__ float exp2c(float d)
     p = __builtin_fmaf(p, f, 0x1.ebdb56p-3f);
     p = __builtin_fmaf(p, f, 0x1.62e4bap-1f);
     p = __builtin_fmaf(p, f, 1.0f);
-    const float e = __builtin_ldexpf(p, (int)n);
-    return (n >= -64.0f) ? e : 0.0f;
+    // p in [1,2], n in [-64,0]: p * 2^n by adding n to the exponent field
+    return __float_as_uint(p) + ((uint32_t)(int)n << 23);
 }
 
-// Fixed-point weight of a token from the bit pattern of e (0 or 2^-64..1):
+// Fixed-point weight of a token from the bit pattern of e (2^-64..1):
 // q = max(1, floor(e * 2^40)).
 __device__ __forceinline__ uint64_t q_of_bits(uint32_t b)
 {
-    const int      ex = (int)(b >> 23);                    // biased exponent, <= 127
+    const int      ex = (int)(b >> 23);                    // biased exponent, 63..127
     const uint32_t m  = (b & 0x7FFFFFu) | 0x800000u;       // 24-bit significand
     const int      sh = ex - 110;                          // e*2^40 = m * 2^sh
     uint64_t q;
@@ -120,32 +123,64 @@ __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint
 }
 
 // ------------------------------------------------------ wave64 primitives --
+// All cross-lane traffic uses DPP (data-parallel primitives on the VALU
+// operand path): row_shr:1,2,4,8 scan inside each row of 16 lanes, then
+// row_bcast:15 carries lane 15 of a row into the next row (rows 1 and 3),
+// row_bcast:31 carries lane 31 into rows 2 and 3.  Six steps, no LDS.  Lanes
+// with no source read 0 (the identity of + and of max on unsigned).
 
-template <typename T>
-__device__ __forceinline__ T wave_sum(T v)
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp0_u32(uint32_t v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+template <int CTRL, int ROW_MASK, typename T>
+__device__ __forceinline__ T dpp0(T v)
+{
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit integers");
+    if constexpr (sizeof(T) == 4) return (T)dpp0_u32<CTRL, ROW_MASK>((uint32_t)v);
+    else {
+        const uint32_t lo = dpp0_u32<CTRL, ROW_MASK>((uint32_t)v), hi = dpp0_u32<CTRL, ROW_MASK>((uint32_t)((uint64_t)v >> 32));
+        return (T)(((uint64_t)hi << 32) | lo);
+    }
+}
+
+// Inclusive scan (sum) over the 64 lanes; lane 63 ends with the wave total.
+// The reference's float ladder has to run 16,8,4,2,1 to stay monotone
+// (sampling.cu:48-58); these are integers, exact in any order.
+template <typename T>
+__device__ __forceinline__ T wave_inclusive_scan(T v)
+{
+    v += dpp0<0x111, 0xf>(v);     // row_shr:1
+    v += dpp0<0x112, 0xf>(v);     // row_shr:2
+    v += dpp0<0x114, 0xf>(v);     // row_shr:4
+    v += dpp0<0x118, 0xf>(v);     // row_shr:8
+    v += dpp0<0x142, 0xa>(v);     // row_bcast:15 -> rows 1,3
+    v += dpp0<0x143, 0xc>(v);     // row_bcast:31 -> rows 2,3
     return v;
 }
+
+__device__ __forceinline__ uint32_t lane63_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readlane((int)v, 63); }
+template <typename T>
+__device__ __forceinline__ T lane63(T v)
+{
+    if constexpr (sizeof(T) == 4) return (T)lane63_u32((uint32_t)v);
+    else return (T)(((uint64_t)lane63_u32((uint32_t)((uint64_t)v >> 32)) << 32) | lane63_u32((uint32_t)v));
+}
+
+// Sum over the wave, returned to every lane (wave-uniform).
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) { return lane63(wave_inclusive_scan(v)); }
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) { uint32_t o = __shfl_xor(v, off, kWave); v = o > v ? o : v; }
-    return v;
-}
-
-// Inclusive scan over the 64 lanes, ladder 32,16,8,4,2,1 (descending, the
-// order the reference requires of its 16..1 ladder, sampling.cu:48-58; on
-// integers any order is exact).
-__device__ __forceinline__ uint64_t wave_inclusive_scan_u64(uint64_t v, int lane)
-{
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const uint64_t n = __shfl_up(v, off, kWave);
-        if (lane >= off) v += n;
-    }
-    return v;
+    v = max(v, dpp0_u32<0x111, 0xf>(v));
+    v = max(v, dpp0_u32<0x112, 0xf>(v));
+    v = max(v, dpp0_u32<0x114, 0xf>(v));
+    v = max(v, dpp0_u32<0x118, 0xf>(v));
+    v = max(v, dpp0_u32<0x142, 0xa>(v));
+    v = max(v, dpp0_u32<0x143, 0xc>(v));
+    return lane63_u32(v);
 }
 
 }  // namespace rs

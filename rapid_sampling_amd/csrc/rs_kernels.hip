@@ -52,10 +52,11 @@ struct alignas(256) WsHeader {
 struct alignas(256) RowCtl {
     uint32_t arrive;      // barrier arrivals so far
     uint32_t done;        // workgroups finished with this row
-    uint32_t maxkey;      // max of fkey(x)
+    uint32_t unused0;
     uint32_t cursor;      // fill of cand[]
     uint32_t index_p1;    // sampled token + 1, once known
     uint32_t pad[3];
+    uint32_t mx[kMaxParts];     // per workgroup: fkey(max x of its slice), 0 = not yet written
     uint64_t A[kMaxParts];      // per workgroup: mass above the gathered bin, or kept weight
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
     uint64_t h[kLevels][kNB];   // cluster histograms, packed (see pack_value)
@@ -100,29 +101,29 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v)
 }
 
 // ---- radix digits and histogram packing ----------------------------------
-// Digits are taken from the bit pattern of e in DESCENDING order (digit 0 =
-// largest e).  Level 1 = bits [30:21] counted down from bits(1.0) >> 21 = 508:
-// 4 bins per octave, aligned with the octaves, so every token of a bin has the
-// same exponent; e == 2^-64 is bin 256 and e == 0 bin 257.  Levels 2..4 take 7
-// more bits each (shifts 14, 7, 0).
-__device__ __forceinline__ uint32_t digit1(uint32_t b) { return min(508u - (b >> 21), 257u); }
-__device__ __forceinline__ uint32_t digit_at(uint32_t b, uint32_t sh) { return 127u - ((b >> sh) & 127u); }
+// The threshold is selected digit by digit on the bit pattern of e, largest e
+// first.  Level 1 looks at bits [30:21]: index = bits >> 21 runs from 252
+// (e = 2^-64) to 508 (e = 1), 4 bins per octave aligned with the octaves, so
+// every token of a bin has the same exponent.  Levels 2..4 take 7 more bits
+// each (shifts 14, 7, 0).  Histograms are stored by index (ascending in e);
+// the scan walks them by digit = top - index (descending in e).
+constexpr uint32_t kTop1 = 508u;                      // index of e = 1.0 at level 1
+constexpr uint32_t kTopN = 127u;                      // largest index of a deeper level
 __device__ __forceinline__ uint32_t level_shift(uint32_t level) { return 21u - 7u * (level - 1u); }   // level >= 2
-__device__ __forceinline__ int      bin1_exponent(uint32_t d1) { return d1 <= 256u ? (int)((508u - d1) >> 2) : 0; }
 
 // A bin is one 64-bit word: count << 43 | sum of per-token values.  The value
-// of a token is its 23 fraction bits when its exponent is >= 110 (q = (2^23 +
-// fraction) << (exponent - 110), exact), else q itself (the significand
-// shifted right, at least 1).  Counts stay below 2^21 and sums below 2^43 for
-// any row of at most 2^20 tokens, so one atomic add carries both.
+// of a token is its 23 fraction bits when its exponent is >= 110 (then q =
+// (2^23 + fraction) << (exponent - 110), exact), else q itself (< 2^23).
+// Counts stay below 2^21 and sums below 2^43 for any row of at most 2^20
+// tokens, so one atomic add carries both.
 constexpr uint64_t kPackOne  = 1ull << 43;
 constexpr uint64_t kPackMask = kPackOne - 1;
 __device__ __forceinline__ uint32_t pack_value(uint32_t b)
 {
-    const int ex = (int)(b >> 23);
-    const uint32_t frac = b & 0x7FFFFFu;
-    const uint32_t low = max((frac | 0x800000u) >> min(max(110 - ex, 0), 31), 1u);
-    return ex >= 110 ? frac : low;
+    uint32_t v = b & 0x7FFFFFu;
+    if (b < 0x37000000u)                               // e < 2^-17: q = floor(e * 2^40) fits 23 bits
+        v = max((uint32_t)(__uint_as_float(b) * 0x1p40f), 1u);
+    return v;
 }
 __device__ __forceinline__ uint32_t pack_count(uint64_t w) { return (uint32_t)(w >> 43); }
 // mass (sum of q) of a bin whose tokens have biased exponent ex
@@ -133,7 +134,7 @@ __device__ __forceinline__ uint64_t pack_mass(uint64_t w, int ex)
 }
 
 struct Found {               // result of a histogram scan (uniform over the workgroup)
-    uint32_t bin;            // first bin at which the kept set becomes sufficient
+    uint32_t bin;            // index of the first bin (largest e first) at which the kept set becomes sufficient
     uint32_t cnt_above;      // tokens in bins before it (plus the carried offset)
     uint32_t cnt_bin;        // tokens in it
     uint64_t mass_above;
@@ -255,13 +256,14 @@ __device__ __forceinline__ bool hist_combine(Lds &s, RowCtl *rc, WsHeader *hdr, 
     return true;
 }
 
-// Scan s.g in bin order and find the first bin at which
-// (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).  With first
-// the total mass of the histogram is the row total D and P is derived from it
-// here.  Thread t owns bins 2t and 2t+1; ex(bin) is the exponent of a bin.
+// Scan s.g from index `top` downwards (largest e first) and find the first
+// bin at which (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).
+// With `first` the total mass of the histogram is the row total D and P is
+// derived from it here.  Thread t owns digits 2t and 2t+1 (index = top -
+// digit); ex(index) is the exponent of a bin.
 template <typename ExFn>
-__device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0, uint64_t top_k, float top_p,
-                                           bool first, int lane, int wave, ExFn ex)
+__device__ __forceinline__ Found hist_find(Lds &s, uint32_t top, uint32_t cnt0, uint64_t mass0, uint64_t top_k,
+                                           float top_p, bool first, int lane, int wave, ExFn ex)
 {
     constexpr int PER = kNB / kThreads;
     const int t = threadIdx.x;
@@ -269,22 +271,24 @@ __device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0
     uint32_t cs = 0; uint64_t ms = 0;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        const uint64_t w = s.g[t * PER + i];
+        const int idx = (int)top - (t * PER + i);
+        const uint64_t w = idx >= 0 ? s.g[idx] : 0ull;
         c[i] = pack_count(w);
-        m[i] = pack_mass(w, ex((uint32_t)(t * PER + i)));
+        m[i] = pack_mass(w, ex((uint32_t)idx));
         cs += c[i]; ms += m[i];
     }
     // inclusive scan over threads
-    uint64_t mi = wave_inclusive_scan_u64(ms, lane);
-    uint64_t ci = wave_inclusive_scan_u64((uint64_t)cs, lane);
+    const uint64_t mi = wave_inclusive_scan(ms);
+    const uint32_t ci = wave_inclusive_scan(cs);
     __syncthreads();
-    if (lane == kWave - 1) { s.u64[wave * 2] = mi; s.u64[wave * 2 + 1] = ci; }
+    if (lane == kWave - 1) { s.u64[wave] = mi; s.u32[wave] = ci; }
     __syncthreads();
-    uint64_t moff = 0, coff = 0, mtot = 0;
+    uint64_t moff = 0, mtot = 0;
+    uint32_t coff = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-        if (w < wave) { moff += s.u64[w * 2]; coff += s.u64[w * 2 + 1]; }
-        mtot += s.u64[w * 2];
+        if (w < wave) { moff += s.u64[w]; coff += s.u32[w]; }
+        mtot += s.u64[w];
     }
     if (first) {
         if (t == 0) { s.D = mtot; s.P = ceil_mul(top_p, mtot); }
@@ -299,7 +303,7 @@ __device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0
         const uint64_t nc = rcnt + c[i], nm = rm + m[i];
         const bool after = nc >= top_k || nm >= P;
         if (!before && after) {
-            s.found.bin = (uint32_t)(t * PER + i);
+            s.found.bin = top - (uint32_t)(t * PER + i);
             s.found.cnt_above = (uint32_t)rcnt; s.found.cnt_bin = c[i];
             s.found.mass_above = rm; s.found.mass_bin = m[i];
         }
@@ -309,13 +313,13 @@ __device__ __forceinline__ Found hist_find(Lds &s, uint32_t cnt0, uint64_t mass0
     return s.found;
 }
 
-// Mass of this workgroup's own tokens in the bins before `bin` (from s.hm),
-// summed over the workgroup.
+// Mass of this workgroup's own tokens in the bins above index `bin` (larger
+// e), from s.hm, summed over the workgroup.
 template <typename ExFn>
-__device__ __forceinline__ uint64_t local_mass_before(Lds &s, uint32_t bin, int lane, int wave, ExFn ex)
+__device__ __forceinline__ uint64_t local_mass_above(Lds &s, uint32_t bin, uint32_t top, int lane, int wave, ExFn ex)
 {
     uint64_t a = 0;
-    for (uint32_t b = threadIdx.x; b < bin; b += kThreads) a += pack_mass(s.hm[b], ex(b));
+    for (uint32_t b = bin + 1 + threadIdx.x; b <= top; b += kThreads) a += pack_mass(s.hm[b], ex(b));
     return block_sum_u64(s, a, lane, wave);
 }
 
@@ -341,6 +345,14 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     const uint32_t ticket = s.bc32[0];
     const uint32_t G = p.G;
     const uint32_t row = ticket / G, part = ticket - row * G;
+    if (tid == 64 && !p.inj_u) {
+        // this call's 64 random bits, drawn while the logits are in flight (the state is
+        // advanced once, at the end, by the row's first workgroup)
+        const uint32_t *st = p.rng + (size_t)row * 16;
+        uint32_t o[4];
+        philox4x32_10(st[2], st[3], st[4], st[5], st[0], st[1], o);
+        s.bc64[5] = ((uint64_t)o[0] << 32) | o[1];
+    }
     RowCtl *rc = p.ctl + row;
     uint32_t bar = 0;                                   // barriers passed
 
@@ -356,6 +368,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     float4 pen[PEN ? R : 1];
 
     // ---- 1. load once, scale, local max ---------------------------------
+    uint32_t kmax_row;
     {
 #pragma unroll
         for (int j = 0; j < R; ++j) {
@@ -404,24 +417,42 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             }
         }
         const uint32_t k = block_max_u32(s, fkey(lmax), lane, wave);
-        if (G > 1) {
-            if (tid == 0) a_max(&rc->maxkey, k);
-            if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
-            if (tid == 0) s.bc32[1] = a_load(&rc->maxkey);
-        } else if (tid == 0) s.bc32[1] = k;
         lds_hist_zero(s);
-        __syncthreads();
+        uint32_t kmax = k;
+        if (G > 1) {
+            // Exchange of the slice maxima without a counter: every workgroup writes its
+            // key (never 0 for a finite x) into its own slot and thread t waits for slot t.
+            if (tid == 0) a_store(&rc->mx[part], k);
+            uint32_t v = k;
+            if ((uint32_t)tid < G) {
+                const uint64_t t0 = wall_clock64();
+                uint32_t spins = 0;
+                while ((v = a_load(&rc->mx[tid])) == 0u) {
+                    if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
+                        a_store(&p.hdr->error, (int32_t)RS_ERR_DEVICE);
+                        s.abort = 1;
+                        break;
+                    }
+                }
+            }
+            kmax = block_max_u32(s, v, lane, wave);
+            if (s.abort) return;
+        } else __syncthreads();
+        kmax_row = kmax;
     }
-    const float xmax = fkey_inv(s.bc32[1]);
+    const float xmax = fkey_inv(kmax_row);
 
     // ---- 2. e = exp2(x - max) in place; level-1 histogram ------------------
 #pragma unroll
     for (int j = 0; j < R; ++j) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t b = __float_as_uint(exp2c(__uint_as_float(eb[j * 4 + k]) - xmax));
-            eb[j * 4 + k] = b;
-            if (j < nv) lds_hist_add(s, digit1(b), pack_value(b));
+        for (int k = 0; k < 4; ++k) eb[j * 4 + k] = exp2c_bits(__uint_as_float(eb[j * 4 + k]) - xmax);
+        if (j < nv) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t b = eb[j * 4 + k];
+                lds_hist_add(s, b >> 21, pack_value(b));
+            }
         }
     }
     if (p.e_bits) {
@@ -431,20 +462,21 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
     }
     if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->h[0])) return;
+    if (G > 1 && tid == 0) a_store(&rc->mx[part], 0u);   // every workgroup has read the maxima by now
     const uint64_t top_k = (uint64_t)p.top_k;
 
     // ---- 3. radix selection of the threshold -------------------------------
-    auto ex1 = [](uint32_t bin) -> int { return bin1_exponent(bin); };
-    Found f = hist_find(s, 0u, 0ull, top_k, p.top_p, true, lane, wave, ex1);
+    auto ex1 = [](uint32_t idx) -> int { return (int)(idx >> 2); };
+    Found f = hist_find(s, kTop1, 0u, 0ull, top_k, p.top_p, true, lane, wave, ex1);
     const uint64_t D = s.D, P = s.P;
-    const int exb = bin1_exponent(f.bin);                // exponent of every token still in play
+    const int exb = (int)(f.bin >> 2);                   // exponent of every token still in play
     auto exc = [exb](uint32_t) -> int { return exb; };
-    // my own tokens: mass in the bins before the boundary, count in the boundary bin
-    uint64_t amass = local_mass_before(s, f.bin, lane, wave, ex1);
+    // my own tokens: mass in the bins above the boundary, count in the boundary bin
+    uint64_t amass = local_mass_above(s, f.bin, kTop1, lane, wave, ex1);
     uint32_t mycnt = pack_count(s.hm[f.bin]);
     // bit patterns of the tokens still undistinguished: [lo, lo + span]
-    uint32_t lo = f.bin <= 256u ? (508u - f.bin) << 21 : 0u;
-    uint32_t span = f.bin <= 256u ? (1u << 21) - 1u : 0u;
+    uint32_t lo = f.bin << 21;
+    uint32_t span = (1u << 21) - 1u;
     uint32_t levels = 1;                                 // histogram levels summed over the cluster
     while (f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
         ++levels;
@@ -458,15 +490,15 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t b = opaque(eb[j * 4 + k]);
-                    if (b - lo <= span) lds_hist_add(s, digit_at(b, dsh), pack_value(b));
+                    if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, pack_value(b));
                 }
             }
         if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->h[levels - 1])) return;
         if (G > 1) zero_slice(rc->h[levels - 2], part, G);      // everyone has read the level above by now
-        f = hist_find(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
-        amass += local_mass_before(s, f.bin, lane, wave, exc);
+        f = hist_find(s, kTopN, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
+        amass += local_mass_above(s, f.bin, kTopN, lane, wave, exc);
         mycnt = pack_count(s.hm[f.bin]);
-        lo |= (127u - f.bin) << dsh;
+        lo |= f.bin << dsh;
         span = (1u << dsh) - 1u;
     }
 
@@ -507,6 +539,31 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         }
         __syncthreads();
 
+        if (ncand <= (uint32_t)kWave) {
+            // A handful of tokens: every thread ranks one of them against all the others.
+            // Token v is a valid threshold when the kept set {e >= v} is sufficient; the
+            // threshold is the largest such v.
+            const uint32_t mine = (uint32_t)tid < ncand ? (uint32_t)(s.cand[tid] >> 32) : 0u;
+            uint32_t cge = 0, cgt = 0;
+            uint64_t mge = 0;
+            for (uint32_t i = 0; i < ncand; ++i) {
+                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
+                if (b >= mine) { ++cge; mge += q_of_bits(b); }
+                if (b > mine) ++cgt;
+            }
+            const bool ok = (uint32_t)tid < ncand &&
+                            ((uint64_t)f.cnt_above + cge >= top_k || f.mass_above + mge >= P);
+            const uint32_t best = block_max_u32(s, ok ? mine : 0u, lane, wave);
+            if (ok && mine == best) {                    // ties write the same values
+                s.found.bin = 0;
+                s.found.cnt_above = f.cnt_above + cgt; s.found.cnt_bin = cge - cgt;
+                s.found.mass_above = f.mass_above + mge - (uint64_t)(cge - cgt) * q_of_bits(mine);
+                s.found.mass_bin = 0;
+            }
+            __syncthreads();
+            f = s.found;
+            lo = best; span = 0;
+        } else
         // resolve the remaining digits on the gathered tokens, in LDS
         for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels; ++lv) {
             const uint32_t dsh = level_shift(lv);
@@ -515,13 +572,13 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             __syncthreads();
             for (uint32_t i = tid; i < ncand; i += kThreads) {
                 const uint32_t b = (uint32_t)(s.cand[i] >> 32);
-                if (b - lo <= span) lds_hist_add(s, digit_at(b, dsh), pack_value(b));
+                if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, pack_value(b));
             }
             __syncthreads();
             for (int b = tid; b < kNB; b += kThreads) s.g[b] = s.hm[b];
             __syncthreads();
-            f = hist_find(s, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
-            lo |= (127u - f.bin) << dsh;
+            f = hist_find(s, kTopN, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
+            lo |= f.bin << dsh;
             span = (1u << dsh) - 1u;
         }
     }
@@ -534,20 +591,16 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     if (tid == 0) {
         const uint64_t q_thr = q_of_bits(thr);
         uint64_t w_tie = q_thr;
-        const uint64_t a = (P > Gm) ? (P - Gm) / n_eq : 0;
-        const uint64_t bk = ((uint32_t)p.top_k > n_gt) ? (q_thr * (uint64_t)((uint32_t)p.top_k - n_gt)) / n_eq : 0;
+        uint64_t a = (P > Gm) ? (P - Gm) : 0;
+        uint64_t bk = ((uint32_t)p.top_k > n_gt) ? (q_thr * (uint64_t)((uint32_t)p.top_k - n_gt)) : 0;
+        if (n_eq > 1) { a /= n_eq; bk /= n_eq; }
         if (a < w_tie) w_tie = a;
         if (bk < w_tie) w_tie = bk;
         if (w_tie == 0 && Gm == 0) w_tie = 1;
         const uint64_t S = Gm + (uint64_t)n_eq * w_tie;
         uint64_t r;
         if (p.inj_u) r = ceil_mul(p.inj_u[row], S);
-        else {
-            const uint32_t *st = p.rng + (size_t)row * 16;
-            uint32_t o[4];
-            philox4x32_10(st[2], st[3], st[4], st[5], st[0], st[1], o);
-            r = r_from_bits(((uint64_t)o[0] << 32) | o[1], S);
-        }
+        else r = r_from_bits(s.bc64[5], S);
         s.bc64[1] = w_tie; s.bc64[2] = S; s.bc64[3] = r;
         if (p.diag && part == 0) {
             rs_row_diag *d = p.diag + row;
@@ -625,7 +678,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         const uint64_t w2 = have ? weight(e4[2]) : 0, w3 = have ? weight(e4[3]) : 0;
         const uint64_t mine = w0 + w1 + w2 + w3;
         // inclusive scan over the 256 threads of slot jstar
-        uint64_t inc = wave_inclusive_scan_u64(mine, lane);
+        uint64_t inc = wave_inclusive_scan(mine);
         __syncthreads();
         if (lane == kWave - 1) s.u64[wave] = inc;
         __syncthreads();
@@ -692,7 +745,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             const uint32_t d = __hip_atomic_fetch_add(&rc->done, 1u, __ATOMIC_RELAXED, RS_AGENT);
             if (d == G - 1) {
                 // last workgroup out of this row: nobody reads the record any more
-                a_store(&rc->arrive, 0u); a_store(&rc->done, 0u); a_store(&rc->maxkey, 0u);
+                a_store(&rc->arrive, 0u); a_store(&rc->done, 0u);
                 a_store(&rc->cursor, 0u); a_store(&rc->index_p1, 0u);
             }
         }
