@@ -50,7 +50,7 @@ struct alignas(256) WsHeader {
 // Per-row record.  Everything a call reads before writing it is zero when the
 // call starts: the call itself re-zeroes what it used before it ends.
 struct alignas(256) RowCtl {
-    uint32_t arrive;      // barrier arrivals so far
+    uint32_t unused1;
     uint32_t done;        // workgroups finished with this row
     uint32_t unused0;
     uint32_t cursor;      // fill of cand[]
@@ -193,34 +193,25 @@ __device__ __forceinline__ void block_sum2_u64(Lds &s, uint64_t &a, uint64_t &b,
     for (int w = 0; w < kWaves; ++w) { a += s.u64[w * 2]; b += s.u64[w * 2 + 1]; }
 }
 
-// Meet the other workgroups of the row.  Every thread's contributions are
-// relaxed device-scope atomics issued before the call; each thread waits for
-// its own to be performed, then thread 0 arrives and polls.  Returns false
-// when the wait gave up (sticky error set).
-__device__ __forceinline__ bool cluster_barrier(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t G, uint32_t target)
-{
-    if (G == 1) { __syncthreads(); return true; }
-    wait_vmem();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(&rc->arrive, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        const uint64_t t0 = wall_clock64();
-        uint32_t spins = 0;
-        while (a_load(&rc->arrive) < target) {
-            if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
-                a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
-                s.abort = 1;
-                break;
-            }
+// Bounded wait bookkeeping: thread 0 looks at the wall clock now and then; the
+// verdict is read by everyone after a workgroup barrier, so it is uniform.
+struct SpinGuard {
+    uint64_t t0;
+    uint32_t spins;
+    __device__ __forceinline__ void start() { t0 = (uint64_t)wall_clock64(); spins = 0; }
+    // call by every thread once per polling round, before the round's __syncthreads
+    __device__ __forceinline__ void tick(Lds &s, WsHeader *hdr)
+    {
+        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
+            a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
+            s.abort = 1;
         }
     }
-    __syncthreads();
-    return s.abort == 0;
-}
+};
 
-__device__ __forceinline__ void lds_hist_zero(Lds &s)
+__device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)
 {
-    for (int b = threadIdx.x; b < kNB; b += kThreads) s.hm[b] = 0;
+    for (int b = threadIdx.x; b < nb; b += kThreads) s.hm[b] = 0;
 }
 // one LDS atomic per token: count and value together
 __device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint32_t value)
@@ -229,31 +220,51 @@ __device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint32_t valu
 }
 
 // Re-zero this workgroup's share of a global histogram (the cluster splits the bins).
-__device__ __forceinline__ void zero_slice(uint64_t *gh, uint32_t part, uint32_t G)
+__device__ __forceinline__ void zero_slice(uint64_t *gh, uint32_t nb, uint32_t part, uint32_t G)
 {
-    const uint32_t lo = (uint32_t)(((uint64_t)kNB * part) / G), hi = (uint32_t)(((uint64_t)kNB * (part + 1)) / G);
+    const uint32_t lo = (uint32_t)(((uint64_t)nb * part) / G), hi = (uint32_t)(((uint64_t)nb * (part + 1)) / G);
     for (uint32_t b = lo + threadIdx.x; b < hi; b += kThreads) a_store(&gh[b], (uint64_t)0);
 }
 
 // Sum the workgroup histograms of a cluster: add mine (s.hm, kept) into the
-// row's global bins, meet, read the totals into s.g.  A cluster of one copies
-// its own.
-__device__ __forceinline__ bool hist_combine(Lds &s, RowCtl *rc, WsHeader *hdr, uint32_t G, uint32_t target, uint64_t *gh)
+// row's global bins with one 64-bit atomic per non-empty bin, then read the
+// bins back until their counts add up to `expected` -- count and value of a
+// contribution arrive in one word, so a complete count means complete data
+// and no arrival counter is needed.  The totals end in s.g.  A cluster of one
+// copies its own.  Returns false when the wait gave up.
+__device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, uint64_t *gh, int nb, uint32_t expected,
+                                             int lane, int wave)
 {
     __syncthreads();
     if (G == 1) {
-        for (int b = threadIdx.x; b < kNB; b += kThreads) s.g[b] = s.hm[b];
+        for (int b = threadIdx.x; b < nb; b += kThreads) s.g[b] = s.hm[b];
         __syncthreads();
         return true;
     }
-    for (int b = threadIdx.x; b < kNB; b += kThreads) {
+    for (int b = threadIdx.x; b < nb; b += kThreads) {
         const uint64_t v = s.hm[b];
         if (v) a_add(&gh[b], v);
     }
-    if (!cluster_barrier(s, rc, hdr, G, target)) return false;
-    for (int b = threadIdx.x; b < kNB; b += kThreads) s.g[b] = a_load(&gh[b]);
-    __syncthreads();
-    return true;
+    SpinGuard guard;
+    guard.start();
+    for (;;) {
+        uint32_t c = 0;
+        for (int b = threadIdx.x; b < nb; b += kThreads) {
+            const uint64_t w = a_load(&gh[b]);
+            s.g[b] = w;
+            c += pack_count(w);
+        }
+        c = wave_sum(c);
+        guard.tick(s, hdr);
+        __syncthreads();
+        if (lane == 0) s.u32[wave] = c;
+        __syncthreads();
+        uint32_t total = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) total += s.u32[w];
+        if (total == expected) return true;
+        if (s.abort) return false;
+    }
 }
 
 // Scan s.g from index `top` downwards (largest e first) and find the first
@@ -313,6 +324,36 @@ __device__ __forceinline__ Found hist_find(Lds &s, uint32_t top, uint32_t cnt0, 
     return s.found;
 }
 
+// The same for a 128-bin level (all tokens share the exponent ex): one wave,
+// lane l owns indices 127-2l and 126-2l, no LDS exchange inside the scan.
+__device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint32_t cnt0, uint64_t mass0,
+                                              uint64_t top_k, int ex, int lane, int wave)
+{
+    if (wave == 0) {
+        const uint64_t w0 = arr[127 - 2 * lane], w1 = arr[126 - 2 * lane];
+        const uint32_t c0 = pack_count(w0), c1 = pack_count(w1);
+        const uint64_t m0 = pack_mass(w0, ex), m1 = pack_mass(w1, ex);
+        const uint32_t cs = c0 + c1;
+        const uint64_t ms = m0 + m1;
+        const uint64_t mi = wave_inclusive_scan(ms);
+        const uint32_t ci = wave_inclusive_scan(cs);
+        const uint64_t P = s.P;
+        const uint64_t r0 = (uint64_t)cnt0 + ci - cs, q0 = mass0 + mi - ms;      // before my first bin
+        const uint64_t r1 = r0 + c0, q1 = q0 + m0;                               // before my second bin
+        const uint64_t r2 = r1 + c1, q2 = q1 + m1;
+        const bool s0 = r0 >= top_k || q0 >= P, s1 = r1 >= top_k || q1 >= P, s2 = r2 >= top_k || q2 >= P;
+        if (!s0 && s1) {
+            s.found.bin = 127u - 2u * (uint32_t)lane;
+            s.found.cnt_above = (uint32_t)r0; s.found.cnt_bin = c0; s.found.mass_above = q0; s.found.mass_bin = m0;
+        } else if (!s1 && s2) {
+            s.found.bin = 126u - 2u * (uint32_t)lane;
+            s.found.cnt_above = (uint32_t)r1; s.found.cnt_bin = c1; s.found.mass_above = q1; s.found.mass_bin = m1;
+        }
+    }
+    __syncthreads();
+    return s.found;
+}
+
 // Mass of this workgroup's own tokens in the bins above index `bin` (larger
 // e), from s.hm, summed over the workgroup.
 template <typename ExFn>
@@ -354,7 +395,6 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         s.bc64[5] = ((uint64_t)o[0] << 32) | o[1];
     }
     RowCtl *rc = p.ctl + row;
-    uint32_t bar = 0;                                   // barriers passed
 
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const uint32_t base4 = part * (uint32_t)(kThreads * R) + (uint32_t)tid;
@@ -417,7 +457,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             }
         }
         const uint32_t k = block_max_u32(s, fkey(lmax), lane, wave);
-        lds_hist_zero(s);
+        lds_hist_zero(s, kNB);
         uint32_t kmax = k;
         if (G > 1) {
             // Exchange of the slice maxima without a counter: every workgroup writes its
@@ -461,7 +501,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         for (int j = 0; j < R; ++j)
             if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
     }
-    if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->h[0])) return;
+    if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return;
     if (G > 1 && tid == 0) a_store(&rc->mx[part], 0u);   // every workgroup has read the maxima by now
     const uint64_t top_k = (uint64_t)p.top_k;
 
@@ -481,8 +521,9 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     while (f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
         ++levels;
         const uint32_t dsh = level_shift(levels);
+        const uint32_t expect = f.cnt_bin;
         __syncthreads();
-        lds_hist_zero(s);
+        lds_hist_zero(s, 128);
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < R; ++j)
@@ -493,28 +534,31 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                     if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, pack_value(b));
                 }
             }
-        if (!hist_combine(s, rc, p.hdr, G, ++bar * G, rc->h[levels - 1])) return;
-        if (G > 1) zero_slice(rc->h[levels - 2], part, G);      // everyone has read the level above by now
-        f = hist_find(s, kTopN, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
+        if (!hist_combine(s, p.hdr, G, rc->h[levels - 1], 128, expect, lane, wave)) return;
+        // every workgroup has finished reading the level above: it published this level after that
+        if (G > 1) zero_slice(rc->h[levels - 2], levels == 2 ? kNB : 128, part, G);
+        f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
         amass += local_mass_above(s, f.bin, kTopN, lane, wave, exc);
         mycnt = pack_count(s.hm[f.bin]);
         lo |= f.bin << dsh;
         span = (1u << dsh) - 1u;
     }
+    const uint32_t last_nb = levels == 1 ? kNB : 128;    // bins of the last summed level
 
     // If the undistinguished tokens are few, gather them (bits and index) so
-    // that every workgroup can finish alone.
+    // that every workgroup can finish alone.  Validity is in the data: a
+    // gathered entry is never 0, and A[] holds mass + 1.
     const bool gather = f.cnt_bin <= (uint32_t)kCap;
-    uint32_t ncand = 0;
+    const uint32_t ncand = gather ? f.cnt_bin : 0u;
+    uint64_t a_mine = 0;                                 // thread t < G: A[t] of workgroup t
     if (gather) {
-        ncand = f.cnt_bin;
         __syncthreads();
         if (tid == 0) {
             s.ctr = 0;
             if (G > 1) {
                 s.bc32[2] = mycnt ? __hip_atomic_fetch_add(&rc->cursor, mycnt, __ATOMIC_RELAXED, RS_AGENT) : 0u;
-                a_store(&rc->A[part], amass);
-            } else s.bc64[7] = amass;
+                a_store(&rc->A[part], amass + 1);
+            }
         }
         __syncthreads();
         const uint32_t gbase = G > 1 ? s.bc32[2] : 0u;
@@ -533,51 +577,44 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                 }
             }
         if (G > 1) {
-            if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
-            for (uint32_t i = tid; i < ncand; i += kThreads) s.cand[i] = a_load(&rc->cand[i]);
-            zero_slice(rc->h[levels - 1], part, G);
-        }
+            SpinGuard guard;
+            guard.start();
+            for (;;) {
+                uint32_t valid = 0;
+                for (uint32_t i = tid; i < ncand; i += kThreads) {
+                    const uint64_t w = a_load(&rc->cand[i]);
+                    s.cand[i] = w;
+                    valid += w != 0;
+                }
+                if ((uint32_t)tid < G) { a_mine = a_load(&rc->A[tid]); valid += a_mine != 0; }
+                valid = wave_sum(valid);
+                guard.tick(s, p.hdr);
+                __syncthreads();
+                if (lane == 0) s.u32[wave] = valid;
+                __syncthreads();
+                uint32_t total = 0;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) total += s.u32[w];
+                if (total == ncand + G) break;
+                if (s.abort) return;
+            }
+            a_mine -= (uint32_t)tid < G ? 1u : 0u;
+            // every workgroup wrote its entries after it had read the last histogram level
+            zero_slice(rc->h[levels - 1], last_nb, part, G);
+        } else a_mine = tid == 0 ? amass : 0;
         __syncthreads();
 
-        if (ncand <= (uint32_t)kWave) {
-            // A handful of tokens: every thread ranks one of them against all the others.
-            // Token v is a valid threshold when the kept set {e >= v} is sufficient; the
-            // threshold is the largest such v.
-            const uint32_t mine = (uint32_t)tid < ncand ? (uint32_t)(s.cand[tid] >> 32) : 0u;
-            uint32_t cge = 0, cgt = 0;
-            uint64_t mge = 0;
-            for (uint32_t i = 0; i < ncand; ++i) {
-                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
-                if (b >= mine) { ++cge; mge += q_of_bits(b); }
-                if (b > mine) ++cgt;
-            }
-            const bool ok = (uint32_t)tid < ncand &&
-                            ((uint64_t)f.cnt_above + cge >= top_k || f.mass_above + mge >= P);
-            const uint32_t best = block_max_u32(s, ok ? mine : 0u, lane, wave);
-            if (ok && mine == best) {                    // ties write the same values
-                s.found.bin = 0;
-                s.found.cnt_above = f.cnt_above + cgt; s.found.cnt_bin = cge - cgt;
-                s.found.mass_above = f.mass_above + mge - (uint64_t)(cge - cgt) * q_of_bits(mine);
-                s.found.mass_bin = 0;
-            }
-            __syncthreads();
-            f = s.found;
-            lo = best; span = 0;
-        } else
         // resolve the remaining digits on the gathered tokens, in LDS
         for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels; ++lv) {
             const uint32_t dsh = level_shift(lv);
-            __syncthreads();
-            lds_hist_zero(s);
+            lds_hist_zero(s, 128);
             __syncthreads();
             for (uint32_t i = tid; i < ncand; i += kThreads) {
                 const uint32_t b = (uint32_t)(s.cand[i] >> 32);
                 if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, pack_value(b));
             }
             __syncthreads();
-            for (int b = tid; b < kNB; b += kThreads) s.g[b] = s.hm[b];
-            __syncthreads();
-            f = hist_find(s, kTopN, f.cnt_above, f.mass_above, top_k, p.top_p, false, lane, wave, exc);
+            f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
             lo |= f.bin << dsh;
             span = (1u << dsh) - 1u;
         }
@@ -632,10 +669,8 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             if (g < part) cb += w;
             if (g == part) cm += w;
         }
-        if (G > 1) {
-            if ((uint32_t)tid < part) cb += a_load(&rc->A[tid]);
-            if ((uint32_t)tid == part) cm += a_load(&rc->A[tid]);
-        } else if (tid == 0) cm += s.bc64[7];
+        if ((uint32_t)tid < part) cb += a_mine;
+        if ((uint32_t)tid == part) cm += a_mine;
         block_sum2_u64(s, cb, cm, lane, wave);
         before = cb; wblock = cm;
     } else {
@@ -645,12 +680,27 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             if (j < nv) wloc += slot_weight(j);
         wblock = block_sum_u64(s, wloc, lane, wave);
         if (G > 1) {
-            if (tid == 0) a_store(&rc->A[part], wblock);
-            if (!cluster_barrier(s, rc, p.hdr, G, ++bar * G)) return;
-            zero_slice(rc->h[levels - 1], part, G);
-            uint64_t bf = 0;
-            if ((uint32_t)tid < part) bf = a_load(&rc->A[tid]);
-            before = block_sum_u64(s, bf, lane, wave);
+            // exchange the kept weights through A[] (weight + 1, never 0)
+            if (tid == 0) a_store(&rc->A[part], wblock + 1);
+            uint64_t v = 0;
+            SpinGuard guard;
+            guard.start();
+            for (;;) {
+                uint32_t valid = 0;
+                if ((uint32_t)tid < G) { v = a_load(&rc->A[tid]); valid = v != 0; }
+                valid = wave_sum(valid);
+                guard.tick(s, p.hdr);
+                __syncthreads();
+                if (lane == 0) s.u32[wave] = valid;
+                __syncthreads();
+                uint32_t total = 0;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) total += s.u32[w];
+                if (total == G) break;
+                if (s.abort) return;
+            }
+            zero_slice(rc->h[levels - 1], last_nb, part, G);
+            before = block_sum_u64(s, (uint32_t)tid < part ? v - 1 : 0ull, lane, wave);
         }
     }
     const bool owner = before < r && r <= before + wblock;   // block-uniform
@@ -734,20 +784,22 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
 
     // ---- leave: advance the RNG, clean the row record, reset the launch ----
     __syncthreads();
+    if (G > 1) {
+        if (tid == 0) s.bc32[0] = __hip_atomic_fetch_add(&rc->done, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        __syncthreads();
+        if (s.bc32[0] == G - 1) {
+            // last workgroup out of this row: nobody reads the record any more
+            for (uint32_t i = tid; i < ncand; i += kThreads) a_store(&rc->cand[i], (uint64_t)0);
+            if ((uint32_t)tid < G) a_store(&rc->A[tid], (uint64_t)0);
+            if (tid == 0) { a_store(&rc->done, 0u); a_store(&rc->cursor, 0u); a_store(&rc->index_p1, 0u); }
+        }
+    }
     if (tid == 0) {
         if (part == 0 && !p.inj_u) {
             uint32_t *st = p.rng + (size_t)row * 16;
             const uint32_t lo32 = st[2] + 1;
             st[2] = lo32;
             if (lo32 == 0) st[3] += 1;
-        }
-        if (G > 1) {
-            const uint32_t d = __hip_atomic_fetch_add(&rc->done, 1u, __ATOMIC_RELAXED, RS_AGENT);
-            if (d == G - 1) {
-                // last workgroup out of this row: nobody reads the record any more
-                a_store(&rc->arrive, 0u); a_store(&rc->done, 0u);
-                a_store(&rc->cursor, 0u); a_store(&rc->index_p1, 0u);
-            }
         }
         wait_vmem();
         const uint32_t fin = __hip_atomic_fetch_add(&p.hdr->finished, 1u, __ATOMIC_RELAXED, RS_AGENT);
