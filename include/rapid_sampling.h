@@ -39,22 +39,23 @@ extern "C" {
  * tensor returned by setup_rand keeps its shape. */
 #define RS_STATE_BYTES_PER_ROW 64
 
-/* Optional per-row diagnostics (device memory, B records). */
+/* Optional per-row diagnostics (device memory, B records).  128-bit
+ * quantities are (low word, high word). */
 typedef struct rs_row_diag {
     float    xmax;        /* row maximum of the scaled logits                 */
-    uint32_t emin_bits;   /* bit pattern of the smallest e in the row         */
-    uint64_t D;           /* sum of the fixed-point weights q over the row    */
-    uint64_t P;           /* ceil(top_p * D)                                  */
-    uint32_t left_bits;   /* lower end of the search interval at loop exit    */
+    uint32_t emin_bits;   /* unused by the library (0)                        */
+    uint64_t D[2];        /* sum of the exact weights W = e * 2^63 over the row */
+    uint64_t P[2];        /* ceil(top_p * D)                                  */
+    uint32_t left_bits;   /* same as thr_bits                                 */
     uint32_t thr_bits;    /* bit pattern of the smallest kept e               */
-    uint32_t rounds;      /* passes of the threshold search                   */
+    uint32_t rounds;      /* histogram levels summed over the cluster         */
     uint32_t n_gt;        /* tokens with e >  threshold                       */
     uint32_t n_eq;        /* tokens with e == threshold                       */
     int32_t  index;       /* sampled token                                    */
-    uint64_t G;           /* sum of q over e > threshold                      */
+    uint64_t G[2];        /* sum of W over e > threshold                      */
     uint64_t w_tie;       /* weight of each token with e == threshold         */
-    uint64_t S;           /* G + n_eq * w_tie                                 */
-    uint64_t r;           /* target of the inverse CDF, 1 <= r <= S           */
+    uint64_t S[2];        /* G + n_eq * w_tie                                 */
+    uint64_t r[2];        /* target of the inverse CDF, 1 <= r <= S           */
 } rs_row_diag;
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -118,9 +119,9 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  *                     1 <= top_k <= V, 0 < top_p <= 1.
  *   workspace_device  rs_workspace_bytes(B,V) bytes, initialised once.
  *   diag_device       B rs_row_diag records, or NULL.
- *   e_bits_device     (B,V) uint32: bit patterns of e = exp2(x - max) per
- *                     token, or NULL.  Together with diag.thr_bits this is
- *                     the kept set {e >= thr}.
+ *   e_bits_device     (B,V) uint32: bit patterns of e = 2^(x - floor(max x))
+ *                     per token (2^-40 <= e < 2), or NULL.  Together with
+ *                     diag.thr_bits this is the kept set {e >= thr}.
  *
  * Calls that share a workspace must be ordered on one stream.
  */

@@ -23,25 +23,36 @@ def build(force=False):
 class Diag(C.Structure):
     _fields_ = [
         ("xmax", C.c_float), ("emin_bits", C.c_uint32),
-        ("D", C.c_uint64), ("P", C.c_uint64),
+        ("D", C.c_uint64 * 2), ("P", C.c_uint64 * 2),
         ("left_bits", C.c_uint32), ("thr_bits", C.c_uint32),
         ("rounds", C.c_uint32), ("n_gt", C.c_uint32),
         ("n_eq", C.c_uint32), ("index", C.c_int32),
-        ("G", C.c_uint64), ("w_tie", C.c_uint64),
-        ("S", C.c_uint64), ("r", C.c_uint64),
+        ("G", C.c_uint64 * 2), ("w_tie", C.c_uint64),
+        ("S", C.c_uint64 * 2), ("r", C.c_uint64 * 2),
     ]
 
     def asdict(self):
-        return {n: getattr(self, n) for n, _ in self._fields_}
+        """128-bit fields come back as Python integers."""
+        out = {}
+        for n, t in self._fields_:
+            v = getattr(self, n)
+            out[n] = (int(v[0]) | (int(v[1]) << 64)) if t is C.c_uint64 * 2 else v
+        return out
 
 
+# numpy view of the same record; 128-bit quantities are (low, high) uint64 pairs
 DIAG_DTYPE = np.dtype([
-    ("xmax", "<f4"), ("emin_bits", "<u4"), ("D", "<u8"), ("P", "<u8"),
+    ("xmax", "<f4"), ("emin_bits", "<u4"), ("D", "<u8", (2,)), ("P", "<u8", (2,)),
     ("left_bits", "<u4"), ("thr_bits", "<u4"), ("rounds", "<u4"), ("n_gt", "<u4"),
-    ("n_eq", "<u4"), ("index", "<i4"), ("G", "<u8"), ("w_tie", "<u8"),
-    ("S", "<u8"), ("r", "<u8"),
+    ("n_eq", "<u4"), ("index", "<i4"), ("G", "<u8", (2,)), ("w_tie", "<u8"),
+    ("S", "<u8", (2,)), ("r", "<u8", (2,)),
 ])
-assert DIAG_DTYPE.itemsize == C.sizeof(Diag) == 80
+assert DIAG_DTYPE.itemsize == C.sizeof(Diag) == 120
+
+
+def u128(pair):
+    """(low, high) uint64 pair -> Python int."""
+    return int(pair[0]) | (int(pair[1]) << 64)
 
 
 class LiteralDiag(C.Structure):
@@ -69,14 +80,14 @@ def lib():
         L.rs_oracle_sf.argtypes = [C.c_float]
         L.rs_oracle_scale.restype = C.c_float
         L.rs_oracle_scale.argtypes = [C.c_float, C.c_float, C.c_int, C.c_float]
-        L.rs_oracle_exp2c.restype = C.c_float
-        L.rs_oracle_exp2c.argtypes = [C.c_float]
-        L.rs_oracle_q.restype = u64
-        L.rs_oracle_q.argtypes = [C.c_float]
-        L.rs_oracle_ceil_mul.restype = u64
-        L.rs_oracle_ceil_mul.argtypes = [C.c_float, u64]
-        L.rs_oracle_r_from_bits.restype = u64
-        L.rs_oracle_r_from_bits.argtypes = [u64, u64]
+        L.rs_oracle_e_bits.restype = C.c_uint32
+        L.rs_oracle_e_bits.argtypes = [C.c_float, C.c_float]
+        L.rs_oracle_w.restype = u64
+        L.rs_oracle_w.argtypes = [C.c_uint32]
+        L.rs_oracle_ceil_mul.restype = None
+        L.rs_oracle_ceil_mul.argtypes = [C.c_float, u64, u64, C.POINTER(u64)]
+        L.rs_oracle_r_from_bits.restype = None
+        L.rs_oracle_r_from_bits.argtypes = [u64, u64, u64, C.POINTER(u64)]
         L.rs_oracle_normalize.restype = C.c_int
         L.rs_oracle_normalize.argtypes = [C.c_double, C.c_int64, C.c_double, C.c_int64, C.c_int64,
                                           C.c_int64, fp, C.POINTER(C.c_int32), fp]
@@ -87,7 +98,7 @@ def lib():
         L.rs_oracle_rng_init.restype = None
         L.rs_oracle_rng_init.argtypes = [C.c_void_p, u64, C.c_int32]
         L.rs_oracle_thr_by_sort.restype = C.c_uint32
-        L.rs_oracle_thr_by_sort.argtypes = [C.c_void_p, C.c_int32, C.c_int32, u64]
+        L.rs_oracle_thr_by_sort.argtypes = [C.c_void_p, C.c_int32, C.c_int32, u64, u64]
         L.rs_oracle_row.restype = None
         L.rs_oracle_row.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_float,
                                     C.c_int, C.c_float, u64, C.c_float, C.c_float, C.c_float,
@@ -121,16 +132,31 @@ def normalize(temperature, top_k, top_p, V, B=1, T=1):
     return c.value, k.value, p.value
 
 
-def exp2c(d):
-    d = np.ascontiguousarray(d, dtype=np.float32)
-    f = lib().rs_oracle_exp2c
-    return np.array([f(float(v)) for v in d.ravel()], dtype=np.float32).reshape(d.shape)
+def e_bits(x, M):
+    """Bit patterns of e = 2^(x - M) for scaled logits x (array) and M = floor(max x)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    f = lib().rs_oracle_e_bits
+    return np.array([f(float(v), float(M)) for v in x.ravel()], dtype=np.uint32).reshape(x.shape)
 
 
-def q_of(e):
-    e = np.ascontiguousarray(e, dtype=np.float32)
-    f = lib().rs_oracle_q
-    return np.array([f(float(v)) for v in e.ravel()], dtype=np.uint64).reshape(e.shape)
+def w_of(bits):
+    """Exact integer weights W = e * 2^63 of bit patterns (array) as uint64."""
+    bits = np.ascontiguousarray(bits, dtype=np.uint32)
+    m = (bits & np.uint32(0x7FFFFF)).astype(np.uint64) | np.uint64(0x800000)
+    ex = (bits >> np.uint32(23)).astype(np.uint64)
+    return m << (ex - np.uint64(87))
+
+
+def ceil_mul(f, s):
+    out = (C.c_uint64 * 2)()
+    lib().rs_oracle_ceil_mul(f, s & (2 ** 64 - 1), s >> 64, out)
+    return int(out[0]) | (int(out[1]) << 64)
+
+
+def r_from_bits(u64, s):
+    out = (C.c_uint64 * 2)()
+    lib().rs_oracle_r_from_bits(u64, s & (2 ** 64 - 1), s >> 64, out)
+    return int(out[0]) | (int(out[1]) << 64)
 
 
 def philox(ctr, key):
@@ -205,7 +231,7 @@ def sample_batch(logits, c, top_k, top_p, rng=None, injected_u=None, penalties=N
 
 def thr_by_sort(e_bits, top_k, P):
     e_bits = np.ascontiguousarray(e_bits, dtype=np.uint32)
-    return lib().rs_oracle_thr_by_sort(_ptr(e_bits), e_bits.shape[0], top_k, P)
+    return lib().rs_oracle_thr_by_sort(_ptr(e_bits), e_bits.shape[0], top_k, P & (2 ** 64 - 1), P >> 64)
 
 
 def literal_row(logits, c, top_k, top_p, u1, u2, variant=0, penalties=None,

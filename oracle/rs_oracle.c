@@ -11,18 +11,23 @@
  *   tie compensation                         :365-371
  *   inverse-CDF pick, first index reached    :374-426
  *   penalty decay with one-hot add           :427-437
- * What is restated so that the result is independent of summation order:
- *   - exp2 is a fixed degree-5 Horner polynomial on the fractional part
- *     (hardware/libm exp2f are not bit-identical across machines), with
- *     the argument clamped at -64 so that every e is a normal float;
- *   - the probability of token i is carried as the integer
- *         q_i = max(1, floor(e_i * 2^40)),    e_max = 1 exactly,
- *     the row total D = sum q_i replaces the float denominator, and "mass
- *     >= top_p" becomes  sum q >= P = ceil(top_p * D)  in exact arithmetic
- *     (the reference divides by the float denominator and sums floats,
- *     :248,:285-292);
+ * What is restated so that the result is independent of summation order AND
+ * of where the row maximum sits (so that a slice of a row can be worked
+ * before the maximum of the whole row is known):
+ *   - exp2 splits x itself, not x - max:  n = floor(x), f = x - n (exact),
+ *     e = poly5(f) * 2^(n - M) with M = floor(max x), a fixed degree-5 Horner
+ *     polynomial with positive coefficients (monotone, poly(1) < 2).  The
+ *     significand of e depends on x alone; the maximum only shifts the
+ *     exponent.  e is clamped from below at 2^-40 (tokens further down all
+ *     become exactly 2^-40), so 2^-40 <= e < 2 and e_max in [1,2);
+ *   - the probability of token i is carried as the exact integer
+ *         W_i = e_i * 2^63  =  significand24(e_i) << (exponent(e_i) - 87),
+ *     the row total D = sum W_i (up to 2^84: 128-bit) replaces the float
+ *     denominator, and "mass >= top_p" becomes  sum W >= P = ceil(top_p * D)
+ *     in exact arithmetic (the reference divides by the float denominator
+ *     and sums floats, :248,:285-292);
  *   - tie compensation and the CDF are integer: each token equal to the
- *     threshold weighs  min(q_thr, (P-G)/n_eq, q_thr*(k-n_gt)/n_eq)
+ *     threshold weighs  min(W_thr, (P-G)/n_eq, W_thr*(k-n_gt)/n_eq)
  *     (the reference's  thr * min(1,(top_p-sgtp)/(thr*neqk),(top_k-sgtk)/neqk)
  *     :368-371,:404), and one uniform picks the first index whose inclusive
  *     CDF reaches r = ceil(u*S) (the reference spends two uniforms on a
@@ -39,6 +44,7 @@ typedef unsigned __int128 u128;
 
 static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
 static inline float    u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static inline void     put128(uint64_t out[2], u128 v) { out[0] = (uint64_t)v; out[1] = (uint64_t)(v >> 64); }
 
 /* sampling.cu:131-134 : NaN -> 0, +-Inf -> +-FLT_MAX */
 float rs_oracle_sf(float x)
@@ -56,13 +62,13 @@ float rs_oracle_scale(float logit, float penalty, int has_penalty, float c)
 }
 
 /*
- * exp2 for d <= 0 (d = x - max, sampling.cu:235), d clamped to >= -64 first
- * (tokens further down all get e = 2^-64, whose weight q is the minimum 1).
- * n = floor(d), f = d - n is exact and lies in [0,1]; 2^f is a degree-5
- * minimax polynomial (relative error 8.3e-8) evaluated by Horner with fmaf;
- * the result is scaled by 2^n exactly.  All coefficients are positive, so the
- * polynomial is monotone in f, and poly(1) <= 2 = 2*poly(0), so exp2c is
- * monotone in d.
+ * Bit pattern of e = 2^(x - M) for a row whose maximum has floor M
+ * (sampling.cu:235 computes exp2f(x - max); the common factor 2^(max - M)
+ * cancels in every probability).  n = floor(x) and f = x - n are exact, f in
+ * [0,1]; 2^f is a degree-5 minimax polynomial (relative error 8.3e-8)
+ * evaluated by Horner with fmaf, all coefficients positive, so it is monotone
+ * in f and poly(1) < 2 = 2*poly(0): e is monotone in x.  The exponent n - M
+ * is added to the exponent field; below 2^-40 the result is 2^-40 exactly.
  */
 static const float RS_C1 = 0x1.62e4bap-1f;
 static const float RS_C2 = 0x1.ebdb56p-3f;
@@ -70,29 +76,31 @@ static const float RS_C3 = 0x1.c91ce6p-5f;
 static const float RS_C4 = 0x1.277856p-7f;
 static const float RS_C5 = 0x1.e974fap-10f;
 
-float rs_oracle_exp2c(float d)
+uint32_t rs_oracle_e_bits(float x, float M)
 {
-    d = fmaxf(d, (float)RS_EXP_CLAMP);
-    float n = floorf(d);
-    float f = d - n;
+    float n = floorf(x);
+    float f = x - n;
     float p = RS_C5;
     p = fmaf(p, f, RS_C4);
     p = fmaf(p, f, RS_C3);
     p = fmaf(p, f, RS_C2);
     p = fmaf(p, f, RS_C1);
     p = fmaf(p, f, 1.0f);
-    return ldexpf(p, (int)n);
+    float k = fmaxf(n - M, -41.0f);             /* <= 0; anything below -40 is clamped anyway */
+    uint32_t b = f2u(p) + ((uint32_t)(int32_t)k << 23);
+    return b < RS_E_MIN_BITS ? RS_E_MIN_BITS : b;
 }
 
-/* fixed-point weight of a token: max(1, floor(e * 2^40)) */
-uint64_t rs_oracle_q(float e)
+/* exact weight of a token: e * 2^63 = significand24 << (exponent - 87), in [2^23, 2^64) */
+uint64_t rs_oracle_w(uint32_t e_bits)
 {
-    uint64_t q = (uint64_t)(e * 0x1p40f);   /* power-of-two scale: exact */
-    return q ? q : 1;
+    uint64_t m = (e_bits & 0x7FFFFFu) | 0x800000u;
+    int ex = (int)(e_bits >> 23);
+    return m << (ex - 87);
 }
 
-/* ceil(f * s) for a float 0 < f <= 1, exact; clamped to [1, s] */
-uint64_t rs_oracle_ceil_mul(float f, uint64_t s)
+/* ceil(f * s) for a float 0 < f <= 1 and s < 2^100, exact; clamped to [1, s] */
+static u128 ceil_mul128(float f, u128 s)
 {
     if (!(f > 0.0f)) return 1;
     if (f >= 1.0f) return s;
@@ -101,16 +109,30 @@ uint64_t rs_oracle_ceil_mul(float f, uint64_t s)
     uint64_t m = b & 0x7FFFFFu;
     if (ex == 0) ex = 1; else m |= 0x800000u;     /* subnormal / normal   */
     int sh = 150 - ex;                            /* f = m * 2^-sh, sh>=24 */
-    u128 prod = (u128)m * s;                      /* < 2^24 * 2^64 = 2^88  */
-    uint64_t r;
-    if (sh >= 96) r = 1;                          /* 0 < prod < 2^88 < 2^sh */
-    else {
-        u128 one = (u128)1 << sh;
-        r = (uint64_t)((prod + one - 1) >> sh);
-    }
+    u128 prod = (u128)m * s;                      /* < 2^24 * 2^100        */
+    u128 r;
+    if (sh >= 126) r = 1;                         /* 0 < prod < 2^124 < 2^sh */
+    else r = (prod + (((u128)1 << sh) - 1)) >> sh;
     if (r < 1) r = 1;
     if (r > s) r = s;
     return r;
+}
+
+void rs_oracle_ceil_mul(float f, uint64_t s_lo, uint64_t s_hi, uint64_t out[2])
+{
+    put128(out, ceil_mul128(f, ((u128)s_hi << 64) | s_lo));
+}
+
+/* 64 random bits -> r in [1,S]: floor(u64 * S / 2^64) + 1 */
+static u128 r_from_bits128(uint64_t u64, u128 S)
+{
+    uint64_t s_lo = (uint64_t)S, s_hi = (uint64_t)(S >> 64);
+    return (u128)u64 * s_hi + (uint64_t)(((u128)u64 * s_lo) >> 64) + 1;
+}
+
+void rs_oracle_r_from_bits(uint64_t u64, uint64_t s_lo, uint64_t s_hi, uint64_t out[2])
+{
+    put128(out, r_from_bits128(u64, ((u128)s_hi << 64) | s_lo));
 }
 
 /* sampling.cu:474-486 / :986-1011 */
@@ -158,12 +180,6 @@ void rs_oracle_philox_draw(uint64_t seed, uint64_t row, uint64_t n, uint32_t out
     rs_oracle_philox(ctr, key, out);
 }
 
-/* 64 random bits -> r in [1,S], each value equally likely up to 2^-64 */
-uint64_t rs_oracle_r_from_bits(uint64_t u64, uint64_t S)
-{
-    return (uint64_t)(((u128)u64 * S) >> 64) + 1;
-}
-
 void rs_oracle_rng_init(uint32_t *rng, uint64_t seed, int32_t B)
 {
     for (int32_t b = 0; b < B; b++) {
@@ -176,23 +192,24 @@ void rs_oracle_rng_init(uint32_t *rng, uint64_t seed, int32_t B)
 }
 
 /* ---- definitional threshold: the largest t with
- *      count{e >= t} >= top_k  or  sum{q : e >= t} >= P   ------------------ */
+ *      count{e >= t} >= top_k  or  sum{W : e >= t} >= P   ------------------ */
 static int cmp_desc_u32(const void *a, const void *b)
 {
     uint32_t x = *(const uint32_t *)a, y = *(const uint32_t *)b;
     return (x < y) - (x > y);
 }
 
-uint32_t rs_oracle_thr_by_sort(const uint32_t *e_bits, int32_t V, int32_t top_k, uint64_t P)
+uint32_t rs_oracle_thr_by_sort(const uint32_t *e_bits, int32_t V, int32_t top_k, uint64_t P_lo, uint64_t P_hi)
 {
+    const u128 P = ((u128)P_hi << 64) | P_lo;
     uint32_t *s = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)V);
     memcpy(s, e_bits, sizeof(uint32_t) * (size_t)V);
     qsort(s, (size_t)V, sizeof(uint32_t), cmp_desc_u32);
-    uint64_t mass = 0;
+    u128 mass = 0;
     uint32_t thr = s[V - 1];
     for (int32_t i = 0; i < V;) {
         int32_t j = i;
-        while (j < V && s[j] == s[i]) { mass += rs_oracle_q(u2f(s[j])); j++; }
+        while (j < V && s[j] == s[i]) { mass += rs_oracle_w(s[j]); j++; }
         if ((int64_t)j >= top_k || mass >= P) { thr = s[i]; break; }
         i = j;
     }
@@ -218,36 +235,38 @@ void rs_oracle_row(const float *logits, float *penalties, int32_t V,
         if (x[i] > xmax) xmax = x[i];
     }
     dg.xmax = xmax;
+    const float M = floorf(xmax);
 
-    /* 2. e = exp2(x - max), total D (sampling.cu:228-258 without the division) */
-    uint64_t D = 0;
+    /* 2. e = 2^(x - M), total D (sampling.cu:228-258 without the division) */
+    u128 D = 0;
     uint32_t emin = 0xFFFFFFFFu, emax = 0;
     for (int32_t i = 0; i < V; i++) {
-        float e = rs_oracle_exp2c(x[i] - xmax);
-        eb[i] = f2u(e);
-        D += rs_oracle_q(e);
+        eb[i] = rs_oracle_e_bits(x[i], M);
+        D += rs_oracle_w(eb[i]);
         if (eb[i] < emin) emin = eb[i];
         if (eb[i] > emax) emax = eb[i];
     }
-    uint64_t P = rs_oracle_ceil_mul(top_p, D);
-    dg.D = D; dg.P = P; dg.emin_bits = emin;
+    const u128 P = ceil_mul128(top_p, D);
+    put128(dg.D, D); put128(dg.P, P); dg.emin_bits = emin;
 
     /* 3. the reference's quaternary search, literally (sampling.cu:261-329),
      *    with exact counts and integer masses */
     uint32_t left = emin, right = emax + 1;
-    uint64_t cnt_x = (uint64_t)V, mass_x = D;
+    uint64_t cnt_x = (uint64_t)V;
+    u128 mass_x = D;
     uint32_t rounds = 0;
     while ((cnt_x > (uint64_t)top_k || mass_x > P) && left < right - 1) {
         uint32_t pz = (left + right) / 2;
         uint32_t py = (left + pz) / 2;
         uint32_t pw = (pz + right) / 2;
-        uint64_t cy = 0, cz = 0, cw = 0, my = 0, mz = 0, mw = 0;
+        uint64_t cy = 0, cz = 0, cw = 0;
+        u128 my = 0, mz = 0, mw = 0;
         for (int32_t i = 0; i < V; i++) {
             uint32_t b = eb[i];
-            uint64_t q = rs_oracle_q(u2f(b));
-            if (b >= py) { cy++; my += q; }
-            if (b >= pz) { cz++; mz += q; }
-            if (b >= pw) { cw++; mw += q; }
+            uint64_t w = rs_oracle_w(b);
+            if (b >= py) { cy++; my += w; }
+            if (b >= pz) { cz++; mz += w; }
+            if (b >= pw) { cw++; mw += w; }
         }
         rounds++;
         if (cy < (uint64_t)top_k && my < P) { right = py; continue; }
@@ -261,32 +280,32 @@ void rs_oracle_row(const float *logits, float *penalties, int32_t V,
     uint32_t thr = 0xFFFFFFFFu;
     for (int32_t i = 0; i < V; i++) if (eb[i] >= left && eb[i] < thr) thr = eb[i];
     uint32_t n_gt = 0, n_eq = 0;
-    uint64_t G = 0;
+    u128 G = 0;
     for (int32_t i = 0; i < V; i++) {
         if (eb[i] == thr) n_eq++;
-        else if (eb[i] > thr) { n_gt++; G += rs_oracle_q(u2f(eb[i])); }
+        else if (eb[i] > thr) { n_gt++; G += rs_oracle_w(eb[i]); }
     }
-    dg.thr_bits = thr; dg.n_gt = n_gt; dg.n_eq = n_eq; dg.G = G;
+    dg.thr_bits = thr; dg.n_gt = n_gt; dg.n_eq = n_eq; put128(dg.G, G);
 
     /* 5. tie compensation (sampling.cu:365-371), integer form */
-    uint64_t q_thr = rs_oracle_q(u2f(thr));
-    uint64_t w_tie = q_thr;
-    uint64_t a = (P > G) ? (P - G) / n_eq : 0;
-    uint64_t bk = ((uint32_t)top_k > n_gt) ? (q_thr * (uint64_t)((uint32_t)top_k - n_gt)) / n_eq : 0;
+    const uint64_t w_thr = rs_oracle_w(thr);
+    u128 w_tie = w_thr;
+    u128 a = (P > G) ? (P - G) / n_eq : 0;
+    u128 bk = ((uint32_t)top_k > n_gt) ? ((u128)w_thr * ((uint32_t)top_k - n_gt)) / n_eq : 0;
     if (a < w_tie) w_tie = a;
     if (bk < w_tie) w_tie = bk;
     if (w_tie == 0 && G == 0) w_tie = 1;
-    uint64_t S = G + (uint64_t)n_eq * w_tie;
-    dg.w_tie = w_tie; dg.S = S;
+    const u128 S = G + (u128)n_eq * w_tie;
+    dg.w_tie = (uint64_t)w_tie; put128(dg.S, S);
 
     /* 6. inverse CDF in index order; first index whose inclusive CDF >= r
      *    (the single false->true transition of sampling.cu:388-397,410-423) */
-    uint64_t r = use_u ? rs_oracle_ceil_mul(u, S) : rs_oracle_r_from_bits(u64, S);
-    dg.r = r;
-    uint64_t cdf = 0;
+    const u128 r = use_u ? ceil_mul128(u, S) : r_from_bits128(u64, S);
+    put128(dg.r, r);
+    u128 cdf = 0;
     int32_t idx = -1;
     for (int32_t i = 0; i < V; i++) {
-        uint64_t w = (eb[i] > thr) ? rs_oracle_q(u2f(eb[i])) : (eb[i] == thr ? w_tie : 0);
+        u128 w = (eb[i] > thr) ? (u128)rs_oracle_w(eb[i]) : (eb[i] == thr ? w_tie : 0);
         cdf += w;
         if (cdf >= r) { idx = i; break; }
     }

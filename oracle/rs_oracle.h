@@ -34,35 +34,34 @@
 extern "C" {
 #endif
 
-/* Fractional bits of the fixed-point weight q = max(1, floor(e * 2^RS_QBITS)). */
-#define RS_QBITS 40
-/* exp2c clamps its argument: exp2c(d) = exp2c(max(d, RS_EXP_CLAMP)) >= 2^-64. */
-#define RS_EXP_CLAMP (-64)
+/* e is clamped from below at 2^-40 (bit pattern 0x2B800000). */
+#define RS_E_MIN_BITS 0x2B800000u
 
-/* Per-row diagnostics; mirrors rs_row_diag of include/rapid_sampling.h. */
+/* Per-row diagnostics; mirrors rs_row_diag of include/rapid_sampling.h.
+ * 128-bit quantities are (low word, high word). */
 typedef struct {
     float    xmax;        /* row maximum of the scaled logits                 */
     uint32_t emin_bits;   /* bit pattern of the smallest e in the row         */
-    uint64_t D;           /* sum of q over the row                            */
-    uint64_t P;           /* ceil(top_p * D)                                  */
+    uint64_t D[2];        /* sum of the weights W over the row                */
+    uint64_t P[2];        /* ceil(top_p * D)                                  */
     uint32_t left_bits;   /* `left` when the reference's search loop ends     */
     uint32_t thr_bits;    /* smallest kept e  (the canonical threshold)       */
     uint32_t rounds;      /* passes of the search loop                        */
     uint32_t n_gt;        /* count of e >  thr                                */
     uint32_t n_eq;        /* count of e == thr                                */
     int32_t  index;       /* sampled token                                    */
-    uint64_t G;           /* sum of q over e > thr                            */
+    uint64_t G[2];        /* sum of W over e > thr                            */
     uint64_t w_tie;       /* weight of each token with e == thr               */
-    uint64_t S;           /* G + n_eq * w_tie                                 */
-    uint64_t r;           /* target of the inverse CDF, 1 <= r <= S           */
+    uint64_t S[2];        /* G + n_eq * w_tie                                 */
+    uint64_t r[2];        /* target of the inverse CDF, 1 <= r <= S           */
 } rs_oracle_diag;
 
 /* ---- element-wise canonical arithmetic -------------------------------- */
 float    rs_oracle_sf(float x);
 float    rs_oracle_scale(float logit, float penalty, int has_penalty, float c);
-float    rs_oracle_exp2c(float d);
-uint64_t rs_oracle_q(float e);
-uint64_t rs_oracle_ceil_mul(float f, uint64_t s);
+uint32_t rs_oracle_e_bits(float x, float M);
+uint64_t rs_oracle_w(uint32_t e_bits);
+void     rs_oracle_ceil_mul(float f, uint64_t s_lo, uint64_t s_hi, uint64_t out[2]);
 
 /* ---- host argument normalisation -------------------------------------- */
 /* returns 0, or -1 (V), -2 (B,T), -3 (temperature) like the reference's throws */
@@ -74,7 +73,7 @@ int rs_oracle_normalize(double temperature, int64_t top_k, double top_p,
 void     rs_oracle_philox(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
 /* draw #n of row `row` for `seed`: counter (n_lo, n_hi, row_lo, row_hi) */
 void     rs_oracle_philox_draw(uint64_t seed, uint64_t row, uint64_t n, uint32_t out[4]);
-uint64_t rs_oracle_r_from_bits(uint64_t u64, uint64_t S);
+void     rs_oracle_r_from_bits(uint64_t u64, uint64_t s_lo, uint64_t s_hi, uint64_t out[2]);
 
 /* ---- one row, canonical ------------------------------------------------ */
 /*
@@ -89,7 +88,7 @@ void rs_oracle_row(const float *logits, float *penalties, int32_t V,
                    uint32_t *e_bits_out, rs_oracle_diag *diag);
 
 /* definitional threshold by sorting (independent of the search loop) */
-uint32_t rs_oracle_thr_by_sort(const uint32_t *e_bits, int32_t V, int32_t top_k, uint64_t P);
+uint32_t rs_oracle_thr_by_sort(const uint32_t *e_bits, int32_t V, int32_t top_k, uint64_t P_lo, uint64_t P_hi);
 
 /* ---- a batch, canonical ------------------------------------------------ */
 /*

@@ -25,40 +25,41 @@ __device__ __forceinline__ float sf(float x)
     return fminf(fmaxf(y, -3.402823466e+38f), 3.402823466e+38f);
 }
 
-// exp2 for d <= 0, argument clamped at -64 (so the result is a normal float in
-// [2^-64, 1]): floor/fraction split, degree-5 Horner with positive
-// coefficients on the fraction (monotone), exact scale by 2^floor(d).
-// Returns the bit pattern.                 (reference: exp2f at sampling.cu:235)
-__device__ __forceinline__ uint32_t exp2c_bits(float d)
+typedef unsigned __int128 u128;
+
+constexpr uint32_t kEMinBits = 0x2B800000u;               // bit pattern of 2^-40, the smallest e
+
+// Bit pattern of e = 2^(x - M), M = floor(max x) of the row (reference:
+// exp2f(x - max) at sampling.cu:235; the common factor 2^(max - M) cancels in
+// every probability).  n = floor(x) and f = x - n are exact; 2^f is a degree-5
+// Horner polynomial with positive coefficients (monotone, poly(1) < 2); the
+// exponent n - M is added to the exponent field and the result is clamped
+// from below at 2^-40.  The significand depends on x alone, so a slice can
+// use its own M and be re-based later by an exponent shift.
+__device__ __forceinline__ uint32_t e_bits_of(float x, float M)
 {
-    d = fmaxf(d, -64.0f);
-    const float n = __builtin_floorf(d);
-    const float f = d - n;
+    const float n = __builtin_floorf(x);
+    const float f = x - n;
     float p = 0x1.e974fap-10f;
     p = __builtin_fmaf(p, f, 0x1.277856p-7f);
     p = __builtin_fmaf(p, f, 0x1.c91ce6p-5f);
     p = __builtin_fmaf(p, f, 0x1.ebdb56p-3f);
     p = __builtin_fmaf(p, f, 0x1.62e4bap-1f);
     p = __builtin_fmaf(p, f, 1.0f);
-    // p in [1,2], n in [-64,0]: p * 2^n by adding n to the exponent field
-    return __float_as_uint(p) + ((uint32_t)(int)n << 23);
+    const float k = fmaxf(n - M, -41.0f);
+    const uint32_t b = __float_as_uint(p) + ((uint32_t)(int)k << 23);
+    return max(b, kEMinBits);
 }
 
-// Fixed-point weight of a token from the bit pattern of e (2^-64..1):
-// q = max(1, floor(e * 2^40)).
-__device__ __forceinline__ uint64_t q_of_bits(uint32_t b)
+// Exact weight of a token from the bit pattern of e (2^-40 <= e < 2):
+// W = e * 2^63 = significand24 << (exponent - 87), in [2^23, 2^64).
+__device__ __forceinline__ uint64_t w_of_bits(uint32_t b)
 {
-    const int      ex = (int)(b >> 23);                    // biased exponent, 63..127
-    const uint32_t m  = (b & 0x7FFFFFu) | 0x800000u;       // 24-bit significand
-    const int      sh = ex - 110;                          // e*2^40 = m * 2^sh
-    uint64_t q;
-    if (sh >= 0) q = (uint64_t)m << sh;
-    else         q = (uint64_t)(m >> (sh < -31 ? 31 : -sh));
-    return q ? q : 1;
+    return (uint64_t)((b & 0x7FFFFFu) | 0x800000u) << ((b >> 23) - 87u);
 }
 
-// ceil(f * s) for a float 0 < f <= 1, exact, clamped to [1, s].
-__device__ inline uint64_t ceil_mul(float f, uint64_t s)
+// ceil(f * s) for a float 0 < f <= 1 and s < 2^100, exact, clamped to [1, s].
+__device__ inline u128 ceil_mul(float f, u128 s)
 {
     if (!(f > 0.0f)) return 1;
     if (f >= 1.0f) return s;
@@ -67,27 +68,34 @@ __device__ inline uint64_t ceil_mul(float f, uint64_t s)
     uint64_t m = b & 0x7FFFFFu;
     if (ex == 0) ex = 1; else m |= 0x800000u;
     const int sh = 150 - ex;                                // f = m * 2^-sh, sh >= 24
-    uint64_t r;
-    if (sh >= 96) r = 1;
-    else {
-        // 128-bit (hi:lo) = m*s + 2^sh - 1, then >> sh
-        uint64_t lo = m * s;
-        uint64_t hi = __umul64hi(m, s);
-        uint64_t add_lo = (sh < 64) ? ((1ull << sh) - 1) : ~0ull;
-        uint64_t add_hi = (sh < 64) ? 0ull : ((1ull << (sh - 64)) - 1);
-        uint64_t lo2 = lo + add_lo;
-        hi += add_hi + (lo2 < lo ? 1 : 0);
-        r = (sh < 64) ? ((lo2 >> sh) | (hi << (64 - sh))) : (hi >> (sh - 64));
-    }
+    u128 r;
+    if (sh >= 126) r = 1;                                   // 0 < m*s < 2^124 < 2^sh
+    else r = ((u128)m * s + (((u128)1 << sh) - 1)) >> sh;
     if (r < 1) r = 1;
     if (r > s) r = s;
     return r;
 }
 
-// 64 random bits -> r in [1, S]
-__device__ __forceinline__ uint64_t r_from_bits(uint64_t u64, uint64_t S)
+// 64 random bits -> r in [1, S]: floor(u64 * S / 2^64) + 1
+__device__ __forceinline__ u128 r_from_bits(uint64_t u64, u128 S)
 {
-    return __umul64hi(u64, S) + 1;
+    const uint64_t s_lo = (uint64_t)S, s_hi = (uint64_t)(S >> 64);
+    return (u128)u64 * s_hi + __umul64hi(u64, s_lo) + 1;
+}
+
+// floor(a / d) for a < 2^96 and a 32-bit divisor, by 32-bit long division
+__device__ inline u128 div_u32(u128 a, uint32_t d)
+{
+    uint64_t rem = 0;
+    u128 q = 0;
+#pragma unroll
+    for (int i = 2; i >= 0; --i) {
+        const uint64_t cur = (rem << 32) | (uint32_t)(a >> (32 * i));
+        const uint64_t qi = cur / d;
+        rem = cur - qi * d;
+        q |= (u128)qi << (32 * i);
+    }
+    return q;
 }
 
 // order-preserving map float -> uint32 (for atomicMax on floats)
@@ -137,11 +145,14 @@ __device__ __forceinline__ uint32_t dpp0_u32(uint32_t v)
 template <int CTRL, int ROW_MASK, typename T>
 __device__ __forceinline__ T dpp0(T v)
 {
-    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit integers");
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8 || sizeof(T) == 16, "32-, 64- or 128-bit integers");
     if constexpr (sizeof(T) == 4) return (T)dpp0_u32<CTRL, ROW_MASK>((uint32_t)v);
-    else {
+    else if constexpr (sizeof(T) == 8) {
         const uint32_t lo = dpp0_u32<CTRL, ROW_MASK>((uint32_t)v), hi = dpp0_u32<CTRL, ROW_MASK>((uint32_t)((uint64_t)v >> 32));
         return (T)(((uint64_t)hi << 32) | lo);
+    } else {
+        const uint64_t lo = dpp0<CTRL, ROW_MASK>((uint64_t)v), hi = dpp0<CTRL, ROW_MASK>((uint64_t)((u128)v >> 64));
+        return (T)(((u128)hi << 64) | lo);
     }
 }
 
@@ -165,7 +176,8 @@ template <typename T>
 __device__ __forceinline__ T lane63(T v)
 {
     if constexpr (sizeof(T) == 4) return (T)lane63_u32((uint32_t)v);
-    else return (T)(((uint64_t)lane63_u32((uint32_t)((uint64_t)v >> 32)) << 32) | lane63_u32((uint32_t)v));
+    else if constexpr (sizeof(T) == 8) return (T)(((uint64_t)lane63_u32((uint32_t)((uint64_t)v >> 32)) << 32) | lane63_u32((uint32_t)v));
+    else return (T)(((u128)lane63((uint64_t)((u128)v >> 64)) << 64) | lane63((uint64_t)v));
 }
 
 // Sum over the wave, returned to every lane (wave-uniform).

@@ -35,10 +35,11 @@ namespace rs {
 constexpr int      kThreads   = 256;          // 4 waves, one per SIMD
 constexpr int      kWaves     = kThreads / kWave;
 constexpr int      kMaxParts  = 256;          // workgroups per row, at most
-constexpr int      kNB        = 512;          // bins per histogram: level 1 uses 258, deeper levels 128
+constexpr int      kNB        = 512;          // bins per histogram: level 1 uses 164, deeper levels 128
 constexpr int      kLevels    = 4;            // 10 + 7 + 7 + 7 bits
 constexpr int      kCap       = 1024;         // tokens of a boundary bin that are gathered
 constexpr uint64_t kSpinLimit = 200000000ull; // 2 s of the 100 MHz wall clock
+constexpr uint64_t kValid     = 1ull << 63;   // marks a written exchange word
 
 struct alignas(256) WsHeader {
     uint32_t ticket;      // next logical workgroup id of the running launch
@@ -50,16 +51,16 @@ struct alignas(256) WsHeader {
 // Per-row record.  Everything a call reads before writing it is zero when the
 // call starts: the call itself re-zeroes what it used before it ends.
 struct alignas(256) RowCtl {
-    uint32_t unused1;
-    uint32_t done;        // workgroups finished with this row
     uint32_t unused0;
+    uint32_t done;        // workgroups finished with this row
+    uint32_t unused1;
     uint32_t cursor;      // fill of cand[]
     uint32_t index_p1;    // sampled token + 1, once known
     uint32_t pad[3];
     uint32_t mx[kMaxParts];     // per workgroup: fkey(max x of its slice), 0 = not yet written
-    uint64_t A[kMaxParts];      // per workgroup: mass above the gathered bin, or kept weight
+    uint64_t A[2 * kMaxParts];  // per workgroup: a 124-bit mass as two words of 62 bits, each | kValid
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
-    uint64_t h[kLevels][kNB];   // cluster histograms, packed (see pack_value)
+    uint64_t h[kLevels][kNB];   // cluster histograms, packed (see kPackOne)
 };
 
 struct Params {
@@ -83,12 +84,11 @@ struct Params {
 #define RS_AGENT __HIP_MEMORY_SCOPE_AGENT
 
 // Everything workgroups exchange goes through relaxed device-scope atomics
-// (they act at the level all XCDs share); "my contributions are performed" is
-// a wait on the vector-memory counter, not a cache write-back.
+// (they act at the level all XCDs share).  No exchange uses an arrival
+// counter: completeness is visible in the data itself.
 template <typename T> __device__ __forceinline__ T a_load(const T *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, RS_AGENT); }
 template <typename T> __device__ __forceinline__ void a_store(T *p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, RS_AGENT); }
 template <typename T> __device__ __forceinline__ void a_add(T *p, T v) { __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, RS_AGENT); }
-template <typename T> __device__ __forceinline__ void a_max(T *p, T v) { __hip_atomic_fetch_max(p, v, __ATOMIC_RELAXED, RS_AGENT); }
 __device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Hides a register from the optimiser for one use, so that work derived from
@@ -102,57 +102,48 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v)
 
 // ---- radix digits and histogram packing ----------------------------------
 // The threshold is selected digit by digit on the bit pattern of e, largest e
-// first.  Level 1 looks at bits [30:21]: index = bits >> 21 runs from 252
-// (e = 2^-64) to 508 (e = 1), 4 bins per octave aligned with the octaves, so
-// every token of a bin has the same exponent.  Levels 2..4 take 7 more bits
-// each (shifts 14, 7, 0).  Histograms are stored by index (ascending in e);
-// the scan walks them by digit = top - index (descending in e).
-constexpr uint32_t kTop1 = 508u;                      // index of e = 1.0 at level 1
+// first.  Level 1 looks at bits [30:21]: index = bits >> 21 runs from 348
+// (e = 2^-40) to 511 (e just below 2), 4 bins per octave aligned with the
+// octaves, so every token of a bin has the same exponent (index >> 2).
+// Levels 2..4 take 7 more bits each (shifts 14, 7, 0).  Histograms are stored
+// by index (ascending in e); the scan walks them by digit = top - index.
+constexpr uint32_t kTop1 = 511u;                      // largest index at level 1
 constexpr uint32_t kTopN = 127u;                      // largest index of a deeper level
 __device__ __forceinline__ uint32_t level_shift(uint32_t level) { return 21u - 7u * (level - 1u); }   // level >= 2
 
-// A bin is one 64-bit word: count << 43 | sum of per-token values.  The value
-// of a token is its 23 fraction bits when its exponent is >= 110 (then q =
-// (2^23 + fraction) << (exponent - 110), exact), else q itself (< 2^23).
-// Counts stay below 2^21 and sums below 2^43 for any row of at most 2^20
-// tokens, so one atomic add carries both.
+// A bin is one 64-bit word: count << 43 | sum of the tokens' 23 fraction bits.
+// With the shared exponent ex the bin's exact mass is
+// (sum + count * 2^23) << (ex - 87).  Counts stay below 2^21 and sums below
+// 2^43 for any row of at most 2^20 tokens, so one atomic add carries both.
 constexpr uint64_t kPackOne  = 1ull << 43;
 constexpr uint64_t kPackMask = kPackOne - 1;
-__device__ __forceinline__ uint32_t pack_value(uint32_t b)
-{
-    uint32_t v = b & 0x7FFFFFu;
-    if (b < 0x37000000u)                               // e < 2^-17: q = floor(e * 2^40) fits 23 bits
-        v = max((uint32_t)(__uint_as_float(b) * 0x1p40f), 1u);
-    return v;
-}
 __device__ __forceinline__ uint32_t pack_count(uint64_t w) { return (uint32_t)(w >> 43); }
-// mass (sum of q) of a bin whose tokens have biased exponent ex
-__device__ __forceinline__ uint64_t pack_mass(uint64_t w, int ex)
+__device__ __forceinline__ u128 pack_mass(uint64_t w, uint32_t ex)
 {
-    const uint64_t sv = w & kPackMask;
-    return ex >= 110 ? ((sv + ((w >> 43) << 23)) << (ex - 110)) : sv;
+    return (u128)((w & kPackMask) + ((w >> 43) << 23)) << (ex - 87u);
 }
 
 struct Found {               // result of a histogram scan (uniform over the workgroup)
+    u128     mass_above;
     uint32_t bin;            // index of the first bin (largest e first) at which the kept set becomes sufficient
     uint32_t cnt_above;      // tokens in bins before it (plus the carried offset)
     uint32_t cnt_bin;        // tokens in it
-    uint64_t mass_above;
-    uint64_t mass_bin;
+    uint32_t pad;
 };
 
 struct Lds {
+    u128     q128[kWaves * 2];
+    u128     bc128[4];
+    u128     wj[kWaves][32];
+    u128     tj[32];
+    u128     D, P;
+    Found    found;
     uint64_t hm[kNB];        // this workgroup's histogram
     uint64_t g[kNB];         // the cluster's histogram
     uint64_t cand[kCap];
-    uint64_t u64[kWaves * 4];
-    uint32_t u32[kWaves * 4];
     uint64_t bc64[8];
+    uint32_t u32[kWaves * 4];
     uint32_t bc32[8];
-    uint64_t wj[kWaves][32];
-    uint64_t tj[32];
-    Found    found;
-    uint64_t D, P;
     uint32_t ctr;
     int      abort;
 };
@@ -169,28 +160,40 @@ __device__ __forceinline__ uint32_t block_max_u32(Lds &s, uint32_t v, int lane, 
     return r;
 }
 
-__device__ __forceinline__ uint64_t block_sum_u64(Lds &s, uint64_t v, int lane, int wave)
+__device__ __forceinline__ uint32_t block_sum_u32(Lds &s, uint32_t v, int lane, int wave)
 {
     v = wave_sum(v);
     __syncthreads();
-    if (lane == 0) s.u64[wave] = v;
+    if (lane == 0) s.u32[wave] = v;
     __syncthreads();
-    uint64_t r = 0;
+    uint32_t r = 0;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) r += s.u64[w];
+    for (int w = 0; w < kWaves; ++w) r += s.u32[w];
+    return r;
+}
+
+__device__ __forceinline__ u128 block_sum_u128(Lds &s, u128 v, int lane, int wave)
+{
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) s.q128[wave] = v;
+    __syncthreads();
+    u128 r = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) r += s.q128[w];
     return r;
 }
 
 // two sums at once
-__device__ __forceinline__ void block_sum2_u64(Lds &s, uint64_t &a, uint64_t &b, int lane, int wave)
+__device__ __forceinline__ void block_sum2_u128(Lds &s, u128 &a, u128 &b, int lane, int wave)
 {
     a = wave_sum(a); b = wave_sum(b);
     __syncthreads();
-    if (lane == 0) { s.u64[wave * 2] = a; s.u64[wave * 2 + 1] = b; }
+    if (lane == 0) { s.q128[wave * 2] = a; s.q128[wave * 2 + 1] = b; }
     __syncthreads();
     a = 0; b = 0;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) { a += s.u64[w * 2]; b += s.u64[w * 2 + 1]; }
+    for (int w = 0; w < kWaves; ++w) { a += s.q128[w * 2]; b += s.q128[w * 2 + 1]; }
 }
 
 // Bounded wait bookkeeping: thread 0 looks at the wall clock now and then; the
@@ -213,10 +216,10 @@ __device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)
 {
     for (int b = threadIdx.x; b < nb; b += kThreads) s.hm[b] = 0;
 }
-// one LDS atomic per token: count and value together
-__device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint32_t value)
+// one LDS atomic per token: count and fraction bits together
+__device__ __forceinline__ void lds_hist_add(Lds &s, uint32_t bin, uint32_t b)
 {
-    atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[bin]), (unsigned long long)(kPackOne | value));
+    atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[bin]), (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
 }
 
 // Re-zero this workgroup's share of a global histogram (the cluster splits the bins).
@@ -254,14 +257,8 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
             s.g[b] = w;
             c += pack_count(w);
         }
-        c = wave_sum(c);
         guard.tick(s, hdr);
-        __syncthreads();
-        if (lane == 0) s.u32[wave] = c;
-        __syncthreads();
-        uint32_t total = 0;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) total += s.u32[w];
+        const uint32_t total = block_sum_u32(s, c, lane, wave);
         if (total == expected) return true;
         if (s.abort) return false;
     }
@@ -271,52 +268,49 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
 // bin at which (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).
 // With `first` the total mass of the histogram is the row total D and P is
 // derived from it here.  Thread t owns digits 2t and 2t+1 (index = top -
-// digit); ex(index) is the exponent of a bin.
-template <typename ExFn>
-__device__ __forceinline__ Found hist_find(Lds &s, uint32_t top, uint32_t cnt0, uint64_t mass0, uint64_t top_k,
-                                           float top_p, bool first, int lane, int wave, ExFn ex)
+// digit); the exponent of level-1 bin idx is idx >> 2.
+__device__ __forceinline__ Found hist_find512(Lds &s, uint64_t top_k, float top_p, int lane, int wave)
 {
     constexpr int PER = kNB / kThreads;
     const int t = threadIdx.x;
-    uint32_t c[PER]; uint64_t m[PER];
-    uint32_t cs = 0; uint64_t ms = 0;
+    uint32_t c[PER]; u128 m[PER];
+    uint32_t cs = 0; u128 ms = 0;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        const int idx = (int)top - (t * PER + i);
-        const uint64_t w = idx >= 0 ? s.g[idx] : 0ull;
+        const uint32_t idx = kTop1 - (uint32_t)(t * PER + i);
+        const uint64_t w = s.g[idx];
         c[i] = pack_count(w);
-        m[i] = pack_mass(w, ex((uint32_t)idx));
+        m[i] = w ? pack_mass(w, idx >> 2) : (u128)0;       // empty bins below 2^-40 have no valid exponent
         cs += c[i]; ms += m[i];
     }
     // inclusive scan over threads
-    const uint64_t mi = wave_inclusive_scan(ms);
+    const u128 mi = wave_inclusive_scan(ms);
     const uint32_t ci = wave_inclusive_scan(cs);
     __syncthreads();
-    if (lane == kWave - 1) { s.u64[wave] = mi; s.u32[wave] = ci; }
+    if (lane == kWave - 1) { s.q128[wave] = mi; s.u32[wave] = ci; }
     __syncthreads();
-    uint64_t moff = 0, mtot = 0;
+    u128 moff = 0, mtot = 0;
     uint32_t coff = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-        if (w < wave) { moff += s.u64[w]; coff += s.u32[w]; }
-        mtot += s.u64[w];
+        if (w < wave) { moff += s.q128[w]; coff += s.u32[w]; }
+        mtot += s.q128[w];
     }
-    if (first) {
-        if (t == 0) { s.D = mtot; s.P = ceil_mul(top_p, mtot); }
-        __syncthreads();
-    }
-    const uint64_t P = s.P;
-    uint64_t rcnt = (uint64_t)cnt0 + coff + ci - cs;     // count before my first bin
-    uint64_t rm = mass0 + moff + mi - ms;                // mass before my first bin
+    if (t == 0) { s.D = mtot; s.P = ceil_mul(top_p, mtot); }
+    __syncthreads();
+    const u128 P = s.P;
+    uint64_t rcnt = (uint64_t)coff + ci - cs;            // count before my first bin
+    u128 rm = moff + mi - ms;                            // mass before my first bin
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const bool before = rcnt >= top_k || rm >= P;
-        const uint64_t nc = rcnt + c[i], nm = rm + m[i];
+        const uint64_t nc = rcnt + c[i];
+        const u128 nm = rm + m[i];
         const bool after = nc >= top_k || nm >= P;
         if (!before && after) {
-            s.found.bin = top - (uint32_t)(t * PER + i);
+            s.found.bin = kTop1 - (uint32_t)(t * PER + i);
             s.found.cnt_above = (uint32_t)rcnt; s.found.cnt_bin = c[i];
-            s.found.mass_above = rm; s.found.mass_bin = m[i];
+            s.found.mass_above = rm;
         }
         rcnt = nc; rm = nm;
     }
@@ -326,28 +320,29 @@ __device__ __forceinline__ Found hist_find(Lds &s, uint32_t top, uint32_t cnt0, 
 
 // The same for a 128-bin level (all tokens share the exponent ex): one wave,
 // lane l owns indices 127-2l and 126-2l, no LDS exchange inside the scan.
-__device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint32_t cnt0, uint64_t mass0,
-                                              uint64_t top_k, int ex, int lane, int wave)
+__device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint32_t cnt0, u128 mass0,
+                                              uint64_t top_k, uint32_t ex, int lane, int wave)
 {
     if (wave == 0) {
         const uint64_t w0 = arr[127 - 2 * lane], w1 = arr[126 - 2 * lane];
         const uint32_t c0 = pack_count(w0), c1 = pack_count(w1);
-        const uint64_t m0 = pack_mass(w0, ex), m1 = pack_mass(w1, ex);
+        const u128 m0 = pack_mass(w0, ex), m1 = pack_mass(w1, ex);
         const uint32_t cs = c0 + c1;
-        const uint64_t ms = m0 + m1;
-        const uint64_t mi = wave_inclusive_scan(ms);
+        const u128 ms = m0 + m1;
+        const u128 mi = wave_inclusive_scan(ms);
         const uint32_t ci = wave_inclusive_scan(cs);
-        const uint64_t P = s.P;
-        const uint64_t r0 = (uint64_t)cnt0 + ci - cs, q0 = mass0 + mi - ms;      // before my first bin
-        const uint64_t r1 = r0 + c0, q1 = q0 + m0;                               // before my second bin
-        const uint64_t r2 = r1 + c1, q2 = q1 + m1;
+        const u128 P = s.P;
+        const uint64_t r0 = (uint64_t)cnt0 + ci - cs;      // before my first bin
+        const u128 q0 = mass0 + mi - ms;
+        const uint64_t r1 = r0 + c0, r2 = r1 + c1;         // before my second bin, after it
+        const u128 q1 = q0 + m0, q2 = q1 + m1;
         const bool s0 = r0 >= top_k || q0 >= P, s1 = r1 >= top_k || q1 >= P, s2 = r2 >= top_k || q2 >= P;
         if (!s0 && s1) {
             s.found.bin = 127u - 2u * (uint32_t)lane;
-            s.found.cnt_above = (uint32_t)r0; s.found.cnt_bin = c0; s.found.mass_above = q0; s.found.mass_bin = m0;
+            s.found.cnt_above = (uint32_t)r0; s.found.cnt_bin = c0; s.found.mass_above = q0;
         } else if (!s1 && s2) {
             s.found.bin = 126u - 2u * (uint32_t)lane;
-            s.found.cnt_above = (uint32_t)r1; s.found.cnt_bin = c1; s.found.mass_above = q1; s.found.mass_bin = m1;
+            s.found.cnt_above = (uint32_t)r1; s.found.cnt_bin = c1; s.found.mass_above = q1;
         }
     }
     __syncthreads();
@@ -355,13 +350,27 @@ __device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint3
 }
 
 // Mass of this workgroup's own tokens in the bins above index `bin` (larger
-// e), from s.hm, summed over the workgroup.
-template <typename ExFn>
-__device__ __forceinline__ uint64_t local_mass_above(Lds &s, uint32_t bin, uint32_t top, int lane, int wave, ExFn ex)
+// e), from s.hm, summed over the workgroup.  level1: exponent = index >> 2,
+// else the shared exponent ex.
+__device__ __forceinline__ u128 local_mass_above(Lds &s, uint32_t bin, uint32_t top, bool level1, uint32_t ex, int lane, int wave)
 {
-    uint64_t a = 0;
-    for (uint32_t b = bin + 1 + threadIdx.x; b <= top; b += kThreads) a += pack_mass(s.hm[b], ex(b));
-    return block_sum_u64(s, a, lane, wave);
+    u128 a = 0;
+    for (uint32_t b = bin + 1 + threadIdx.x; b <= top; b += kThreads) {
+        const uint64_t w = s.hm[b];
+        if (w) a += pack_mass(w, level1 ? b >> 2 : ex);
+    }
+    return block_sum_u128(s, a, lane, wave);
+}
+
+// A 124-bit mass in two self-validating words (62 bits each | kValid).
+__device__ __forceinline__ void put_mass(uint64_t *slot, u128 v)
+{
+    a_store(&slot[0], (uint64_t)(((uint64_t)v & ((1ull << 62) - 1)) | kValid));
+    a_store(&slot[1], (uint64_t)((uint64_t)(v >> 62) | kValid));
+}
+__device__ __forceinline__ u128 get_mass(uint64_t w0, uint64_t w1)
+{
+    return ((u128)(w1 & ~kValid) << 62) | (w0 & ~kValid);
 }
 
 // Waves per SIMD the register allocation must leave room for: the resident
@@ -481,17 +490,18 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         kmax_row = kmax;
     }
     const float xmax = fkey_inv(kmax_row);
+    const float M = __builtin_floorf(xmax);
 
-    // ---- 2. e = exp2(x - max) in place; level-1 histogram ------------------
+    // ---- 2. e = 2^(x - M) in place; level-1 histogram ----------------------
 #pragma unroll
     for (int j = 0; j < R; ++j) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) eb[j * 4 + k] = exp2c_bits(__uint_as_float(eb[j * 4 + k]) - xmax);
+        for (int k = 0; k < 4; ++k) eb[j * 4 + k] = e_bits_of(__uint_as_float(eb[j * 4 + k]), M);
         if (j < nv) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const uint32_t b = eb[j * 4 + k];
-                lds_hist_add(s, b >> 21, pack_value(b));
+                lds_hist_add(s, b >> 21, b);
             }
         }
     }
@@ -506,13 +516,11 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     const uint64_t top_k = (uint64_t)p.top_k;
 
     // ---- 3. radix selection of the threshold -------------------------------
-    auto ex1 = [](uint32_t idx) -> int { return (int)(idx >> 2); };
-    Found f = hist_find(s, kTop1, 0u, 0ull, top_k, p.top_p, true, lane, wave, ex1);
-    const uint64_t D = s.D, P = s.P;
-    const int exb = (int)(f.bin >> 2);                   // exponent of every token still in play
-    auto exc = [exb](uint32_t) -> int { return exb; };
+    Found f = hist_find512(s, top_k, p.top_p, lane, wave);
+    const u128 D = s.D, P = s.P;
+    const uint32_t exb = f.bin >> 2;                     // exponent of every token still in play
     // my own tokens: mass in the bins above the boundary, count in the boundary bin
-    uint64_t amass = local_mass_above(s, f.bin, kTop1, lane, wave, ex1);
+    u128 amass = local_mass_above(s, f.bin, kTop1, true, 0u, lane, wave);
     uint32_t mycnt = pack_count(s.hm[f.bin]);
     // bit patterns of the tokens still undistinguished: [lo, lo + span]
     uint32_t lo = f.bin << 21;
@@ -531,14 +539,14 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t b = opaque(eb[j * 4 + k]);
-                    if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, pack_value(b));
+                    if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, b);
                 }
             }
         if (!hist_combine(s, p.hdr, G, rc->h[levels - 1], 128, expect, lane, wave)) return;
         // every workgroup has finished reading the level above: it published this level after that
         if (G > 1) zero_slice(rc->h[levels - 2], levels == 2 ? kNB : 128, part, G);
         f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
-        amass += local_mass_above(s, f.bin, kTopN, lane, wave, exc);
+        amass += local_mass_above(s, f.bin, kTopN, false, exb, lane, wave);
         mycnt = pack_count(s.hm[f.bin]);
         lo |= f.bin << dsh;
         span = (1u << dsh) - 1u;
@@ -547,17 +555,17 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
 
     // If the undistinguished tokens are few, gather them (bits and index) so
     // that every workgroup can finish alone.  Validity is in the data: a
-    // gathered entry is never 0, and A[] holds mass + 1.
+    // gathered entry is never 0, and the words of A[] carry kValid.
     const bool gather = f.cnt_bin <= (uint32_t)kCap;
     const uint32_t ncand = gather ? f.cnt_bin : 0u;
-    uint64_t a_mine = 0;                                 // thread t < G: A[t] of workgroup t
+    u128 a_mine = 0;                                     // thread t < G: mass above the bin in workgroup t
     if (gather) {
         __syncthreads();
         if (tid == 0) {
             s.ctr = 0;
             if (G > 1) {
                 s.bc32[2] = mycnt ? __hip_atomic_fetch_add(&rc->cursor, mycnt, __ATOMIC_RELAXED, RS_AGENT) : 0u;
-                a_store(&rc->A[part], amass + 1);
+                put_mass(&rc->A[2 * part], amass);
             }
         }
         __syncthreads();
@@ -577,6 +585,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                 }
             }
         if (G > 1) {
+            uint64_t w0 = 0, w1 = 0;
             SpinGuard guard;
             guard.start();
             for (;;) {
@@ -586,22 +595,19 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                     s.cand[i] = w;
                     valid += w != 0;
                 }
-                if ((uint32_t)tid < G) { a_mine = a_load(&rc->A[tid]); valid += a_mine != 0; }
-                valid = wave_sum(valid);
+                if ((uint32_t)tid < G) {
+                    w0 = a_load(&rc->A[2 * tid]); w1 = a_load(&rc->A[2 * tid + 1]);
+                    valid += (w0 & w1 & kValid) != 0;
+                }
                 guard.tick(s, p.hdr);
-                __syncthreads();
-                if (lane == 0) s.u32[wave] = valid;
-                __syncthreads();
-                uint32_t total = 0;
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w) total += s.u32[w];
+                const uint32_t total = block_sum_u32(s, valid, lane, wave);
                 if (total == ncand + G) break;
                 if (s.abort) return;
             }
-            a_mine -= (uint32_t)tid < G ? 1u : 0u;
+            if ((uint32_t)tid < G) a_mine = get_mass(w0, w1);
             // every workgroup wrote its entries after it had read the last histogram level
             zero_slice(rc->h[levels - 1], last_nb, part, G);
-        } else a_mine = tid == 0 ? amass : 0;
+        } else a_mine = tid == 0 ? amass : (u128)0;
         __syncthreads();
 
         // resolve the remaining digits on the gathered tokens, in LDS
@@ -611,7 +617,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             __syncthreads();
             for (uint32_t i = tid; i < ncand; i += kThreads) {
                 const uint32_t b = (uint32_t)(s.cand[i] >> 32);
-                if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, pack_value(b));
+                if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, b);
             }
             __syncthreads();
             f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
@@ -622,46 +628,48 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     // every digit is known: the threshold is the one value left in [lo, lo + span]
     const uint32_t thr = lo;
     const uint32_t n_gt = f.cnt_above, n_eq = f.cnt_bin;
-    const uint64_t Gm = f.mass_above;
+    const u128 Gm = f.mass_above;
 
     // ---- 5. tie weight, total S, target r (every workgroup, identically) ----
     if (tid == 0) {
-        const uint64_t q_thr = q_of_bits(thr);
-        uint64_t w_tie = q_thr;
-        uint64_t a = (P > Gm) ? (P - Gm) : 0;
-        uint64_t bk = ((uint32_t)p.top_k > n_gt) ? (q_thr * (uint64_t)((uint32_t)p.top_k - n_gt)) : 0;
-        if (n_eq > 1) { a /= n_eq; bk /= n_eq; }
-        if (a < w_tie) w_tie = a;
-        if (bk < w_tie) w_tie = bk;
-        if (w_tie == 0 && Gm == 0) w_tie = 1;
-        const uint64_t S = Gm + (uint64_t)n_eq * w_tie;
-        uint64_t r;
-        if (p.inj_u) r = ceil_mul(p.inj_u[row], S);
-        else r = r_from_bits(s.bc64[5], S);
-        s.bc64[1] = w_tie; s.bc64[2] = S; s.bc64[3] = r;
+        const uint64_t w_thr = w_of_bits(thr);
+        u128 a = (P > Gm) ? (P - Gm) : (u128)0;
+        u128 bk = ((uint32_t)p.top_k > n_gt) ? (u128)w_thr * ((uint32_t)p.top_k - n_gt) : (u128)0;
+        if (n_eq > 1) { a = div_u32(a, n_eq); bk = div_u32(bk, n_eq); }
+        u128 wt = w_thr;
+        if (a < wt) wt = a;
+        if (bk < wt) wt = bk;
+        if (wt == 0 && Gm == 0) wt = 1;
+        const uint64_t w_tie = (uint64_t)wt;
+        const u128 S = Gm + (u128)n_eq * w_tie;
+        const u128 r = p.inj_u ? ceil_mul(p.inj_u[row], S) : r_from_bits(s.bc64[5], S);
+        s.bc64[1] = w_tie; s.bc128[0] = r;
         if (p.diag && part == 0) {
             rs_row_diag *d = p.diag + row;
-            d->xmax = xmax; d->emin_bits = 0; d->D = D; d->P = P;
-            d->left_bits = thr; d->thr_bits = thr; d->rounds = levels;
-            d->n_gt = n_gt; d->n_eq = n_eq; d->G = Gm; d->w_tie = w_tie; d->S = S; d->r = r;
+            d->xmax = xmax; d->emin_bits = 0;
+            d->D[0] = (uint64_t)D; d->D[1] = (uint64_t)(D >> 64); d->P[0] = (uint64_t)P; d->P[1] = (uint64_t)(P >> 64);
+            d->left_bits = thr; d->thr_bits = thr; d->rounds = levels; d->n_gt = n_gt; d->n_eq = n_eq;
+            d->G[0] = (uint64_t)Gm; d->G[1] = (uint64_t)(Gm >> 64); d->w_tie = w_tie;
+            d->S[0] = (uint64_t)S; d->S[1] = (uint64_t)(S >> 64); d->r[0] = (uint64_t)r; d->r[1] = (uint64_t)(r >> 64);
         }
     }
     __syncthreads();
-    const uint64_t w_tie = s.bc64[1], r = s.bc64[3];
+    const uint64_t w_tie = s.bc64[1];
+    const u128 r = s.bc128[0];
 
     // ---- 6. inverse CDF: which workgroup, which float4 slot, which thread ---
     auto weight = [&](uint32_t b) -> uint64_t {
         b = opaque(b);
-        return (b > thr) ? q_of_bits(b) : (b == thr ? w_tie : 0);
+        return (b > thr) ? w_of_bits(b) : (b == thr ? w_tie : 0);
     };
-    auto slot_weight = [&](int j) -> uint64_t {         // weight of float4 slot j of this thread
-        return weight(eb[j * 4]) + weight(eb[j * 4 + 1]) + weight(eb[j * 4 + 2]) + weight(eb[j * 4 + 3]);
+    auto slot_weight = [&](int j) -> u128 {             // weight of float4 slot j of this thread
+        return (u128)weight(eb[j * 4]) + weight(eb[j * 4 + 1]) + weight(eb[j * 4 + 2]) + weight(eb[j * 4 + 3]);
     };
-    uint64_t before = 0, wblock = 0;
+    u128 before = 0, wblock = 0;
     if (gather) {
-        // kept weight of workgroup g = A[g] + weights of its gathered tokens
+        // kept weight of workgroup g = mass above the bin in g + weights of its gathered tokens
         const uint32_t shift = 2 + 8 + (uint32_t)__builtin_ctz((unsigned)R);   // token index -> workgroup
-        uint64_t cb = 0, cm = 0;
+        u128 cb = 0, cm = 0;
         for (uint32_t i = tid; i < ncand; i += kThreads) {
             const uint64_t cd = s.cand[i];
             const uint32_t g = ((uint32_t)cd) >> shift;
@@ -671,73 +679,70 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         }
         if ((uint32_t)tid < part) cb += a_mine;
         if ((uint32_t)tid == part) cm += a_mine;
-        block_sum2_u64(s, cb, cm, lane, wave);
+        block_sum2_u128(s, cb, cm, lane, wave);
         before = cb; wblock = cm;
     } else {
-        uint64_t wloc = 0;
+        u128 wloc = 0;
 #pragma unroll
         for (int j = 0; j < R; ++j)
             if (j < nv) wloc += slot_weight(j);
-        wblock = block_sum_u64(s, wloc, lane, wave);
+        wblock = block_sum_u128(s, wloc, lane, wave);
         if (G > 1) {
-            // exchange the kept weights through A[] (weight + 1, never 0)
-            if (tid == 0) a_store(&rc->A[part], wblock + 1);
-            uint64_t v = 0;
+            // exchange the kept weights through A[]
+            if (tid == 0) put_mass(&rc->A[2 * part], wblock);
+            uint64_t w0 = 0, w1 = 0;
             SpinGuard guard;
             guard.start();
             for (;;) {
                 uint32_t valid = 0;
-                if ((uint32_t)tid < G) { v = a_load(&rc->A[tid]); valid = v != 0; }
-                valid = wave_sum(valid);
+                if ((uint32_t)tid < G) {
+                    w0 = a_load(&rc->A[2 * tid]); w1 = a_load(&rc->A[2 * tid + 1]);
+                    valid = (w0 & w1 & kValid) != 0;
+                }
                 guard.tick(s, p.hdr);
-                __syncthreads();
-                if (lane == 0) s.u32[wave] = valid;
-                __syncthreads();
-                uint32_t total = 0;
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w) total += s.u32[w];
+                const uint32_t total = block_sum_u32(s, valid, lane, wave);
                 if (total == G) break;
                 if (s.abort) return;
             }
             zero_slice(rc->h[levels - 1], last_nb, part, G);
-            before = block_sum_u64(s, (uint32_t)tid < part ? v - 1 : 0ull, lane, wave);
+            before = block_sum_u128(s, (uint32_t)tid < part ? get_mass(w0, w1) : (u128)0, lane, wave);
         }
     }
     const bool owner = before < r && r <= before + wblock;   // block-uniform
 
     if (owner) {
-        uint64_t rl = r - before;                        // 1 <= rl <= wblock
+        u128 rl = r - before;                            // 1 <= rl <= wblock
         // totals per float4 slot j over the workgroup
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            const uint64_t t = wave_sum(j < nv ? slot_weight(j) : 0ull);
+            const u128 t = wave_sum(j < nv ? slot_weight(j) : (u128)0);
             if (lane == 0) s.wj[wave][j] = t;
         }
         __syncthreads();
-        if (tid < R) { uint64_t t = 0; for (int w = 0; w < kWaves; ++w) t += s.wj[w][tid]; s.tj[tid] = t; }
+        if (tid < R) { u128 t = 0; for (int w = 0; w < kWaves; ++w) t += s.wj[w][tid]; s.tj[tid] = t; }
         __syncthreads();
         int jstar = 0;
-        for (int j = 0; j < R - 1; ++j) { const uint64_t t = s.tj[j]; if (rl > t) { rl -= t; jstar = j + 1; } else break; }
+        for (int j = 0; j < R - 1; ++j) { const u128 t = s.tj[j]; if (rl > t) { rl -= t; jstar = j + 1; } else break; }
         // rl <= wblock = sum of tj, so rl now lies inside slot jstar
         uint32_t e4[4] = {0, 0, 0, 0};
         bool have = false;
 #pragma unroll
         for (int j = 0; j < R; ++j)
             if (j == jstar) { have = j < nv; e4[0] = eb[j * 4]; e4[1] = eb[j * 4 + 1]; e4[2] = eb[j * 4 + 2]; e4[3] = eb[j * 4 + 3]; }
-        const uint64_t w0 = have ? weight(e4[0]) : 0, w1 = have ? weight(e4[1]) : 0;
-        const uint64_t w2 = have ? weight(e4[2]) : 0, w3 = have ? weight(e4[3]) : 0;
-        const uint64_t mine = w0 + w1 + w2 + w3;
+        const u128 w0 = have ? weight(e4[0]) : 0, w1 = have ? weight(e4[1]) : 0;
+        const u128 w2 = have ? weight(e4[2]) : 0, w3 = have ? weight(e4[3]) : 0;
+        const u128 mine = w0 + w1 + w2 + w3;
         // inclusive scan over the 256 threads of slot jstar
-        uint64_t inc = wave_inclusive_scan(mine);
+        u128 inc = wave_inclusive_scan(mine);
         __syncthreads();
-        if (lane == kWave - 1) s.u64[wave] = inc;
+        if (lane == kWave - 1) s.q128[wave] = inc;
         __syncthreads();
-        uint64_t woff = 0;
-        for (int w = 0; w < wave; ++w) woff += s.u64[w];
+        u128 woff = 0;
+        for (int w = 0; w < wave; ++w) woff += s.q128[w];
         inc += woff;
-        const uint64_t exc_ = inc - mine;
+        const u128 exc_ = inc - mine;
         if (exc_ < rl && rl <= inc) {                     // exactly one thread
-            const uint64_t rr = rl - exc_;                // 1 <= rr <= mine
+            const u128 rr = rl - exc_;                    // 1 <= rr <= mine
             const int kk = (rr <= w0) ? 0 : (rr <= w0 + w1) ? 1 : (rr <= w0 + w1 + w2) ? 2 : 3;
             const int32_t idx = (int32_t)((base4 + (uint32_t)jstar * kThreads) * 4 + (uint32_t)kk);
             p.out[row] = idx;
@@ -790,7 +795,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         if (s.bc32[0] == G - 1) {
             // last workgroup out of this row: nobody reads the record any more
             for (uint32_t i = tid; i < ncand; i += kThreads) a_store(&rc->cand[i], (uint64_t)0);
-            if ((uint32_t)tid < G) a_store(&rc->A[tid], (uint64_t)0);
+            if ((uint32_t)tid < G) { a_store(&rc->A[2 * tid], (uint64_t)0); a_store(&rc->A[2 * tid + 1], (uint64_t)0); }
             if (tid == 0) { a_store(&rc->done, 0u); a_store(&rc->cursor, 0u); a_store(&rc->index_p1, 0u); }
         }
     }

@@ -9,11 +9,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(ROOT, "rapid_sampling_amd", "librapid_sampling_hip.so")
 HEADER = os.path.join(ROOT, "include", "rapid_sampling.h")
 
+# 128-bit quantities are (low, high) uint64 pairs
 DIAG_DTYPE = np.dtype([
-    ("xmax", "<f4"), ("emin_bits", "<u4"), ("D", "<u8"), ("P", "<u8"),
+    ("xmax", "<f4"), ("emin_bits", "<u4"), ("D", "<u8", (2,)), ("P", "<u8", (2,)),
     ("left_bits", "<u4"), ("thr_bits", "<u4"), ("rounds", "<u4"), ("n_gt", "<u4"),
-    ("n_eq", "<u4"), ("index", "<i4"), ("G", "<u8"), ("w_tie", "<u8"),
-    ("S", "<u8"), ("r", "<u8"),
+    ("n_eq", "<u4"), ("index", "<i4"), ("G", "<u8", (2,)), ("w_tie", "<u8"),
+    ("S", "<u8", (2,)), ("r", "<u8", (2,)),
 ])
 
 _lib = None

@@ -45,10 +45,12 @@ def test_error_strings_cover_every_code():
 def test_diag_struct_layout_matches_header():
     text = open(capi.HEADER).read()
     body = re.search(r"typedef struct rs_row_diag \{(.*?)\} rs_row_diag;", text, flags=re.S).group(1)
-    fields = re.findall(r"\b(float|uint32_t|int32_t|uint64_t)\s+(\w+);", body)
+    fields = re.findall(r"\b(float|uint32_t|int32_t|uint64_t)\s+(\w+)(?:\[(\d+)\])?;", body)
     assert [f[1] for f in fields] == list(capi.DIAG_DTYPE.names)
     size = {"float": 4, "uint32_t": 4, "int32_t": 4, "uint64_t": 8}
-    assert sum(size[t] for t, _ in fields) == capi.DIAG_DTYPE.itemsize == 80
+    assert sum(size[t] * int(n or 1) for t, _, n in fields) == capi.DIAG_DTYPE.itemsize == 120
+    from oracle import oracle as O
+    assert O.DIAG_DTYPE == capi.DIAG_DTYPE
 
 
 @pytest.mark.parametrize("temp,k,p,V,exp_k,exp_p", [

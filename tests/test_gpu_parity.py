@@ -227,7 +227,7 @@ def test_chi_square_one_million_draws(torch_cuda, oracle):
     rc, c, k, p = capi.normalize(1.0, 40, 0.9, V, B, 1)
     d = oracle.sample_row(row[0], c, k, p, u=0.5, want_e=True)
     e, thr = d["e_bits"], d["thr_bits"]
-    w = np.where(e > thr, oracle.q_of(e.view(np.float32)).astype(np.float64), 0.0)
+    w = np.where(e > thr, oracle.w_of(e).astype(np.float64), 0.0)
     w[e == thr] = float(d["w_tie"])
     assert abs(w.sum() - float(d["S"])) <= 1e-6 * float(d["S"])
     lg = torch.from_numpy(np.repeat(row, B, axis=0)).cuda()

@@ -48,49 +48,69 @@ def test_scale_order_of_operations(oracle):
     assert L.rs_oracle_scale(float("nan"), 0.0, 1, 2.0) == 0.0
 
 
-# ------------------------------------------------------------------ exp2c
-def test_exp2c_accuracy_monotone_and_anchors(oracle):
-    d = -np.abs(np.random.default_rng(1).normal(size=20000) * 12).astype(np.float32)
-    d = np.sort(np.concatenate([d, -np.arange(0, 66, dtype=np.float32), F32([-1e-8, -1e-20, -0.5, -63.999])]))
-    e = oracle.exp2c(d)
-    ref = np.exp2(d.astype(np.float64))
-    live = d >= -64
-    rel = np.abs(e[live].astype(np.float64) - ref[live]) / ref[live]
-    assert rel.max() < 2.0 * 2.0 ** -23, rel.max()        # within 2 ulp, as the reference's exp2f
-    assert np.all(np.diff(e) >= 0)                         # monotone in d
-    assert oracle.exp2c(F32([0.0]))[0] == 1.0              # e_max is exactly 1
-    for k in range(0, 65):
-        assert oracle.exp2c(F32([-k]))[0] == F32(2.0 ** -k)  # exact powers of two
-    assert oracle.exp2c(F32([-64.5]))[0] == F32(2.0 ** -64)   # argument clamped at -64
-    assert oracle.exp2c(F32([-1e30]))[0] == F32(2.0 ** -64)
-    assert oracle.exp2c(F32([-np.inf]))[0] == F32(2.0 ** -64)
+# ------------------------------------------------------------------ e = 2^(x - M)
+def test_e_bits_accuracy_monotone_and_anchors(oracle):
+    rng = np.random.default_rng(1)
+    for M in (0.0, 3.0, -7.0, 1000.0):
+        x = np.sort((M + 1 - np.abs(rng.normal(size=6000) * 9)).astype(np.float32))
+        x = x[x < M + 1]                                    # floor(max) = M means every x < M + 1
+        b = oracle.e_bits(x, M)
+        e = b.view(np.float32).astype(np.float64)
+        ref = np.exp2(x.astype(np.float64) - M)
+        live = ref >= 2.0 ** -40
+        rel = np.abs(e[live] - ref[live]) / ref[live]
+        assert rel.max() < 2.0 * 2.0 ** -23, rel.max()     # within 2 ulp, as the reference's exp2f
+        assert np.all(e[~live] == 2.0 ** -40)              # clamped from below
+        assert np.all(np.diff(b.astype(np.int64)) >= 0)    # monotone in x
+        assert b.max() < 0x40000000                        # e < 2
+    assert oracle.e_bits(F32([5.0]), 5.0)[0] == bits(F32(1.0))[()]
+    for k in range(0, 41):
+        assert oracle.e_bits(F32([-k]), 0.0)[0] == bits(F32(2.0 ** -k))[()]     # exact powers of two
+    assert oracle.e_bits(F32([-40.5, -1e30, -3.4e38]), 0.0).tolist() == [0x2B800000] * 3
 
 
-def test_exp2c_monotone_across_every_octave_boundary(oracle):
-    """poly(f -> 1) must not exceed 2 * poly(0): check the floats on both sides of each integer."""
-    for k in range(1, 64):
-        lo = np.nextafter(F32(-k), F32(-np.inf))
-        hi = np.nextafter(F32(-k), F32(0))
-        e = oracle.exp2c(np.array([lo, F32(-k), hi], dtype=np.float32))
-        assert e[0] <= e[1] <= e[2]
+def test_e_significand_does_not_depend_on_the_maximum(oracle):
+    """Shifting M by an integer only moves the exponent field: a slice can be worked with its own
+    maximum and re-based later."""
+    x = (np.random.default_rng(2).normal(size=4000) * 6).astype(np.float32)
+    x = x[x < 20]
+    b0 = oracle.e_bits(x, 20.0)
+    for d in (1, 2, 7, 19):
+        b1 = oracle.e_bits(x, 20.0 + d)
+        rebased = np.maximum(b0.astype(np.int64) - (d << 23), 0x2B800000)
+        keep = (b0 > 0x2B800000)
+        assert np.array_equal(b1[keep].astype(np.int64), rebased[keep])
+        assert np.all(b1[~keep] == 0x2B800000)
 
 
-# ------------------------------------------------------------------ fixed point
-def test_q_is_floor_e_times_2_pow_40(oracle):
+def test_e_monotone_across_every_octave_boundary(oracle):
+    """poly(f -> 1) stays below 2 * poly(0): the floats on both sides of each integer are ordered."""
+    for k in range(-39, 1):
+        lo = np.nextafter(F32(k), F32(-np.inf))
+        hi = np.nextafter(F32(k), F32(np.inf))
+        b = oracle.e_bits(np.array([lo, F32(k), hi], dtype=np.float32), 0.0)
+        assert b[0] <= b[1] <= b[2]
+    tiny = oracle.e_bits(F32([-1e-10]), -1.0)[0]           # f rounds to 1.0: poly(1) < 2
+    assert tiny < 0x40000000 and tiny >= bits(F32(1.999))[()]
+
+
+# ------------------------------------------------------------------ exact weights
+def test_w_is_e_times_2_pow_63(oracle):
     rng = np.random.default_rng(2)
-    e = np.concatenate([oracle.exp2c(-np.abs(rng.normal(size=3000) * 15).astype(np.float32)),
-                        F32([1.0, 2.0 ** -40, 2.0 ** -41, 2.0 ** -64, 2.0 ** -17, 0.75])])
-    q = oracle.q_of(e)
-    for ei, qi in zip(e, q):
-        exact = math.floor(Fraction(float(ei)) * 2 ** 40)
-        assert int(qi) == max(1, exact)
+    b = np.concatenate([oracle.e_bits((-np.abs(rng.normal(size=3000) * 15)).astype(np.float32), 0.0),
+                        bits(F32([1.0, 1.5, 1.9999999, 2.0 ** -40, 2.0 ** -17, 0.75]))])
+    w = oracle.w_of(b)
+    for bi, wi in zip(b, w):
+        exact = Fraction(float(np.uint32(bi).view(np.float32))) * 2 ** 63
+        assert exact.denominator == 1 and int(wi) == exact.numerator == oracle.lib().rs_oracle_w(int(bi))
+    assert int(w.min()) == 2 ** 23 and int(w.max()) < 2 ** 64
 
 
 @settings(max_examples=300, deadline=None)
-@given(st.floats(min_value=0.0, max_value=1.0, width=32), st.integers(min_value=1, max_value=2 ** 62))
+@given(st.floats(min_value=0.0, max_value=1.0, width=32), st.integers(min_value=1, max_value=2 ** 84))
 def test_ceil_mul_exact(f, s):
     from oracle import oracle as O
-    got = O.lib().rs_oracle_ceil_mul(f, s)
+    got = O.ceil_mul(f, s)
     if f <= 0.0:
         assert got == 1
     else:
@@ -99,10 +119,10 @@ def test_ceil_mul_exact(f, s):
 
 
 @settings(max_examples=200, deadline=None)
-@given(st.integers(min_value=0, max_value=2 ** 64 - 1), st.integers(min_value=1, max_value=2 ** 62))
+@given(st.integers(min_value=0, max_value=2 ** 64 - 1), st.integers(min_value=1, max_value=2 ** 84))
 def test_r_from_bits_exact(u, s):
     from oracle import oracle as O
-    assert O.lib().rs_oracle_r_from_bits(u, s) == (u * s) // 2 ** 64 + 1
+    assert O.r_from_bits(u, s) == (u * s) // 2 ** 64 + 1
 
 
 # ------------------------------------------------------------------ Philox
@@ -157,10 +177,11 @@ def brute_force_row(logits, c, top_k, top_p, u=None, u64=None, pen=None):
     x = [L.rs_oracle_scale(float(logits[i]), float(pen[i]) if pen is not None else 0.0, pen is not None, c)
          for i in range(V)]
     xmax = max(x)
-    e = O.exp2c(np.array([F32(F32(xi) - F32(xmax)) for xi in x], dtype=np.float32))
-    eb = e.view(np.uint32)
-    q = [max(1, math.floor(Fraction(float(v)) * 2 ** 40)) for v in e]
-    D = sum(q)
+    eb = O.e_bits(np.array(x, dtype=np.float32), math.floor(xmax))
+    w = [Fraction(float(np.uint32(b).view(np.float32))) * 2 ** 63 for b in eb]
+    assert all(v.denominator == 1 for v in w)
+    w = [v.numerator for v in w]
+    D = sum(w)
     P = min(max(math.ceil(Fraction(float(F32(top_p))) * D), 1), D)
     order = sorted(set(int(b) for b in eb), reverse=True)
     cnt = mass = 0
@@ -168,15 +189,15 @@ def brute_force_row(logits, c, top_k, top_p, u=None, u64=None, pen=None):
     for val in order:
         members = [i for i in range(V) if eb[i] == val]
         cnt += len(members)
-        mass += sum(q[i] for i in members)
+        mass += sum(w[i] for i in members)
         if cnt >= top_k or mass >= P:
             thr = val
             break
     n_gt = sum(1 for b in eb if b > thr)
     n_eq = sum(1 for b in eb if b == thr)
-    G = sum(q[i] for i in range(V) if eb[i] > thr)
-    q_thr = max(1, math.floor(Fraction(float(np.uint32(thr).view(np.float32))) * 2 ** 40))
-    w_tie = min(q_thr, (P - G) // n_eq if P > G else 0, (q_thr * (top_k - n_gt)) // n_eq if top_k > n_gt else 0)
+    G = sum(w[i] for i in range(V) if eb[i] > thr)
+    w_thr = (Fraction(float(np.uint32(thr).view(np.float32))) * 2 ** 63).numerator
+    w_tie = min(w_thr, (P - G) // n_eq if P > G else 0, (w_thr * (top_k - n_gt)) // n_eq if top_k > n_gt else 0)
     if w_tie == 0 and G == 0:
         w_tie = 1
     S = G + n_eq * w_tie
@@ -186,7 +207,7 @@ def brute_force_row(logits, c, top_k, top_p, u=None, u64=None, pen=None):
         r = (u64 * S) // 2 ** 64 + 1
     cdf, idx = 0, -1
     for i in range(V):
-        cdf += q[i] if eb[i] > thr else (w_tie if eb[i] == thr else 0)
+        cdf += w[i] if eb[i] > thr else (w_tie if eb[i] == thr else 0)
         if cdf >= r:
             idx = i
             break
@@ -276,14 +297,14 @@ def test_invariants_on_random_rows(oracle):
         c, kk, pp = oracle.normalize(float(rng.uniform(0.3, 3)), k, p, V)
         d = oracle.sample_row(lg, c, kk, pp, u=float(F32(1.0 - rng.random())), want_e=True)
         e, thr = d["e_bits"], d["thr_bits"]
-        q = oracle.q_of(e.view(np.float32)).astype(object)
+        q = oracle.w_of(e).astype(object)
         assert d["n_gt"] < kk and sum(q[e > thr]) < d["P"]                 # the set above thr is insufficient
         assert d["n_gt"] + d["n_eq"] >= kk or sum(q[e >= thr]) >= d["P"]    # the set at thr is sufficient
-        assert 0 <= d["w_tie"] <= int(oracle.q_of(np.array([thr], dtype=np.uint32).view(np.float32))[0])
+        assert 0 <= d["w_tie"] <= int(oracle.w_of(np.array([thr], dtype=np.uint32))[0])
         assert d["S"] <= max(d["P"], d["G"] + d["n_eq"]) and 1 <= d["r"] <= d["S"]
         assert d["n_gt"] * 1 + 0 <= kk and e[d["index"]] >= thr           # never a dropped token
         if d["n_eq"] * d["w_tie"] > 0:
-            assert d["n_gt"] + d["n_eq"] * d["w_tie"] / int(oracle.q_of(np.array([thr], dtype=np.uint32).view(np.float32))[0]) <= kk + 1e-9
+            assert d["n_gt"] + d["n_eq"] * d["w_tie"] / int(oracle.w_of(np.array([thr], dtype=np.uint32))[0]) <= kk + 1e-9
 
 
 # ------------------------------------------------------------------ penalties
@@ -325,7 +346,7 @@ def test_oracle_pick_chi_square(oracle):
     c, kk, pp = oracle.normalize(1.0, 12, 0.95, V)
     d = oracle.sample_row(lg, c, kk, pp, u=0.5, want_e=True)
     e, thr = d["e_bits"], d["thr_bits"]
-    w = np.where(e > thr, oracle.q_of(e.view(np.float32)).astype(np.float64), 0.0)
+    w = np.where(e > thr, oracle.w_of(e).astype(np.float64), 0.0)
     w[e == thr] = float(d["w_tie"])
     n = 100000
     logits2d = np.repeat(lg[None, :], n, axis=0)

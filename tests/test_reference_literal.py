@@ -39,7 +39,7 @@ def test_kept_set_matches_literal_reference(oracle, name, lg, temp, k, p, varian
         assert diff == 0, (name, diff)
     assert diff <= max(2, n // 2000), (name, diff, n)
     # probabilities agree to a few ulp: e / D  vs  exp2f(x - max) / denom
-    pc = can["e_bits"].view(np.float32).astype(np.float64) * 2.0 ** 40 / float(can["D"])
+    pc = can["e_bits"].view(np.float32).astype(np.float64) * 2.0 ** 63 / float(can["D"])
     live = lit["probs"] > 1e-30
     rel = np.abs(pc[live] - lit["probs"][live].astype(np.float64)) / lit["probs"][live]
     assert rel.max() < 2e-5, (name, rel.max())
@@ -56,7 +56,7 @@ def test_literal_tie_compensation_matches_integer_form(oracle):
         can = oracle.sample_row(lg, c, kk, pp, u=0.5)
         lit = oracle.literal_row(lg, c, kk, pp, 0.5, 0.5, variant=0)
         assert can["n_eq"] == lit["n_eq"] and can["n_gt"] == lit["n_gt"]
-        q_thr = int(oracle.q_of(np.array([can["thr_bits"]], dtype=np.uint32).view(np.float32))[0])
+        q_thr = int(oracle.w_of(np.array([can["thr_bits"]], dtype=np.uint32))[0])
         assert abs(can["w_tie"] / q_thr - lit["comp"]) < 1e-4
 
 
@@ -67,7 +67,7 @@ def test_literal_and_canonical_picks_share_a_distribution(oracle):
     c, kk, pp = oracle.normalize(1.0, 20, 0.9, V)
     can = oracle.sample_row(lg, c, kk, pp, u=0.5, want_e=True)
     e, thr = can["e_bits"], can["thr_bits"]
-    w = np.where(e > thr, oracle.q_of(e.view(np.float32)).astype(np.float64), 0.0)
+    w = np.where(e > thr, oracle.w_of(e).astype(np.float64), 0.0)
     w[e == thr] = float(can["w_tie"])
     rng = np.random.default_rng(22)
     n = 20000
