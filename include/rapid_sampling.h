@@ -48,7 +48,8 @@ typedef struct rs_row_diag {
     uint64_t P[2];        /* ceil(top_p * D)                                  */
     uint32_t left_bits;   /* same as thr_bits                                 */
     uint32_t thr_bits;    /* bit pattern of the smallest kept e               */
-    uint32_t rounds;      /* histogram levels summed over the cluster         */
+    uint32_t rounds;      /* histogram levels summed over the cluster; 0 = row
+                             finished by the streaming path                   */
     uint32_t n_gt;        /* tokens with e >  threshold                       */
     uint32_t n_eq;        /* tokens with e == threshold                       */
     int32_t  index;       /* sampled token                                    */

@@ -45,7 +45,8 @@ struct alignas(256) WsHeader {
     uint32_t ticket;      // next logical workgroup id of the running launch
     uint32_t finished;    // workgroups that have left the running launch
     int32_t  error;       // sticky RS_ERR_DEVICE
-    uint32_t pad[61];
+    uint32_t n_need;      // rows the streaming pass handed to the cluster kernel
+    uint32_t pad[60];
 };
 
 // Per-row record.  Everything a call reads before writing it is zero when the
@@ -73,6 +74,7 @@ struct Params {
     uint32_t    *e_bits;       // or null
     WsHeader    *hdr;
     RowCtl      *ctl;
+    const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
     int64_t      row_stride;
     int32_t      B, V;
     uint32_t     G;            // workgroups per row
@@ -373,6 +375,47 @@ __device__ __forceinline__ u128 get_mass(uint64_t w0, uint64_t w1)
     return ((u128)(w1 & ~kValid) << 62) | (w0 & ~kValid);
 }
 
+// Last act of a workgroup of the cluster kernel: the workgroup that leaves last
+// resets the launch-wide counters for the next call.
+__device__ __forceinline__ void leave_launch(WsHeader *hdr)
+{
+    if (threadIdx.x == 0) {
+        wait_vmem();
+        const uint32_t fin = __hip_atomic_fetch_add(&hdr->finished, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        if (fin == gridDim.x - 1) { a_store(&hdr->finished, 0u); a_store(&hdr->ticket, 0u); a_store(&hdr->n_need, 0u); }
+    }
+}
+
+// Tie weight, kept total S and inverse-CDF target r from the threshold and
+// the masses around it (reference: sampling.cu:365-371 and :374-381).  One
+// thread; also fills the diagnostics record when there is one.
+struct Target { uint64_t w_tie; u128 r; };
+__device__ inline Target tie_and_target(const Params &p, uint32_t row, uint64_t rand64, float xmax, u128 D, u128 P,
+                                        uint32_t thr, uint32_t n_gt, uint32_t n_eq, u128 Gm, uint32_t levels, bool write_diag)
+{
+    const uint64_t w_thr = w_of_bits(thr);
+    u128 a = (P > Gm) ? (P - Gm) : (u128)0;
+    u128 bk = ((uint32_t)p.top_k > n_gt) ? (u128)w_thr * ((uint32_t)p.top_k - n_gt) : (u128)0;
+    if (n_eq > 1) { a = div_u32(a, n_eq); bk = div_u32(bk, n_eq); }
+    u128 wt = w_thr;
+    if (a < wt) wt = a;
+    if (bk < wt) wt = bk;
+    if (wt == 0 && Gm == 0) wt = 1;
+    Target t;
+    t.w_tie = (uint64_t)wt;
+    const u128 S = Gm + (u128)n_eq * t.w_tie;
+    t.r = p.inj_u ? ceil_mul(p.inj_u[row], S) : r_from_bits(rand64, S);
+    if (p.diag && write_diag) {
+        rs_row_diag *d = p.diag + row;
+        d->xmax = xmax; d->emin_bits = 0;
+        d->D[0] = (uint64_t)D; d->D[1] = (uint64_t)(D >> 64); d->P[0] = (uint64_t)P; d->P[1] = (uint64_t)(P >> 64);
+        d->left_bits = thr; d->thr_bits = thr; d->rounds = levels; d->n_gt = n_gt; d->n_eq = n_eq;
+        d->G[0] = (uint64_t)Gm; d->G[1] = (uint64_t)(Gm >> 64); d->w_tie = t.w_tie;
+        d->S[0] = (uint64_t)S; d->S[1] = (uint64_t)(S >> 64); d->r[0] = (uint64_t)t.r; d->r[1] = (uint64_t)(t.r >> 64);
+    }
+    return t;
+}
+
 // Waves per SIMD the register allocation must leave room for: the resident
 // tokens take 4R registers (8R with penalties), the rest is working set.
 template <int R, bool PEN> constexpr int min_waves()
@@ -381,20 +424,13 @@ template <int R, bool PEN> constexpr int min_waves()
     return data <= 32 ? 4 : data <= 64 ? 3 : 2;
 }
 
+// One slice of one row, start to finish.  Returns false when a bounded wait
+// gave up (the error word is set; the workgroup must leave at once).
 template <int R, bool PEN>
-__global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
+__device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint32_t row, const uint32_t part)
 {
-    __shared__ Lds s;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-
-    if (tid == 0) {
-        s.abort = 0;
-        s.bc32[0] = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
-    }
-    __syncthreads();
-    const uint32_t ticket = s.bc32[0];
     const uint32_t G = p.G;
-    const uint32_t row = ticket / G, part = ticket - row * G;
     if (tid == 64 && !p.inj_u) {
         // this call's 64 random bits, drawn while the logits are in flight (the state is
         // advanced once, at the end, by the row's first workgroup)
@@ -485,7 +521,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                 }
             }
             kmax = block_max_u32(s, v, lane, wave);
-            if (s.abort) return;
+            if (s.abort) return false;
         } else __syncthreads();
         kmax_row = kmax;
     }
@@ -511,7 +547,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         for (int j = 0; j < R; ++j)
             if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
     }
-    if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return;
+    if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return false;
     if (G > 1 && tid == 0) a_store(&rc->mx[part], 0u);   // every workgroup has read the maxima by now
     const uint64_t top_k = (uint64_t)p.top_k;
 
@@ -542,7 +578,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                     if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, b);
                 }
             }
-        if (!hist_combine(s, p.hdr, G, rc->h[levels - 1], 128, expect, lane, wave)) return;
+        if (!hist_combine(s, p.hdr, G, rc->h[levels - 1], 128, expect, lane, wave)) return false;
         // every workgroup has finished reading the level above: it published this level after that
         if (G > 1) zero_slice(rc->h[levels - 2], levels == 2 ? kNB : 128, part, G);
         f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
@@ -602,7 +638,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                 guard.tick(s, p.hdr);
                 const uint32_t total = block_sum_u32(s, valid, lane, wave);
                 if (total == ncand + G) break;
-                if (s.abort) return;
+                if (s.abort) return false;
             }
             if ((uint32_t)tid < G) a_mine = get_mass(w0, w1);
             // every workgroup wrote its entries after it had read the last histogram level
@@ -632,26 +668,8 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
 
     // ---- 5. tie weight, total S, target r (every workgroup, identically) ----
     if (tid == 0) {
-        const uint64_t w_thr = w_of_bits(thr);
-        u128 a = (P > Gm) ? (P - Gm) : (u128)0;
-        u128 bk = ((uint32_t)p.top_k > n_gt) ? (u128)w_thr * ((uint32_t)p.top_k - n_gt) : (u128)0;
-        if (n_eq > 1) { a = div_u32(a, n_eq); bk = div_u32(bk, n_eq); }
-        u128 wt = w_thr;
-        if (a < wt) wt = a;
-        if (bk < wt) wt = bk;
-        if (wt == 0 && Gm == 0) wt = 1;
-        const uint64_t w_tie = (uint64_t)wt;
-        const u128 S = Gm + (u128)n_eq * w_tie;
-        const u128 r = p.inj_u ? ceil_mul(p.inj_u[row], S) : r_from_bits(s.bc64[5], S);
-        s.bc64[1] = w_tie; s.bc128[0] = r;
-        if (p.diag && part == 0) {
-            rs_row_diag *d = p.diag + row;
-            d->xmax = xmax; d->emin_bits = 0;
-            d->D[0] = (uint64_t)D; d->D[1] = (uint64_t)(D >> 64); d->P[0] = (uint64_t)P; d->P[1] = (uint64_t)(P >> 64);
-            d->left_bits = thr; d->thr_bits = thr; d->rounds = levels; d->n_gt = n_gt; d->n_eq = n_eq;
-            d->G[0] = (uint64_t)Gm; d->G[1] = (uint64_t)(Gm >> 64); d->w_tie = w_tie;
-            d->S[0] = (uint64_t)S; d->S[1] = (uint64_t)(S >> 64); d->r[0] = (uint64_t)r; d->r[1] = (uint64_t)(r >> 64);
-        }
+        const Target t = tie_and_target(p, row, s.bc64[5], xmax, D, P, thr, n_gt, n_eq, Gm, levels, part == 0);
+        s.bc64[1] = t.w_tie; s.bc128[0] = t.r;
     }
     __syncthreads();
     const uint64_t w_tie = s.bc64[1];
@@ -702,7 +720,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                 guard.tick(s, p.hdr);
                 const uint32_t total = block_sum_u32(s, valid, lane, wave);
                 if (total == G) break;
-                if (s.abort) return;
+                if (s.abort) return false;
             }
             zero_slice(rc->h[levels - 1], last_nb, part, G);
             before = block_sum_u128(s, (uint32_t)tid < part ? get_mass(w0, w1) : (u128)0, lane, wave);
@@ -769,7 +787,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
                 s.bc32[7] = v - 1u;
             }
             __syncthreads();
-            if (s.abort) return;
+            if (s.abort) return false;
         }
         const uint32_t idx = s.bc32[7];
 #pragma unroll
@@ -806,9 +824,471 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
             st[2] = lo32;
             if (lo32 == 0) st[3] += 1;
         }
-        wait_vmem();
-        const uint32_t fin = __hip_atomic_fetch_add(&p.hdr->finished, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        if (fin == gridDim.x - 1) { a_store(&p.hdr->finished, 0u); a_store(&p.hdr->ticket, 0u); }
+    }
+    return true;
+}
+
+// Workgroups take their (row, slice) from a ticket counter, so that logical
+// ids follow the order in which workgroups actually start: a workgroup only
+// ever waits for lower tickets, whose holders are running or done.
+template <int R, bool PEN>
+__global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
+{
+    __shared__ Lds s;
+    if (threadIdx.x == 0) {
+        s.abort = 0;
+        s.bc32[0] = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
+    }
+    __syncthreads();
+    const uint32_t ticket = s.bc32[0];
+    const uint32_t row = ticket / p.G;
+    if (!sample_slice<R, PEN>(p, s, row, ticket - row * p.G)) return;
+    leave_launch(p.hdr);
+}
+
+// The launch that follows the streaming pass: workgroups work through the
+// rows on its list, taking tickets until the list is exhausted.
+template <int R>
+__global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list_kernel(const Params p)
+{
+    __shared__ Lds s;
+    const uint32_t G = p.G;
+    if (a_load(&p.hdr->n_need) == 0u) return;                    // nothing left over: no ticket was taken
+    for (;;) {
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            s.abort = 0;
+            s.bc32[0] = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        }
+        __syncthreads();
+        const uint32_t ticket = s.bc32[0];
+        const uint32_t slot = ticket / G;
+        if (slot >= a_load(&p.hdr->n_need)) break;
+        if (!sample_slice<R, false>(p, s, p.need[slot], ticket - slot * G)) return;
+    }
+    leave_launch(p.hdr);
+}
+
+// ---------------------------------------------------------- streaming path --
+// For large batches with a small top_k the cluster kernel's exchanges cost
+// more than the data movement.  The streaming path has no waits at all:
+//
+//   stream_kernel   one workgroup per slice.  It reads the slice once, takes
+//                   its OWN maximum as the frame (the significand of e does
+//                   not depend on the frame, so a slice's histogram is the
+//                   row's up to a shift of whole octaves), writes its level-1
+//                   histogram and stashes its top_k largest tokens -- the
+//                   row's top_k tokens are among them -- ordered by bin.
+//   finish_kernel   one workgroup per row.  It shifts the slice histograms
+//                   into the row's frame and adds them, finds the boundary
+//                   bin, pulls the few stashed tokens at or above it, resolves
+//                   the threshold on them and picks.  A row whose stashes do
+//                   not reach down to the boundary bin (top_p cuts deeper
+//                   than any slice's top_k, or a huge tie) is put on a list,
+//                   and the cluster kernel then runs for the listed rows.
+constexpr int      kSB       = 164;           // level-1 bins in use: indices 348..511
+constexpr uint32_t kBin0     = 348u;          // index of e = 2^-40
+constexpr int      kStashCap = 2048;          // stash entries per slice
+constexpr int      kStreamK  = 1024;          // largest top_k the streaming path takes
+constexpr int      kFinCap   = 4096;          // tokens the finishing workgroup can hold
+
+struct PartHdr {
+    uint32_t mkey;        // fkey(max x of the slice)
+    uint32_t cov;         // the stash holds every token of the slice with bin - 348 >= cov
+    uint32_t n;           // entries in the stash
+    uint32_t pad;
+};
+
+struct StreamView {
+    PartHdr  *hdr;        // [B][G]
+    uint64_t *hist;       // [B][G][kSB]   packed bins in the slice's frame
+    uint64_t *stash;      // [B][G][kStashCap]   bits(e, slice frame) << 32 | index, by descending bin
+    uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
+    uint32_t *need;       // [B]  rows left to the cluster kernel
+    uint32_t  G;          // slices per row
+};
+
+struct LdsA {
+    uint64_t hm[kSB];
+    uint64_t list[kStashCap];
+    uint32_t off[kSB];
+    uint32_t u32[kWaves * 4];
+    uint32_t ctr, cov, n;
+};
+
+template <int R>
+__global__ void __launch_bounds__(kThreads, (R <= 4 ? 8 : R <= 8 ? 6 : 3)) stream_kernel(const Params p, const StreamView v)
+{
+    __shared__ LdsA s;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const uint32_t G = v.G;
+    const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
+    const uint32_t V4 = (uint32_t)p.V >> 2;
+    const uint32_t base4 = part * (uint32_t)(kThreads * R) + (uint32_t)tid;
+    const int nv = base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - base4 + kThreads - 1) / kThreads);
+    const float4 *lg = reinterpret_cast<const float4 *>(p.logits + (int64_t)row * p.row_stride);
+
+    uint32_t eb[R * 4];                                 // x, then bits(e)
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const float4 l = lg[min(base4 + (uint32_t)(j * kThreads), V4 - 1)];
+        eb[j * 4 + 0] = __float_as_uint(l.x * p.c); eb[j * 4 + 1] = __float_as_uint(l.y * p.c);
+        eb[j * 4 + 2] = __float_as_uint(l.z * p.c); eb[j * 4 + 3] = __float_as_uint(l.w * p.c);
+    }
+    // x = l * c is the definition unless a NaN or Inf shows up (see sample_kernel)
+    constexpr int kSpecial = 0x207;
+    bool special = false;
+    float lmax = -3.402823466e+38f;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) special |= __builtin_amdgcn_classf(__uint_as_float(eb[j * 4 + k]), kSpecial);
+        if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(__uint_as_float(eb[j * 4]), __uint_as_float(eb[j * 4 + 1])),
+                                             fmaxf(__uint_as_float(eb[j * 4 + 2]), __uint_as_float(eb[j * 4 + 3]))));
+    }
+    if (special) {
+        lmax = -3.402823466e+38f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const float4 l = lg[min(base4 + (uint32_t)(j * kThreads), V4 - 1)];
+            const float x0 = sf(sf(l.x) * p.c), x1 = sf(sf(l.y) * p.c), x2 = sf(sf(l.z) * p.c), x3 = sf(sf(l.w) * p.c);
+            if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
+            eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
+            eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
+        }
+    }
+    if (tid < kSB) s.hm[tid] = 0;
+    if (tid == 0) s.ctr = 0;
+    uint32_t k = wave_max_u32(fkey(lmax));
+    if (lane == 0) s.u32[wave] = k;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) k = max(k, s.u32[w]);
+    const float M = __builtin_floorf(fkey_inv(k));
+
+    // e in the slice's frame and its histogram
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) eb[j * 4 + q] = e_bits_of(__uint_as_float(eb[j * 4 + q]), M);
+        if (j < nv) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t b = eb[j * 4 + q];
+                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) - kBin0]),
+                          (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < kSB) v.hist[((size_t)row * G + part) * kSB + tid] = s.hm[tid];
+
+    // The slice's own top_k: first bin (largest e first) at which its count reaches top_k.
+    // The stash takes that bin too if it fits, else only the bins above it.
+    if (wave == 0) {
+        const uint32_t Ks = (uint32_t)p.top_k;
+        uint32_t c3[3];
+        uint32_t cs = 0;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int b = kSB - 1 - 3 * lane - i;
+            c3[i] = b >= 0 ? pack_count(s.hm[b]) : 0u;
+            cs += c3[i];
+        }
+        const uint32_t ci = wave_inclusive_scan(cs);
+        uint32_t run = ci - cs;
+        const uint32_t total = lane63(ci);
+        if (lane == 0 && total < Ks) { s.cov = 0u; s.n = total; }       // a short slice: all of it (total < top_k <= cap)
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int b = kSB - 1 - 3 * lane - i;
+            if (b >= 0) s.off[b] = run;                                   // tokens in the bins above b
+            const uint32_t nx = run + c3[i];
+            if (b >= 0) v.cum[((size_t)row * G + part) * kSB + b] = nx;
+            if (run < Ks && nx >= Ks) {
+                if (nx <= (uint32_t)kStashCap) { s.cov = (uint32_t)b; s.n = nx; }
+                else { s.cov = (uint32_t)b + 1u; s.n = run; }
+            }
+            run = nx;
+        }
+    }
+    __syncthreads();
+    const uint32_t cov = s.cov, n = s.n;
+    const uint32_t cut = (cov + kBin0) << 21;
+
+    // Compact the candidates into LDS (order irrelevant), one counter update per wave.
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const bool ok = j < nv;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) cnt += __popcll(__ballot(ok && eb[j * 4 + q] >= cut));
+    }
+    uint32_t basew = 0;
+    if (lane == 0) basew = atomicAdd(&s.ctr, cnt);
+    basew = __builtin_amdgcn_readfirstlane(basew);
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const bool ok = j < nv;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t bq = eb[j * 4 + q];
+            const bool pass = ok && bq >= cut;
+            const uint64_t m = __ballot(pass);
+            if (pass) {
+                const uint32_t o = basew + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                if (o < (uint32_t)kStashCap) s.list[o] = ((uint64_t)bq << 32) | ((base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)q);
+            }
+            basew += __popcll(m);
+        }
+    }
+    __syncthreads();
+    // Write them out grouped by bin, largest e first, so that the finishing
+    // workgroup can take a prefix.
+    uint64_t *st = v.stash + ((size_t)row * G + part) * kStashCap;
+    for (uint32_t i = tid; i < n; i += kThreads) {
+        const uint64_t e = s.list[i];
+        const uint32_t o = atomicAdd(&s.off[(uint32_t)(e >> 53) - kBin0], 1u);
+        if (o < (uint32_t)kStashCap) st[o] = e;
+    }
+    if (tid == 0) {
+        PartHdr ph;
+        ph.mkey = k; ph.cov = cov; ph.n = n; ph.pad = 0;
+        v.hdr[(size_t)row * G + part] = ph;
+    }
+}
+
+struct LdsB {
+    uint64_t list[kFinCap];      // gathered tokens, row frame: bits << 32 | index
+    uint64_t blo[kMaxParts], bhi[kMaxParts];
+    uint64_t small[128];
+    uint32_t delta[kMaxParts];   // octaves between the row's frame and slice g's
+    uint32_t take[kMaxParts];    // inclusive prefix of the entries taken from each stash
+    uint32_t nsmall, bucket, fail;
+};
+
+// Inverse CDF by buckets of the token index: sum the kept weights per bucket
+// (bucket = (index >> shift) & 255, tokens outside [lo_idx, hi_idx) ignored),
+// scan, and return the bucket that holds target r, with r reduced to an offset
+// inside it.  Weights are < 2^64 and a sum has < 2^12 terms, so the halves
+// summed separately stay below 2^44 + 2^32.
+template <typename W>
+__device__ __forceinline__ uint32_t bucket_step(Lds &s, LdsB &t, uint32_t nlist, uint32_t shift, uint32_t lo_idx, uint32_t hi_idx,
+                                                u128 &r, W weight, int lane, int wave)
+{
+    const int tid = threadIdx.x;
+    t.blo[tid] = 0; t.bhi[tid] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < nlist; i += kThreads) {
+        const uint64_t e = t.list[i];
+        const uint32_t idx = (uint32_t)e;
+        if (idx >= lo_idx && idx < hi_idx) {
+            const uint64_t w = weight((uint32_t)(e >> 32));
+            if (w) {
+                const uint32_t bk = (idx >> shift) & 255u;
+                atomicAdd(reinterpret_cast<unsigned long long *>(&t.blo[bk]), (unsigned long long)(w & 0xFFFFFFFFull));
+                atomicAdd(reinterpret_cast<unsigned long long *>(&t.bhi[bk]), (unsigned long long)(w >> 32));
+            }
+        }
+    }
+    __syncthreads();
+    const u128 mine = (u128)t.blo[tid] + ((u128)t.bhi[tid] << 32);
+    u128 inc = wave_inclusive_scan(mine);
+    if (lane == kWave - 1) s.q128[wave] = inc;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) inc += s.q128[w];
+    const u128 exc = inc - mine;
+    if (exc < r && r <= inc) { t.bucket = (uint32_t)tid; s.bc128[1] = r - exc; }
+    __syncthreads();
+    r = s.bc128[1];
+    return t.bucket;
+}
+
+template <int R>     // R of the stream_kernel that filled the view
+__global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const StreamView v)
+{
+    __shared__ Lds s;
+    __shared__ LdsB t;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const uint32_t G = v.G, row = blockIdx.x;
+    const PartHdr *hdrs = v.hdr + (size_t)row * G;
+    const uint64_t *hists = v.hist + (size_t)row * G * kSB;
+
+    if (tid == 0) { s.abort = 0; t.fail = 0; s.ctr = 0; }
+    PartHdr ph;
+    ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.pad = 0;
+    if ((uint32_t)tid < G) ph = hdrs[tid];
+    const uint32_t kmax = block_max_u32(s, ph.mkey, lane, wave);
+    const float xmax = fkey_inv(kmax);
+    const float M = __builtin_floorf(xmax);
+    uint32_t dl = 0;
+    if ((uint32_t)tid < G) {
+        const float d = M - __builtin_floorf(fkey_inv(ph.mkey));      // >= 0, a whole number or huge
+        dl = d >= 64.0f ? 64u : (uint32_t)d;
+        t.delta[tid] = dl;
+    }
+    for (int b = tid; b < kNB; b += kThreads) s.g[b] = 0;
+    __syncthreads();
+
+    // the row's level-1 histogram: slice bins shifted down by 4 bins per octave; what falls below
+    // 2^-40 is clamped there, which leaves a count and no fraction bits.  Loads go out 8 at a time.
+    {
+        constexpr int kBatch = 8;
+        const uint32_t nh = G * (uint32_t)kSB;
+        for (uint32_t i0 = tid; i0 < nh; i0 += kBatch * kThreads) {
+            uint64_t w[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t i = i0 + (uint32_t)u * kThreads;
+                w[u] = i < nh ? hists[i] : 0ull;
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                if (w[u]) {
+                    const uint32_t i = i0 + (uint32_t)u * kThreads;
+                    const uint32_t g = i / (uint32_t)kSB, bin = i - g * (uint32_t)kSB;
+                    const int rb = (int)bin - 4 * (int)t.delta[g];
+                    const uint64_t add = rb >= 0 ? w[u] : (w[u] >> 43) << 43;
+                    atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[kBin0 + (uint32_t)max(rb, 0)]), (unsigned long long)add);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const uint64_t top_k = (uint64_t)p.top_k;
+    Found f = hist_find512(s, top_k, p.top_p, lane, wave);
+    const u128 D = s.D, P = s.P;
+    const uint32_t exb = f.bin >> 2;
+
+    // what each stash must hold, and whether it does
+    const uint32_t total = f.cnt_above + f.cnt_bin;
+    uint32_t mtake = 0;
+    bool bad = total > (uint32_t)kFinCap;
+    if ((uint32_t)tid < G) {
+        const int lb = (int)(f.bin - kBin0) + 4 * (int)dl;            // boundary bin in the slice's frame
+        if (dl >= 64u) mtake = 0;                                      // the whole slice is clamped; the boundary bin
+                                                                       // can then only be bin 348, handled below
+        else if (lb < kSB) mtake = v.cum[((size_t)row * G + tid) * kSB + lb];
+        if (f.bin == kBin0) bad = true;                                // clamped tokens of other frames are not in a stash
+        else if (mtake && ((int)ph.cov > lb || mtake > ph.n)) bad = true;
+    }
+    if (bad) t.fail = 1;
+    // prefix of the takes
+    uint32_t inc = wave_inclusive_scan(mtake);
+    __syncthreads();
+    if (lane == kWave - 1) s.u32[wave] = inc;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) inc += s.u32[w];
+    t.take[tid] = inc;
+    __syncthreads();
+    if (t.fail || t.take[kThreads - 1] != total) {
+        // not resolvable from the stashes: leave the row to the cluster kernel
+        if (tid == 0) {
+            const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
+            v.need[slot] = row;
+        }
+        return;
+    }
+
+    // gather the tokens at or above the boundary bin, re-based to the row's frame
+    {
+        constexpr int kBatch = 4;
+        for (uint32_t i0 = tid; i0 < total; i0 += kBatch * kThreads) {
+            uint64_t e[kBatch];
+            uint32_t sl[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t i = i0 + (uint32_t)u * kThreads;
+                e[u] = 0; sl[u] = 0;
+                if (i < total) {
+                    uint32_t lo_g = 0, hi_g = G - 1;                   // first slice whose prefix exceeds i
+                    while (lo_g < hi_g) {
+                        const uint32_t mid = (lo_g + hi_g) >> 1;
+                        if (t.take[mid] > i) hi_g = mid; else lo_g = mid + 1;
+                    }
+                    const uint32_t j = i - (lo_g ? t.take[lo_g - 1] : 0u);
+                    e[u] = v.stash[((size_t)row * G + lo_g) * kStashCap + j];
+                    sl[u] = lo_g;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t i = i0 + (uint32_t)u * kThreads;
+                if (i < total) {
+                    const uint32_t b = (uint32_t)(e[u] >> 32) - (t.delta[sl[u]] << 23);
+                    t.list[i] = ((uint64_t)b << 32) | (uint32_t)e[u];
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // remaining digits of the threshold, on the gathered tokens
+    uint32_t lo = f.bin << 21, span = (1u << 21) - 1u;
+    for (uint32_t lv = 2; lv <= (uint32_t)kLevels; ++lv) {
+        const uint32_t dsh = level_shift(lv);
+        lds_hist_zero(s, 128);
+        __syncthreads();
+        for (uint32_t i = tid; i < total; i += kThreads) {
+            const uint32_t b = (uint32_t)(t.list[i] >> 32);
+            if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, b);
+        }
+        __syncthreads();
+        f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
+        lo |= f.bin << dsh;
+        span = (1u << dsh) - 1u;
+    }
+    const uint32_t thr = lo;
+    if (tid == 0) {
+        uint64_t rand64 = 0;
+        if (!p.inj_u) {
+            uint32_t *st = p.rng + (size_t)row * 16;
+            uint32_t o[4];
+            philox4x32_10(st[2], st[3], st[4], st[5], st[0], st[1], o);
+            rand64 = ((uint64_t)o[0] << 32) | o[1];
+            const uint32_t lo32 = st[2] + 1;
+            st[2] = lo32;
+            if (lo32 == 0) st[3] += 1;
+        }
+        const Target tg = tie_and_target(p, row, rand64, xmax, D, P, thr, f.cnt_above, f.cnt_bin, f.mass_above, 0u, true);   // rounds = 0: no cluster histogram
+        s.bc64[1] = tg.w_tie; s.bc128[0] = tg.r;
+    }
+    __syncthreads();
+    const uint64_t w_tie = s.bc64[1];
+    u128 r = s.bc128[0];
+    auto weight = [&](uint32_t b) -> uint64_t { return (b > thr) ? w_of_bits(b) : (b == thr ? w_tie : 0); };
+
+    // inverse CDF in index order: slice, then run of 4R tokens, then token
+    constexpr uint32_t sh_run = 2 + (uint32_t)__builtin_ctz((unsigned)R);      // 4R tokens
+    constexpr uint32_t sh_slice = sh_run + 8;                                  // 256 runs
+    const uint32_t ga = bucket_step(s, t, total, sh_slice, 0u, 0xFFFFFFFFu, r, weight, lane, wave);
+    const uint32_t lo_a = ga << sh_slice;
+    const uint32_t gb = bucket_step(s, t, total, sh_run, lo_a, lo_a + (1u << sh_slice), r, weight, lane, wave);
+    const uint32_t lo_b = lo_a + (gb << sh_run);
+    if (tid == 0) t.nsmall = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < total; i += kThreads) {
+        const uint64_t e = t.list[i];
+        const uint32_t idx = (uint32_t)e;
+        if (idx >= lo_b && idx < lo_b + (1u << sh_run) && weight((uint32_t)(e >> 32))) {
+            const uint32_t o = atomicAdd(&t.nsmall, 1u);
+            if (o < 128u) t.small[o] = e;
+        }
+    }
+    __syncthreads();
+    const uint32_t ns = min(t.nsmall, 128u);
+    if ((uint32_t)tid < ns) {
+        const uint64_t me = t.small[tid];
+        const uint64_t wme = weight((uint32_t)(me >> 32));
+        u128 upto = 0;
+        for (uint32_t j = 0; j < ns; ++j) {
+            const uint64_t o = t.small[j];
+            if ((uint32_t)o <= (uint32_t)me) upto += weight((uint32_t)(o >> 32));
+        }
+        if (upto - wme < r && r <= upto) {
+            p.out[row] = (int32_t)(uint32_t)me;
+            if (p.diag) p.diag[row].index = (int32_t)(uint32_t)me;
+        }
     }
 }
 
@@ -869,6 +1349,35 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
     return {maxR, parts(maxR)};
 }
 
+// Streaming geometry: slices of 16 float4 per thread (16384 tokens).
+constexpr int kStreamR = 16;
+static uint32_t stream_parts(int32_t V) { return ((uint32_t)V / 4 + kThreads * kStreamR - 1) / (kThreads * kStreamR); }
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+struct StreamLayout { size_t hdr, hist, cum, stash, need, end; };
+static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
+{
+    const size_t parts = (size_t)B * stream_parts(V);
+    StreamLayout l;
+    l.hdr = align256(base);
+    l.hist = align256(l.hdr + parts * sizeof(PartHdr));
+    l.cum = align256(l.hist + parts * kSB * sizeof(uint64_t));
+    l.stash = align256(l.cum + parts * kSB * sizeof(uint32_t));
+    l.need = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
+    l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
+    return l;
+}
+
+// The streaming path pays off when a call is many workgroup-rounds long and
+// top_k bounds the kept set; RS_FORCE_PATH=cluster|stream overrides (tests).
+static bool choose_stream(int32_t B, int32_t V, int32_t top_k, bool pen, bool want_e, const Geometry &g)
+{
+    const bool eligible = !pen && !want_e && top_k <= kStreamK;
+    const char *force = getenv("RS_FORCE_PATH");
+    if (force && force[0] == 'c') return false;
+    if (force && force[0] == 's') return eligible;
+    return eligible && g.G >= 4 && (uint64_t)B * g.G >= 2048;
+}
+
 template <bool PEN>
 static hipError_t launch_sample(int R, dim3 grid, hipStream_t st, const Params &p)
 {
@@ -881,6 +1390,19 @@ static hipError_t launch_sample(int R, dim3 grid, hipStream_t st, const Params &
     default:
         if constexpr (!PEN) hipLaunchKernelGGL((sample_kernel<32, false>), grid, dim3(kThreads), 0, st, p);
         break;
+    }
+    return hipGetLastError();
+}
+
+static hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p)
+{
+    switch (R) {
+    case 1:  hipLaunchKernelGGL((sample_list_kernel<1>),  grid, dim3(kThreads), 0, st, p); break;
+    case 2:  hipLaunchKernelGGL((sample_list_kernel<2>),  grid, dim3(kThreads), 0, st, p); break;
+    case 4:  hipLaunchKernelGGL((sample_list_kernel<4>),  grid, dim3(kThreads), 0, st, p); break;
+    case 8:  hipLaunchKernelGGL((sample_list_kernel<8>),  grid, dim3(kThreads), 0, st, p); break;
+    case 16: hipLaunchKernelGGL((sample_list_kernel<16>), grid, dim3(kThreads), 0, st, p); break;
+    default: hipLaunchKernelGGL((sample_list_kernel<32>), grid, dim3(kThreads), 0, st, p); break;
     }
     return hipGetLastError();
 }
@@ -932,7 +1454,7 @@ int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes)
     if (!bytes) return RS_ERR_NULL;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
-    *bytes = sizeof(WsHeader) + (size_t)B * sizeof(RowCtl);
+    *bytes = stream_layout(B, V, sizeof(WsHeader) + (size_t)B * sizeof(RowCtl)).end;
     return RS_OK;
 }
 
@@ -990,8 +1512,23 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
-    const dim3 grid((uint32_t)B * g.G);
-    const hipError_t e = pen ? launch_sample<true>(g.R, grid, (hipStream_t)stream, p)
+    p.need = nullptr;
+    dim3 grid((uint32_t)B * g.G);
+    if (choose_stream(B, V, top_k, pen, e_bits != nullptr, g)) {
+        const StreamLayout l = stream_layout(B, V, sizeof(WsHeader) + (size_t)B * sizeof(RowCtl));
+        char *w = (char *)workspace;
+        StreamView v;
+        v.hdr = (PartHdr *)(w + l.hdr); v.hist = (uint64_t *)(w + l.hist); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
+        v.need = (uint32_t *)(w + l.need); v.G = stream_parts(V);
+        hipStream_t st = (hipStream_t)stream;
+        hipLaunchKernelGGL((stream_kernel<kStreamR>), dim3((uint32_t)B * v.G), dim3(kThreads), 0, st, p, v);
+        hipLaunchKernelGGL((finish_kernel<kStreamR>), dim3((uint32_t)B), dim3(kThreads), 0, st, p, v);
+        if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
+        p.need = v.need;               // the cluster kernel follows for the rows the finish left over
+        if (grid.x > 1024u) grid.x = 1024u / g.G * g.G > 0 ? 1024u / g.G * g.G : g.G;
+    }
+    const hipError_t e = p.need ? launch_list(g.R, grid, (hipStream_t)stream, p)
+                       : pen ? launch_sample<true>(g.R, grid, (hipStream_t)stream, p)
                              : launch_sample<false>(g.R, grid, (hipStream_t)stream, p);
     return e == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
 }

@@ -66,9 +66,18 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
         res2 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen2, presence=presence, repetition=repetition,
                           decay=decay)
         _check(res2, ref_out, ref_diag, what + " (second call)")
+        if pen_np is None:
+            # the wait-free streaming path (taken for top_k <= 1024; rows it cannot finish go on to
+            # the cluster kernel), then the cluster path again on the workspace it leaves behind
+            for path in ("stream", "cluster"):
+                os.environ["RS_FORCE_PATH"] = path
+                res3 = smp.sample(lg, c, k, p, uniforms=u)
+                _check(res3, ref_out, ref_diag, what + " (path %s)" % path)
+                assert smp.status() == 0
         return res, ref_diag
     finally:
         os.environ.pop("RS_FORCE_R", None)
+        os.environ.pop("RS_FORCE_PATH", None)
 
 
 def test_c1_uniform_logits_top_p(torch_cuda, oracle):
@@ -152,6 +161,37 @@ def test_uniform_extremes(torch_cuda, oracle):
     kept0 = np.nonzero(e[0] >= thr[0])[0]
     kept1 = np.nonzero(e[1] >= thr[1])[0]
     assert res["out"][0] == kept0[-1] and res["out"][1] == kept1[0]
+
+
+def test_streaming_path_mixed_rows(torch_cuda, oracle):
+    """Rows of one batch that end differently on the streaming path: top_k-bound rows finished from the
+    stashes, rows where top_p cuts inside the stashes, peaked rows, masked (-inf) stretches that put whole
+    slices in another frame, a row of ties too large to gather, NaN/Inf entries."""
+    from tests import capi
+    V = 65536 + 4096                 # 5 slices of 16384 tokens, the last one short
+    rng = np.random.default_rng(77)
+    lg = (rng.standard_normal((10, V)) * 2.0).astype(np.float32)
+    lg[1, 1000] = 40.0                                   # one dominant token
+    lg[2, 16384:49152] = -np.inf                         # two slices fully masked
+    lg[3, :] = -np.inf; lg[3, 60000:60010] = 1.0         # almost everything masked, small tie
+    lg[4, :] = 0.25                                      # all equal
+    lg[5, 5] = np.nan; lg[5, 6] = np.inf; lg[5, 7] = -np.inf
+    lg[6, 16384:32768] -= 200.0                          # a slice 288 octaves down: clamped in the row's frame
+    lg[7, :32768] = lg[7, 32768]                         # a tie of 32768 tokens at a middling value
+    lg[8, 20000:20600] = 9.0                             # a tie of 600 tokens at the top
+    for (k, p) in [(50, 0.9), (1024, 0.95), (1, 1.0), (1000, 0.2), (7, 1.0), (1024, 1.0)]:
+        _run_case(torch_cuda, oracle, capi, lg, 0.9, k, p, u_np=H.uniforms(10, 91), what="stream mixed k=%s p=%s" % (k, p))
+    # which rows the streaming path finished itself (diag.rounds == 0) and which it handed on
+    os.environ["RS_FORCE_PATH"] = "stream"
+    try:
+        rc, c, k, p = capi.normalize(0.9, 50, 0.9, V, 10, 1)
+        res = capi.Sampler(10, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p,
+                                         uniforms=torch_cuda.from_numpy(H.uniforms(10, 91)).cuda())
+        rounds = res["diag"]["rounds"]
+        assert rounds[0] == 0 and rounds[1] == 0 and rounds[2] == 0 and rounds[9] == 0, rounds
+        assert rounds[4] >= 1, rounds                             # a tie of all 69632 tokens: not gatherable
+    finally:
+        os.environ.pop("RS_FORCE_PATH", None)
 
 
 def test_penalty_path_single_step(torch_cuda, oracle):
