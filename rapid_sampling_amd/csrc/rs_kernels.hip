@@ -888,7 +888,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
 //                   and the cluster kernel then runs for the listed rows.
 constexpr int      kSB       = 164;           // level-1 bins in use: indices 348..511
 constexpr uint32_t kBin0     = 348u;          // index of e = 2^-40
-constexpr int      kStashCap = 2048;          // stash entries per slice
+constexpr int      kStashCap = 1280;          // stash entries per slice (at least kStreamK)
 constexpr int      kStreamK  = 1024;          // largest top_k the streaming path takes
 constexpr int      kFinCap   = 4096;          // tokens the finishing workgroup can hold
 
@@ -909,29 +909,30 @@ struct StreamView {
 };
 
 struct LdsA {
+    uint4    grp[kStashCap];     // float4 groups that hold a candidate: bits of their 4 tokens
+    uint32_t gidx[kStashCap];    // and the index of their first token
     uint64_t hm[kSB];
-    uint64_t list[kStashCap];
     uint32_t off[kSB];
-    uint32_t u32[kWaves * 4];
-    uint32_t ctr, cov, n;
+    uint32_t u32[16];
+    uint32_t cov, n;
 };
 
-template <int R>
-__global__ void __launch_bounds__(kThreads, (R <= 4 ? 8 : R <= 8 ? 6 : 3)) stream_kernel(const Params p, const StreamView v)
+template <int R, int NT>     // NT threads, each with R float4 of the slice
+__global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Params p, const StreamView v)
 {
     __shared__ LdsA s;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t G = v.G;
     const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
     const uint32_t V4 = (uint32_t)p.V >> 2;
-    const uint32_t base4 = part * (uint32_t)(kThreads * R) + (uint32_t)tid;
-    const int nv = base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - base4 + kThreads - 1) / kThreads);
+    const uint32_t base4 = part * (uint32_t)(NT * R) + (uint32_t)tid;
+    const int nv = base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - base4 + NT - 1) / NT);
     const float4 *lg = reinterpret_cast<const float4 *>(p.logits + (int64_t)row * p.row_stride);
 
     uint32_t eb[R * 4];                                 // x, then bits(e)
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-        const float4 l = lg[min(base4 + (uint32_t)(j * kThreads), V4 - 1)];
+        const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
         eb[j * 4 + 0] = __float_as_uint(l.x * p.c); eb[j * 4 + 1] = __float_as_uint(l.y * p.c);
         eb[j * 4 + 2] = __float_as_uint(l.z * p.c); eb[j * 4 + 3] = __float_as_uint(l.w * p.c);
     }
@@ -950,7 +951,7 @@ __global__ void __launch_bounds__(kThreads, (R <= 4 ? 8 : R <= 8 ? 6 : 3)) strea
         lmax = -3.402823466e+38f;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            const float4 l = lg[min(base4 + (uint32_t)(j * kThreads), V4 - 1)];
+            const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
             const float x0 = sf(sf(l.x) * p.c), x1 = sf(sf(l.y) * p.c), x2 = sf(sf(l.z) * p.c), x3 = sf(sf(l.w) * p.c);
             if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
             eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
@@ -958,26 +959,26 @@ __global__ void __launch_bounds__(kThreads, (R <= 4 ? 8 : R <= 8 ? 6 : 3)) strea
         }
     }
     if (tid < kSB) s.hm[tid] = 0;
-    if (tid == 0) s.ctr = 0;
     uint32_t k = wave_max_u32(fkey(lmax));
     if (lane == 0) s.u32[wave] = k;
     __syncthreads();
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) k = max(k, s.u32[w]);
+    for (int w = 0; w < (NT / kWave); ++w) k = max(k, s.u32[w]);
     const float M = __builtin_floorf(fkey_inv(k));
 
-    // e in the slice's frame and its histogram
+    // e in the slice's frame and its histogram; slots past the end of the row become 0, below any cut
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) eb[j * 4 + q] = e_bits_of(__uint_as_float(eb[j * 4 + q]), M);
         if (j < nv) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const uint32_t b = eb[j * 4 + q];
+                const uint32_t b = e_bits_of(__uint_as_float(eb[j * 4 + q]), M);
+                eb[j * 4 + q] = b;
                 atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) - kBin0]),
                           (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
             }
+        } else {
+            eb[j * 4] = 0; eb[j * 4 + 1] = 0; eb[j * 4 + 2] = 0; eb[j * 4 + 3] = 0;
         }
     }
     __syncthreads();
@@ -1002,9 +1003,11 @@ __global__ void __launch_bounds__(kThreads, (R <= 4 ? 8 : R <= 8 ? 6 : 3)) strea
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             const int b = kSB - 1 - 3 * lane - i;
-            if (b >= 0) s.off[b] = run;                                   // tokens in the bins above b
             const uint32_t nx = run + c3[i];
-            if (b >= 0) v.cum[((size_t)row * G + part) * kSB + b] = nx;
+            if (b >= 0) {
+                s.off[b] = run;                                           // tokens in the bins above b
+                v.cum[((size_t)row * G + part) * kSB + b] = nx;
+            }
             if (run < Ks && nx >= Ks) {
                 if (nx <= (uint32_t)kStashCap) { s.cov = (uint32_t)b; s.n = nx; }
                 else { s.cov = (uint32_t)b + 1u; s.n = run; }
@@ -1016,40 +1019,44 @@ __global__ void __launch_bounds__(kThreads, (R <= 4 ? 8 : R <= 8 ? 6 : 3)) strea
     const uint32_t cov = s.cov, n = s.n;
     const uint32_t cut = (cov + kBin0) << 21;
 
-    // Compact the candidates into LDS (order irrelevant), one counter update per wave.
-    uint32_t cnt = 0;
+    // Candidates (bits >= cut) are at most n <= kStashCap, so at most that many float4 groups
+    // hold one.  Each thread copies its groups with a candidate into LDS at an offset from a scan
+    // of the per-thread counts; the tokens of those groups are then gone through densely.
+    uint32_t mine = 0;
 #pragma unroll
-    for (int j = 0; j < R; ++j) {
-        const bool ok = j < nv;
+    for (int j = 0; j < R; ++j)
+        mine += max(max(eb[j * 4], eb[j * 4 + 1]), max(eb[j * 4 + 2], eb[j * 4 + 3])) >= cut ? 1u : 0u;
+    uint32_t o = wave_inclusive_scan(mine);
+    if (lane == kWave - 1) s.u32[wave] = o;
+    __syncthreads();
+    uint32_t ngroups = 0;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) cnt += __popcll(__ballot(ok && eb[j * 4 + q] >= cut));
+    for (int w = 0; w < (NT / kWave); ++w) {
+        if (w < wave) o += s.u32[w];
+        ngroups += s.u32[w];
     }
-    uint32_t basew = 0;
-    if (lane == 0) basew = atomicAdd(&s.ctr, cnt);
-    basew = __builtin_amdgcn_readfirstlane(basew);
+    o -= mine;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-        const bool ok = j < nv;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t bq = eb[j * 4 + q];
-            const bool pass = ok && bq >= cut;
-            const uint64_t m = __ballot(pass);
-            if (pass) {
-                const uint32_t o = basew + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-                if (o < (uint32_t)kStashCap) s.list[o] = ((uint64_t)bq << 32) | ((base4 + (uint32_t)j * kThreads) * 4 + (uint32_t)q);
+        if (max(max(eb[j * 4], eb[j * 4 + 1]), max(eb[j * 4 + 2], eb[j * 4 + 3])) >= cut) {
+            if (o < (uint32_t)kStashCap) {
+                s.grp[o] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
+                s.gidx[o] = (base4 + (uint32_t)j * NT) * 4;
             }
-            basew += __popcll(m);
+            ++o;
         }
     }
     __syncthreads();
-    // Write them out grouped by bin, largest e first, so that the finishing
+    // Write the candidates out grouped by bin, largest e first, so that the finishing
     // workgroup can take a prefix.
     uint64_t *st = v.stash + ((size_t)row * G + part) * kStashCap;
-    for (uint32_t i = tid; i < n; i += kThreads) {
-        const uint64_t e = s.list[i];
-        const uint32_t o = atomicAdd(&s.off[(uint32_t)(e >> 53) - kBin0], 1u);
-        if (o < (uint32_t)kStashCap) st[o] = e;
+    const uint32_t *gb = reinterpret_cast<const uint32_t *>(s.grp);
+    for (uint32_t i = tid; i < min(ngroups, (uint32_t)kStashCap) * 4u; i += NT) {
+        const uint32_t b = gb[i];
+        if (b >= cut) {
+            const uint32_t slot = atomicAdd(&s.off[(b >> 21) - kBin0], 1u);
+            if (slot < (uint32_t)kStashCap) st[slot] = ((uint64_t)b << 32) | (s.gidx[i >> 2] + (i & 3u));
+        }
     }
     if (tid == 0) {
         PartHdr ph;
@@ -1104,7 +1111,7 @@ __device__ __forceinline__ uint32_t bucket_step(Lds &s, LdsB &t, uint32_t nlist,
     return t.bucket;
 }
 
-template <int R>     // R of the stream_kernel that filled the view
+template <int SLICE_LOG2>     // log2 of the tokens per slice of the view
 __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const StreamView v)
 {
     __shared__ Lds s;
@@ -1258,9 +1265,10 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     u128 r = s.bc128[0];
     auto weight = [&](uint32_t b) -> uint64_t { return (b > thr) ? w_of_bits(b) : (b == thr ? w_tie : 0); };
 
-    // inverse CDF in index order: slice, then run of 4R tokens, then token
-    constexpr uint32_t sh_run = 2 + (uint32_t)__builtin_ctz((unsigned)R);      // 4R tokens
-    constexpr uint32_t sh_slice = sh_run + 8;                                  // 256 runs
+    // inverse CDF in index order: slice, then run of tokens, then token
+    constexpr uint32_t sh_slice = SLICE_LOG2;
+    constexpr uint32_t sh_run = sh_slice - 8;                                  // 256 runs of at most 128 tokens
+    static_assert(SLICE_LOG2 >= 8 && SLICE_LOG2 <= 15, "runs must fit the final all-pairs step");
     const uint32_t ga = bucket_step(s, t, total, sh_slice, 0u, 0xFFFFFFFFu, r, weight, lane, wave);
     const uint32_t lo_a = ga << sh_slice;
     const uint32_t gb = bucket_step(s, t, total, sh_run, lo_a, lo_a + (1u << sh_slice), r, weight, lane, wave);
@@ -1349,9 +1357,10 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
     return {maxR, parts(maxR)};
 }
 
-// Streaming geometry: slices of 16 float4 per thread (16384 tokens).
-constexpr int kStreamR = 16;
-static uint32_t stream_parts(int32_t V) { return ((uint32_t)V / 4 + kThreads * kStreamR - 1) / (kThreads * kStreamR); }
+// Streaming geometry: workgroups of 256 threads with 16 float4 each: slices of 16384 tokens.
+constexpr int kStreamR = 16, kStreamNT = 256, kStreamSliceLog2 = 14;
+static_assert(kStreamR * kStreamNT * 4 == 1 << kStreamSliceLog2, "slice size");
+static uint32_t stream_parts(int32_t V) { return ((uint32_t)V / 4 + kStreamNT * kStreamR - 1) / (kStreamNT * kStreamR); }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 struct StreamLayout { size_t hdr, hist, cum, stash, need, end; };
 static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
@@ -1521,8 +1530,8 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         v.hdr = (PartHdr *)(w + l.hdr); v.hist = (uint64_t *)(w + l.hist); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.need = (uint32_t *)(w + l.need); v.G = stream_parts(V);
         hipStream_t st = (hipStream_t)stream;
-        hipLaunchKernelGGL((stream_kernel<kStreamR>), dim3((uint32_t)B * v.G), dim3(kThreads), 0, st, p, v);
-        hipLaunchKernelGGL((finish_kernel<kStreamR>), dim3((uint32_t)B), dim3(kThreads), 0, st, p, v);
+        hipLaunchKernelGGL((stream_kernel<kStreamR, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
+        hipLaunchKernelGGL((finish_kernel<kStreamSliceLog2>), dim3((uint32_t)B), dim3(kThreads), 0, st, p, v);
         if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
         p.need = v.need;               // the cluster kernel follows for the rows the finish left over
         if (grid.x > 1024u) grid.x = 1024u / g.G * g.G > 0 ? 1024u / g.G * g.G : g.G;
