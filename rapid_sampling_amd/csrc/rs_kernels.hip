@@ -901,7 +901,8 @@ struct PartHdr {
 
 struct StreamView {
     PartHdr  *hdr;        // [B][G]
-    uint64_t *hist;       // [B][G][kSB]   packed bins in the slice's frame
+    uint64_t *rowhist;    // [B][512]  packed bins by absolute octave mod 128, summed over the row's slices with
+                          //           device atomics; zero between calls
     uint64_t *stash;      // [B][G][kStashCap]   bits(e, slice frame) << 32 | index, by descending bin
     uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
     uint32_t *need;       // [B]  rows left to the cluster kernel
@@ -982,7 +983,14 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         }
     }
     __syncthreads();
-    if (tid < kSB) v.hist[((size_t)row * G + part) * kSB + tid] = s.hm[tid];
+    // Add the slice's bins to the row's, which are kept by absolute octave (mod 128, 4 bins each):
+    // bin t of this frame is octave M - 40 + t/4.  Slices of one row may use different frames; as
+    // long as their maxima lie within 87 octaves of each other no two octaves in use coincide.
+    if (tid < kSB) {
+        const uint64_t w = s.hm[tid];
+        const float mm = M - 128.0f * __builtin_floorf(M * 0.0078125f);          // M mod 128, exact
+        if (w) a_add(&v.rowhist[(size_t)row * kNB + (((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u)], w);
+    }
 
     // The slice's own top_k: first bin (largest e first) at which its count reaches top_k.
     // The stash takes that bin too if it fits, else only the bins above it.
@@ -1119,47 +1127,39 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t G = v.G, row = blockIdx.x;
     const PartHdr *hdrs = v.hdr + (size_t)row * G;
-    const uint64_t *hists = v.hist + (size_t)row * G * kSB;
+    uint64_t *rowhist = v.rowhist + (size_t)row * kNB;
 
     if (tid == 0) { s.abort = 0; t.fail = 0; s.ctr = 0; }
     PartHdr ph;
     ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.pad = 0;
     if ((uint32_t)tid < G) ph = hdrs[tid];
+    const uint64_t h0 = rowhist[tid], h1 = rowhist[tid + kThreads];
+    rowhist[tid] = 0; rowhist[tid + kThreads] = 0;                   // left clean for the next call
     const uint32_t kmax = block_max_u32(s, ph.mkey, lane, wave);
+    const uint32_t kmin = ~block_max_u32(s, (uint32_t)tid < G ? ~ph.mkey : 0u, lane, wave);
     const float xmax = fkey_inv(kmax);
     const float M = __builtin_floorf(xmax);
+    // frames further apart than this may have put different octaves into one bin
+    const bool mixed = !(M - __builtin_floorf(fkey_inv(kmin)) < 88.0f);
     uint32_t dl = 0;
     if ((uint32_t)tid < G) {
         const float d = M - __builtin_floorf(fkey_inv(ph.mkey));      // >= 0, a whole number or huge
         dl = d >= 64.0f ? 64u : (uint32_t)d;
         t.delta[tid] = dl;
     }
-    for (int b = tid; b < kNB; b += kThreads) s.g[b] = 0;
-    __syncthreads();
-
-    // the row's level-1 histogram: slice bins shifted down by 4 bins per octave; what falls below
-    // 2^-40 is clamped there, which leaves a count and no fraction bits.  Loads go out 8 at a time.
+    // the row's level-1 histogram in the row's frame: bin r (octave M - 40 + r/4) sits at absolute
+    // position 4 (M mod 128) + r - 160; the other 348 positions hold tokens below 2^-40 of this
+    // frame, which are clamped there: a count and no fraction bits
     {
-        constexpr int kBatch = 8;
-        const uint32_t nh = G * (uint32_t)kSB;
-        for (uint32_t i0 = tid; i0 < nh; i0 += kBatch * kThreads) {
-            uint64_t w[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const uint32_t i = i0 + (uint32_t)u * kThreads;
-                w[u] = i < nh ? hists[i] : 0ull;
-            }
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                if (w[u]) {
-                    const uint32_t i = i0 + (uint32_t)u * kThreads;
-                    const uint32_t g = i / (uint32_t)kSB, bin = i - g * (uint32_t)kSB;
-                    const int rb = (int)bin - 4 * (int)t.delta[g];
-                    const uint64_t add = rb >= 0 ? w[u] : (w[u] >> 43) << 43;
-                    atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[kBin0 + (uint32_t)max(rb, 0)]), (unsigned long long)add);
-                }
-            }
-        }
+        const float mm = M - 128.0f * __builtin_floorf(M * 0.0078125f);
+        const uint32_t m4 = (uint32_t)(int)mm * 4u;
+        const uint32_t r0 = ((uint32_t)tid + 160u - m4) & 511u, r1 = ((uint32_t)tid + kThreads + 160u - m4) & 511u;
+        uint32_t low = 0;
+        if (r0 < (uint32_t)kSB) s.g[kBin0 + r0] = h0; else low += pack_count(h0);
+        if (r1 < (uint32_t)kSB) s.g[kBin0 + r1] = h1; else low += pack_count(h1);
+        for (int b = tid; b < (int)kBin0; b += kThreads) s.g[b] = 0;
+        low = block_sum_u32(s, low, lane, wave);
+        if (tid == 0) s.g[kBin0] += (uint64_t)low << 43;
     }
     __syncthreads();
     const uint64_t top_k = (uint64_t)p.top_k;
@@ -1170,7 +1170,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     // what each stash must hold, and whether it does
     const uint32_t total = f.cnt_above + f.cnt_bin;
     uint32_t mtake = 0;
-    bool bad = total > (uint32_t)kFinCap;
+    bool bad = mixed || total > (uint32_t)kFinCap;
     if ((uint32_t)tid < G) {
         const int lb = (int)(f.bin - kBin0) + 4 * (int)dl;            // boundary bin in the slice's frame
         if (dl >= 64u) mtake = 0;                                      // the whole slice is clamped; the boundary bin
@@ -1369,7 +1369,7 @@ static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
     StreamLayout l;
     l.hdr = align256(base);
     l.hist = align256(l.hdr + parts * sizeof(PartHdr));
-    l.cum = align256(l.hist + parts * kSB * sizeof(uint64_t));
+    l.cum = align256(l.hist + (size_t)B * kNB * sizeof(uint64_t));
     l.stash = align256(l.cum + parts * kSB * sizeof(uint32_t));
     l.need = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
     l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
@@ -1527,7 +1527,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         const StreamLayout l = stream_layout(B, V, sizeof(WsHeader) + (size_t)B * sizeof(RowCtl));
         char *w = (char *)workspace;
         StreamView v;
-        v.hdr = (PartHdr *)(w + l.hdr); v.hist = (uint64_t *)(w + l.hist); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
+        v.hdr = (PartHdr *)(w + l.hdr); v.rowhist = (uint64_t *)(w + l.hist); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.need = (uint32_t *)(w + l.need); v.G = stream_parts(V);
         hipStream_t st = (hipStream_t)stream;
         hipLaunchKernelGGL((stream_kernel<kStreamR, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
