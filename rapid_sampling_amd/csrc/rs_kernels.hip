@@ -74,6 +74,7 @@ struct Params {
     uint32_t    *e_bits;       // or null
     WsHeader    *hdr;
     RowCtl      *ctl;
+    uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
     int64_t      row_stride;
     int32_t      B, V;
@@ -992,10 +993,13 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         if (w) a_add(&v.rowhist[(size_t)row * kNB + (((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u)], w);
     }
 
-    // The slice's own top_k: first bin (largest e first) at which its count reaches top_k.
-    // The stash takes that bin too if it fits, else only the bins above it.
+    // What to stash: the bins from the top down to the first one at which the count reaches
+    // stash_k (that bin too if it fits).  With stash_k = top_k the row's top_k tokens are certainly
+    // in the stashes; the host aims lower when a row has many slices, since a slice then holds
+    // about top_k / slices of them, and the finishing workgroup checks that each stash reaches
+    // down to the row's boundary bin before it relies on it.
     if (wave == 0) {
-        const uint32_t Ks = (uint32_t)p.top_k;
+        const uint32_t Ks = p.stash_k;
         uint32_t c3[3];
         uint32_t cs = 0;
 #pragma unroll
@@ -1059,6 +1063,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     // workgroup can take a prefix.
     uint64_t *st = v.stash + ((size_t)row * G + part) * kStashCap;
     const uint32_t *gb = reinterpret_cast<const uint32_t *>(s.grp);
+#pragma unroll 4
     for (uint32_t i = tid; i < min(ngroups, (uint32_t)kStashCap) * 4u; i += NT) {
         const uint32_t b = gb[i];
         if (b >= cut) {
@@ -1376,15 +1381,16 @@ static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
     return l;
 }
 
-// The streaming path pays off when a call is many workgroup-rounds long and
-// top_k bounds the kept set; RS_FORCE_PATH=cluster|stream overrides (tests).
+// The streaming path (three launches, no waits) pays off when a call moves a
+// few hundred MB and top_k bounds the kept set; below that the single launch
+// of the cluster kernel wins.  RS_FORCE_PATH=cluster|stream overrides (tests).
 static bool choose_stream(int32_t B, int32_t V, int32_t top_k, bool pen, bool want_e, const Geometry &g)
 {
     const bool eligible = !pen && !want_e && top_k <= kStreamK;
     const char *force = getenv("RS_FORCE_PATH");
     if (force && force[0] == 'c') return false;
     if (force && force[0] == 's') return eligible;
-    return eligible && g.G >= 4 && (uint64_t)B * g.G >= 2048;
+    return eligible && g.G >= 4 && (uint64_t)B * (uint64_t)V >= (1ull << 25);
 }
 
 template <bool PEN>
@@ -1521,7 +1527,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
-    p.need = nullptr;
+    p.need = nullptr; p.stash_k = (uint32_t)top_k;
     dim3 grid((uint32_t)B * g.G);
     if (choose_stream(B, V, top_k, pen, e_bits != nullptr, g)) {
         const StreamLayout l = stream_layout(B, V, sizeof(WsHeader) + (size_t)B * sizeof(RowCtl));
@@ -1529,6 +1535,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         StreamView v;
         v.hdr = (PartHdr *)(w + l.hdr); v.rowhist = (uint64_t *)(w + l.hist); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.need = (uint32_t *)(w + l.need); v.G = stream_parts(V);
+        p.stash_k = (uint32_t)top_k < 128u ? (uint32_t)top_k : min((uint32_t)top_k, max(128u, 8u * (uint32_t)top_k / v.G));
         hipStream_t st = (hipStream_t)stream;
         hipLaunchKernelGGL((stream_kernel<kStreamR, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
         hipLaunchKernelGGL((finish_kernel<kStreamSliceLog2>), dim3((uint32_t)B), dim3(kThreads), 0, st, p, v);
