@@ -61,7 +61,7 @@ struct alignas(256) RowCtl {
     uint32_t mx[kMaxParts];     // per workgroup: fkey(max x of its slice), 0 = not yet written
     uint64_t A[2 * kMaxParts];  // per workgroup: a 124-bit mass as two words of 62 bits, each | kValid
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
-    uint64_t h[kLevels][kNB];   // cluster histograms, packed (see kPackOne)
+    uint64_t h[kLevels + 1][kNB];   // cluster histograms, packed (see kPackOne); one spare for the re-framed level 1
 };
 
 struct Params {
@@ -111,6 +111,7 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v)
 // Levels 2..4 take 7 more bits each (shifts 14, 7, 0).  Histograms are stored
 // by index (ascending in e); the scan walks them by digit = top - index.
 constexpr uint32_t kTop1 = 511u;                      // largest index at level 1
+constexpr uint32_t kBin0 = 348u;                      // smallest: e = 2^-40
 constexpr uint32_t kTopN = 127u;                      // largest index of a deeper level
 __device__ __forceinline__ uint32_t level_shift(uint32_t level) { return 21u - 7u * (level - 1u); }   // level >= 2
 
@@ -124,6 +125,14 @@ __device__ __forceinline__ uint32_t pack_count(uint64_t w) { return (uint32_t)(w
 __device__ __forceinline__ u128 pack_mass(uint64_t w, uint32_t ex)
 {
     return (u128)((w & kPackMask) + ((w >> 43) << 23)) << (ex - 87u);
+}
+
+// Bits of e in a frame `delta` octaves above the one they were computed in
+// (delta <= 64): the exponent drops by delta, clamped at 2^-40.
+__device__ __forceinline__ uint32_t rebase_bits(uint32_t b, uint32_t delta)
+{
+    const uint32_t d = delta << 23;
+    return max(b, d + kEMinBits) - d;
 }
 
 struct Found {               // result of a histogram scan (uniform over the workgroup)
@@ -237,9 +246,11 @@ __device__ __forceinline__ void zero_slice(uint64_t *gh, uint32_t nb, uint32_t p
 // bins back until their counts add up to `expected` -- count and value of a
 // contribution arrive in one word, so a complete count means complete data
 // and no arrival counter is needed.  The totals end in s.g.  A cluster of one
-// copies its own.  Returns false when the wait gave up.
+// copies its own.  With `slots`, the same polling rounds also fetch one
+// per-workgroup word each (thread t takes slot t) and go on until none of
+// them is 0.  Returns false when the wait gave up.
 __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, uint64_t *gh, int nb, uint32_t expected,
-                                             int lane, int wave)
+                                             int lane, int wave, const uint32_t *slots = nullptr, uint32_t *slot_value = nullptr)
 {
     __syncthreads();
     if (G == 1) {
@@ -259,6 +270,12 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
             const uint64_t w = a_load(&gh[b]);
             s.g[b] = w;
             c += pack_count(w);
+        }
+        if (slots && threadIdx.x < G) {
+            // thread t also waits for slot t (never 0 once written); a missing slot spoils the sum
+            const uint32_t v = a_load(&slots[threadIdx.x]);
+            *slot_value = v;
+            c += v == 0u ? 1u << 24 : 0u;
         }
         guard.tick(s, hdr);
         const uint32_t total = block_sum_u32(s, c, lane, wave);
@@ -502,44 +519,91 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
             }
         }
-        const uint32_t k = block_max_u32(s, fkey(lmax), lane, wave);
+        kmax_row = block_max_u32(s, fkey(lmax), lane, wave);            // of this slice, for now
         lds_hist_zero(s, kNB);
-        uint32_t kmax = k;
-        if (G > 1) {
-            // Exchange of the slice maxima without a counter: every workgroup writes its
-            // key (never 0 for a finite x) into its own slot and thread t waits for slot t.
-            if (tid == 0) a_store(&rc->mx[part], k);
-            uint32_t v = k;
-            if ((uint32_t)tid < G) {
-                const uint64_t t0 = wall_clock64();
-                uint32_t spins = 0;
-                while ((v = a_load(&rc->mx[tid])) == 0u) {
-                    if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
-                        a_store(&p.hdr->error, (int32_t)RS_ERR_DEVICE);
-                        s.abort = 1;
-                        break;
-                    }
-                }
-            }
-            kmax = block_max_u32(s, v, lane, wave);
-            if (s.abort) return false;
-        } else __syncthreads();
-        kmax_row = kmax;
+        if (tid == 0) { s.bc32[3] = 0; s.bc32[4] = 0; }
+        // every workgroup posts its key (never 0 for a finite x) in its own slot
+        if (G > 1 && tid == 0) a_store(&rc->mx[part], kmax_row);
+        __syncthreads();
     }
-    const float xmax = fkey_inv(kmax_row);
-    const float M = __builtin_floorf(xmax);
-
-    // ---- 2. e = 2^(x - M) in place; level-1 histogram ----------------------
+    // ---- 2. e in the slice's own frame; level-1 histogram --------------------
+    // The significand of e does not depend on the frame, so the row's maximum is not needed
+    // yet: bins are kept by absolute octave (mod 128, 4 bins each), where the slices' bins
+    // add up as long as their maxima lie within 87 octaves of each other.  The maxima come
+    // back with the histogram, in the same polling rounds.
+    const float Mloc = __builtin_floorf(fkey_inv(kmax_row));
+    const uint32_t pos0 = G > 1 ? (uint32_t)(int)(Mloc - 128.0f * __builtin_floorf(Mloc * 0.0078125f)) * 4u - 508u : 0u;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) eb[j * 4 + k] = e_bits_of(__uint_as_float(eb[j * 4 + k]), M);
+        for (int k = 0; k < 4; ++k) eb[j * 4 + k] = e_bits_of(__uint_as_float(eb[j * 4 + k]), Mloc);
         if (j < nv) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const uint32_t b = eb[j * 4 + k];
-                lds_hist_add(s, b >> 21, b);
+                lds_hist_add(s, ((b >> 21) + pos0) & 511u, b);
             }
+        }
+    }
+    uint32_t slot_key = kmax_row;
+    if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave, rc->mx, &slot_key)) return false;
+    uint32_t hx = 0;                                     // cluster histogram last summed
+    uint32_t hx_nb = kNB;                                // and its size
+    bool mx_posted = G > 1;                              // my slot is still to be cleared
+    if (G > 1) {
+        // the row's frame, and this slice's distance from it
+        const bool in = (uint32_t)tid < G;
+        const uint32_t kmax = block_max_u32(s, in ? slot_key : 0u, lane, wave);
+        const uint32_t kmin = ~block_max_u32(s, in ? ~slot_key : 0u, lane, wave);
+        const float Mrow = __builtin_floorf(fkey_inv(kmax));
+        const bool mixed = !(Mrow - __builtin_floorf(fkey_inv(kmin)) < 88.0f);
+        const float dd = Mrow - Mloc;
+        const uint32_t delta = dd >= 64.0f ? 64u : (uint32_t)dd;
+        kmax_row = kmax;
+        if (delta) {
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) eb[j * 4 + k] = rebase_bits(eb[j * 4 + k], delta);
+        }
+        if (!mixed) {
+            // bring both histograms into the row's frame: position c holds bin 348 + r,
+            // r = c - pos(M); r >= 164 is below 2^-40 of this frame: clamped, a count only
+            const uint32_t m4 = (uint32_t)(int)(Mrow - 128.0f * __builtin_floorf(Mrow * 0.0078125f)) * 4u;
+            const uint32_t r0 = ((uint32_t)tid + 160u - m4) & 511u, r1 = ((uint32_t)tid + kThreads + 160u - m4) & 511u;
+            const uint64_t g0 = s.g[tid], g1 = s.g[tid + kThreads], h0 = s.hm[tid], h1 = s.hm[tid + kThreads];
+            __syncthreads();
+            s.g[tid] = 0; s.g[tid + kThreads] = 0; s.hm[tid] = 0; s.hm[tid + kThreads] = 0;
+            __syncthreads();
+            uint32_t glow = 0, hlow = 0;
+            if (r0 < 164u) { s.g[kBin0 + r0] = g0; s.hm[kBin0 + r0] = h0; } else { glow += pack_count(g0); hlow += pack_count(h0); }
+            if (r1 < 164u) { s.g[kBin0 + r1] = g1; s.hm[kBin0 + r1] = h1; } else { glow += pack_count(g1); hlow += pack_count(h1); }
+            if (glow) atomicAdd(&s.bc32[3], glow);
+            if (hlow) atomicAdd(&s.bc32[4], hlow);
+            __syncthreads();
+            if (tid == 0) { s.g[kBin0] += (uint64_t)s.bc32[3] << 43; s.hm[kBin0] += (uint64_t)s.bc32[4] << 43; }
+            __syncthreads();
+        } else {
+            // maxima too far apart for the shared octave positions: level 1 again, in the row's
+            // frame, through the spare histogram
+            __syncthreads();
+            lds_hist_zero(s, kNB);
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+                if (j < nv) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t b = opaque(eb[j * 4 + k]);
+                        lds_hist_add(s, b >> 21, b);
+                    }
+                }
+            if (!hist_combine(s, p.hdr, G, rc->h[kLevels], kNB, (uint32_t)p.V, lane, wave)) return false;
+            // every workgroup has read the first histogram and the slots: it published this one after that
+            zero_slice(rc->h[0], kNB, part, G);
+            if (tid == 0) a_store(&rc->mx[part], 0u);
+            mx_posted = false;
+            hx = kLevels;
         }
     }
     if (p.e_bits) {
@@ -548,8 +612,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         for (int j = 0; j < R; ++j)
             if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
     }
-    if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return false;
-    if (G > 1 && tid == 0) a_store(&rc->mx[part], 0u);   // every workgroup has read the maxima by now
+    const float xmax = fkey_inv(kmax_row);
     const uint64_t top_k = (uint64_t)p.top_k;
 
     // ---- 3. radix selection of the threshold -------------------------------
@@ -581,14 +644,18 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
             }
         if (!hist_combine(s, p.hdr, G, rc->h[levels - 1], 128, expect, lane, wave)) return false;
         // every workgroup has finished reading the level above: it published this level after that
-        if (G > 1) zero_slice(rc->h[levels - 2], levels == 2 ? kNB : 128, part, G);
+        if (G > 1) {
+            zero_slice(rc->h[hx], hx_nb, part, G);
+            if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
+            mx_posted = false;
+        }
+        hx = levels - 1; hx_nb = 128;
         f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
         amass += local_mass_above(s, f.bin, kTopN, false, exb, lane, wave);
         mycnt = pack_count(s.hm[f.bin]);
         lo |= f.bin << dsh;
         span = (1u << dsh) - 1u;
     }
-    const uint32_t last_nb = levels == 1 ? kNB : 128;    // bins of the last summed level
 
     // If the undistinguished tokens are few, gather them (bits and index) so
     // that every workgroup can finish alone.  Validity is in the data: a
@@ -643,7 +710,8 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
             }
             if ((uint32_t)tid < G) a_mine = get_mass(w0, w1);
             // every workgroup wrote its entries after it had read the last histogram level
-            zero_slice(rc->h[levels - 1], last_nb, part, G);
+            zero_slice(rc->h[hx], hx_nb, part, G);
+            if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
         } else a_mine = tid == 0 ? amass : (u128)0;
         __syncthreads();
 
@@ -723,7 +791,8 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 if (total == G) break;
                 if (s.abort) return false;
             }
-            zero_slice(rc->h[levels - 1], last_nb, part, G);
+            zero_slice(rc->h[hx], hx_nb, part, G);
+            if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
             before = block_sum_u128(s, (uint32_t)tid < part ? get_mass(w0, w1) : (u128)0, lane, wave);
         }
     }
@@ -888,7 +957,6 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
 //                   than any slice's top_k, or a huge tie) is put on a list,
 //                   and the cluster kernel then runs for the listed rows.
 constexpr int      kSB       = 164;           // level-1 bins in use: indices 348..511
-constexpr uint32_t kBin0     = 348u;          // index of e = 2^-40
 constexpr int      kStashCap = 1280;          // stash entries per slice (at least kStreamK)
 constexpr int      kStreamK  = 1024;          // largest top_k the streaming path takes
 constexpr int      kFinCap   = 4096;          // tokens the finishing workgroup can hold
