@@ -246,11 +246,9 @@ __device__ __forceinline__ void zero_slice(uint64_t *gh, uint32_t nb, uint32_t p
 // bins back until their counts add up to `expected` -- count and value of a
 // contribution arrive in one word, so a complete count means complete data
 // and no arrival counter is needed.  The totals end in s.g.  A cluster of one
-// copies its own.  With `slots`, the same polling rounds also fetch one
-// per-workgroup word each (thread t takes slot t) and go on until none of
-// them is 0.  Returns false when the wait gave up.
+// copies its own.  Returns false when the wait gave up.
 __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, uint64_t *gh, int nb, uint32_t expected,
-                                             int lane, int wave, const uint32_t *slots = nullptr, uint32_t *slot_value = nullptr)
+                                             int lane, int wave)
 {
     __syncthreads();
     if (G == 1) {
@@ -271,17 +269,73 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
             s.g[b] = w;
             c += pack_count(w);
         }
-        if (slots && threadIdx.x < G) {
-            // thread t also waits for slot t (never 0 once written); a missing slot spoils the sum
-            const uint32_t v = a_load(&slots[threadIdx.x]);
-            *slot_value = v;
-            c += v == 0u ? 1u << 24 : 0u;
-        }
         guard.tick(s, hdr);
         const uint32_t total = block_sum_u32(s, c, lane, wave);
         if (total == expected) return true;
         if (s.abort) return false;
     }
+}
+
+// Level 1 of a cluster of several workgroups.  s.hm holds this slice's bins by
+// absolute octave position; they are added to the row's (gh) and the row's are
+// polled until complete, together with the slots of the slice maxima (thread t
+// takes slot t).  Once all is there the row's frame M = floor(max) is known,
+// and both histograms are stored in that frame: position c holds bin 348 + r,
+// r = c - pos(M) mod 512; r >= 164 lies below 2^-40 of the frame, where
+// tokens are clamped: their count goes to bin 348, without fraction bits.
+// Indices below 348 of s.g and s.hm are left stale.  Returns 0 on success, 1
+// when the slices' maxima are too far apart for shared positions (s.g and
+// s.hm are then undefined), -1 when the wait gave up.
+__device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G, uint64_t *gh, const uint32_t *slots,
+                                              uint32_t expected, uint32_t &kmax_out, int lane, int wave)
+{
+    const int tid = threadIdx.x;
+    __syncthreads();
+    const uint64_t h0 = s.hm[tid], h1 = s.hm[tid + kThreads];
+    if (h0) a_add(&gh[tid], h0);
+    if (h1) a_add(&gh[tid + kThreads], h1);
+    uint64_t g0, g1;
+    uint32_t kmax, kmin;
+    SpinGuard guard;
+    guard.start();
+    for (;;) {
+        g0 = a_load(&gh[tid]); g1 = a_load(&gh[tid + kThreads]);
+        uint32_t c = pack_count(g0) + pack_count(g1);
+        uint32_t key = 0, nkey = 0;
+        if ((uint32_t)tid < G) {
+            key = a_load(&slots[tid]);                   // never 0 once written; a missing slot spoils the sum
+            nkey = ~key;
+            c += key == 0u ? 1u << 24 : 0u;
+        }
+        guard.tick(s, hdr);
+        c = wave_sum(c); key = wave_max_u32(key); nkey = wave_max_u32(nkey);
+        __syncthreads();
+        if (lane == 0) { s.u32[wave] = c; s.u32[kWaves + wave] = key; s.u32[2 * kWaves + wave] = nkey; }
+        __syncthreads();
+        uint32_t total = 0;
+        kmax = 0; kmin = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            total += s.u32[w]; kmax = max(kmax, s.u32[kWaves + w]); kmin = max(kmin, s.u32[2 * kWaves + w]);
+        }
+        if (total == expected) break;
+        if (s.abort) return -1;
+    }
+    kmin = ~kmin;
+    kmax_out = kmax;
+    const float M = __builtin_floorf(fkey_inv(kmax));
+    if (!(M - __builtin_floorf(fkey_inv(kmin)) < 88.0f)) return 1;
+    const uint32_t m4 = (uint32_t)(int)(M - 128.0f * __builtin_floorf(M * 0.0078125f)) * 4u;
+    const uint32_t r0 = ((uint32_t)tid + 160u - m4) & 511u, r1 = ((uint32_t)tid + kThreads + 160u - m4) & 511u;
+    uint32_t glow = 0, hlow = 0;
+    if (r0 < 164u) { s.g[kBin0 + r0] = g0; s.hm[kBin0 + r0] = h0; } else { glow += pack_count(g0); hlow += pack_count(h0); }
+    if (r1 < 164u) { s.g[kBin0 + r1] = g1; s.hm[kBin0 + r1] = h1; } else { glow += pack_count(g1); hlow += pack_count(h1); }
+    if (glow) atomicAdd(&s.bc32[3], glow);
+    if (hlow) atomicAdd(&s.bc32[4], hlow);
+    __syncthreads();
+    if (tid == 0) { s.g[kBin0] += (uint64_t)s.bc32[3] << 43; s.hm[kBin0] += (uint64_t)s.bc32[4] << 43; }
+    __syncthreads();
+    return 0;
 }
 
 // Scan s.g from index `top` downwards (largest e first) and find the first
@@ -298,9 +352,9 @@ __device__ __forceinline__ Found hist_find512(Lds &s, uint64_t top_k, float top_
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const uint32_t idx = kTop1 - (uint32_t)(t * PER + i);
-        const uint64_t w = s.g[idx];
+        const uint64_t w = idx >= kBin0 ? s.g[idx] : 0ull;  // nothing lives below 2^-40 (what s.g holds there is stale)
         c[i] = pack_count(w);
-        m[i] = w ? pack_mass(w, idx >> 2) : (u128)0;       // empty bins below 2^-40 have no valid exponent
+        m[i] = w ? pack_mass(w, idx >> 2) : (u128)0;
         cs += c[i]; ms += m[i];
     }
     // inclusive scan over threads
@@ -545,45 +599,24 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
             }
         }
     }
-    uint32_t slot_key = kmax_row;
-    if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave, rc->mx, &slot_key)) return false;
     uint32_t hx = 0;                                     // cluster histogram last summed
     uint32_t hx_nb = kNB;                                // and its size
     bool mx_posted = G > 1;                              // my slot is still to be cleared
-    if (G > 1) {
+    if (G == 1) {
+        if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return false;
+    } else {
+        const int st = combine_level1(s, p.hdr, G, rc->h[0], rc->mx, (uint32_t)p.V, kmax_row, lane, wave);
+        if (st < 0) return false;
         // the row's frame, and this slice's distance from it
-        const bool in = (uint32_t)tid < G;
-        const uint32_t kmax = block_max_u32(s, in ? slot_key : 0u, lane, wave);
-        const uint32_t kmin = ~block_max_u32(s, in ? ~slot_key : 0u, lane, wave);
-        const float Mrow = __builtin_floorf(fkey_inv(kmax));
-        const bool mixed = !(Mrow - __builtin_floorf(fkey_inv(kmin)) < 88.0f);
-        const float dd = Mrow - Mloc;
+        const float dd = __builtin_floorf(fkey_inv(kmax_row)) - Mloc;
         const uint32_t delta = dd >= 64.0f ? 64u : (uint32_t)dd;
-        kmax_row = kmax;
         if (delta) {
 #pragma unroll
             for (int j = 0; j < R; ++j)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) eb[j * 4 + k] = rebase_bits(eb[j * 4 + k], delta);
         }
-        if (!mixed) {
-            // bring both histograms into the row's frame: position c holds bin 348 + r,
-            // r = c - pos(M); r >= 164 is below 2^-40 of this frame: clamped, a count only
-            const uint32_t m4 = (uint32_t)(int)(Mrow - 128.0f * __builtin_floorf(Mrow * 0.0078125f)) * 4u;
-            const uint32_t r0 = ((uint32_t)tid + 160u - m4) & 511u, r1 = ((uint32_t)tid + kThreads + 160u - m4) & 511u;
-            const uint64_t g0 = s.g[tid], g1 = s.g[tid + kThreads], h0 = s.hm[tid], h1 = s.hm[tid + kThreads];
-            __syncthreads();
-            s.g[tid] = 0; s.g[tid + kThreads] = 0; s.hm[tid] = 0; s.hm[tid + kThreads] = 0;
-            __syncthreads();
-            uint32_t glow = 0, hlow = 0;
-            if (r0 < 164u) { s.g[kBin0 + r0] = g0; s.hm[kBin0 + r0] = h0; } else { glow += pack_count(g0); hlow += pack_count(h0); }
-            if (r1 < 164u) { s.g[kBin0 + r1] = g1; s.hm[kBin0 + r1] = h1; } else { glow += pack_count(g1); hlow += pack_count(h1); }
-            if (glow) atomicAdd(&s.bc32[3], glow);
-            if (hlow) atomicAdd(&s.bc32[4], hlow);
-            __syncthreads();
-            if (tid == 0) { s.g[kBin0] += (uint64_t)s.bc32[3] << 43; s.hm[kBin0] += (uint64_t)s.bc32[4] << 43; }
-            __syncthreads();
-        } else {
+        if (st == 1) {
             // maxima too far apart for the shared octave positions: level 1 again, in the row's
             // frame, through the spare histogram
             __syncthreads();
