@@ -196,6 +196,48 @@ def test_streaming_path_mixed_rows(torch_cuda, oracle):
         os.environ.pop("RS_FORCE_PATH", None)
 
 
+def test_c5_full_size_paths_agree(torch_cuda, oracle):
+    """BASELINE config 5 at its full size, (B,T,V) = (128,4,1048576) fp32 = 2 GiB, top_k 1024, top_p 0.95.
+    Too large for the oracle in a test; checked through what does not depend on size: the streaming path
+    and the cluster path are different decompositions of the same integer arithmetic, so every diagnostic
+    and every index must be equal; the sampled token must lie in the kept set; 8 of the rows are also run
+    through the oracle."""
+    torch = torch_cuda
+    from tests import capi
+    B, T, V = 128, 4, 1048576
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    lg = torch.randn((B, T, V), generator=g, device="cuda", dtype=torch.float32) * 1.5
+    rc, c, k, p = capi.normalize(1.0, 1024, 0.95, V, B, T)
+    u = torch.from_numpy(H.uniforms(B, 123)).cuda()
+    smp = capi.Sampler(B, V)
+    res = {}
+    try:
+        for path in ("stream", "cluster", "stream"):
+            os.environ["RS_FORCE_PATH"] = path
+            print("full C5", path, flush=True)
+            r = smp.sample(lg, c, k, p, uniforms=u)
+            assert r["rc"] == 0 and smp.status() == 0
+            if path in res:
+                for f in FIELDS:
+                    assert np.array_equal(res[path]["diag"][f], r["diag"][f]), "repeat differs: " + f
+            res[path] = r
+    finally:
+        os.environ.pop("RS_FORCE_PATH", None)
+    for f in FIELDS:
+        assert np.array_equal(res["stream"]["diag"][f], res["cluster"]["diag"][f]), f
+    assert np.array_equal(res["stream"]["out"], res["cluster"]["out"])
+    assert (res["stream"]["diag"]["rounds"] == 0).all()            # every row finished by the streaming path
+    d = res["stream"]["diag"]
+    assert (d["n_gt"] < 1024).all() and (d["n_gt"] + d["n_eq"] >= 1).all()
+    rows = [0, 1, 17, 63, 64, 100, 126, 127]
+    sub = lg[rows, T - 1, :].cpu().numpy()
+    ref_out, ref_diag = oracle.sample_batch(sub, c, k, p, injected_u=H.uniforms(B, 123)[rows])
+    for f in FIELDS:
+        assert np.array_equal(d[f][rows], ref_diag[f]), f
+    assert np.array_equal(res["stream"]["out"][rows], ref_out)
+
+
 def test_penalty_path_single_step(torch_cuda, oracle):
     from tests import capi
     B, V = 8, 32768
