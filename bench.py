@@ -15,7 +15,9 @@ stream the kernel runs on).  Next to it, in the same JSON line:
              reference's own bench measures (reference bench.py:84-92)
   roofline   the bandwidth-bound configuration (BASELINE.json configs[4]):
              logits (128,4,1048576) fp32 = 2 GiB resident, top_k 1024,
-             top_p 0.95; algorithmic bytes = 4*V per sampled row
+             top_p 0.95; algorithmic bytes = 4*V per sampled row; the time
+             is that of the whole call (its three launches), averaged over
+             back-to-back calls between two HIP events
   cpu_baseline  the CPU oracle (single thread) on a bounded sample of the
              headline workload; cpu_torch is torch-CPU softmax/sort/cumsum/
              multinomial on the same row with its thread count
@@ -221,6 +223,11 @@ def main():
         t_btv = block_time_us(torch, call_btv, args.bandwidth_steps, 3)
         t_flat = block_time_us(torch, call_flat, max(2, args.bandwidth_steps // 2), 2)
         t_floor = block_time_us(torch, floor_btv, args.bandwidth_steps, 3)
+        os.environ["RS_FORCE_PATH"] = "cluster"          # the general single-launch kernel on the same input
+        try:
+            t_cluster = block_time_us(torch, call_btv, max(2, args.bandwidth_steps // 2), 2)
+        finally:
+            del os.environ["RS_FORCE_PATH"]
         bytes_btv = Bb * Vb * 4
         bytes_flat = Bb * Tb * Vb * 4
         ach = bytes_btv / (t_btv * 1e-6) / 1e9
@@ -230,6 +237,9 @@ def main():
             "workload": "(B,T,V)=(128,4,1048576) N(0,1.5), top_k 1024, top_p 0.95: 128 sampled rows of 4 MiB, "
                         "stride T*V, algorithmic bytes 4*V per row = 512 MiB per call",
             "us_per_call": round(t_btv, 2), "rows_per_s": round(Bb / (t_btv * 1e-6), 1),
+            "kernels": "streaming path, three launches per call: rs::stream_kernel (reads the logits; dominant), "
+                       "rs::finish_kernel, rs::sample_list_kernel; achieved = bytes / time of the whole call",
+            "cluster_path_us_per_call": round(t_cluster, 2),
             "read_once_floor_GBs": round(bytes_btv / (t_floor * 1e-6) / 1e9, 1),
             "flattened_512_rows": {"us_per_call": round(t_flat, 2),
                                    "achieved": round(bytes_flat / (t_flat * 1e-6) / 1e9, 1),

