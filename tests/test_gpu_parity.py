@@ -301,6 +301,56 @@ def test_philox_stream_matches_oracle(torch_cuda, oracle):
     assert np.array_equal(st.cpu().numpy().view(np.uint32).reshape(B, 16), rng_ref)
 
 
+@pytest.mark.parametrize("path,pen_on", [("cluster", False), ("cluster", True), ("stream", False)])
+def test_hip_graph_decode_loop(torch_cuda, oracle, path, pen_on):
+    """A sampling call captured into a HIP graph (rs_sample records only kernel launches: no memset,
+    no allocation, no synchronisation) and replayed as a decode loop: every replay draws the next Philox
+    number and, with penalties, continues from the penalties the previous replay left.  Each replay is
+    checked against the oracle, with eager work and synchronisations between replays."""
+    torch = torch_cuda
+    from tests import capi
+    B, V, replays = 6, 65536 + 4096, 6
+    lg_np = H.logits_normal(B, V, 2.0, seed=70)
+    pen_ref = H.penalties_sparse(B, V, seed=71) if pen_on else None
+    rc, c, k, p = capi.normalize(0.9, 40, 0.9, V, B, 1)
+    smp = capi.Sampler(B, V)
+    lg = torch.from_numpy(lg_np).cuda()
+    pen = torch.from_numpy(pen_ref.copy()).cuda() if pen_on else None
+    out = torch.full((B,), -1, dtype=torch.int32, device="cuda")
+    hist = torch.zeros((B,), dtype=torch.int64, device="cuda")
+    st = torch.empty(B * 64, dtype=torch.int8, device="cuda")
+    assert capi.lib().rs_philox_init(st.data_ptr(), 99, B, smp.stream()) == 0
+    rng_ref = oracle.rng_init(99, B)
+    torch.cuda.synchronize()
+    os.environ["RS_FORCE_PATH"] = path
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rc = capi.lib().rs_sample(lg.data_ptr(), V, pen.data_ptr() if pen_on else None, out.data_ptr(),
+                                      st.data_ptr(), None, B, V, 0.1, 0.2, 0.9, c, k, p,
+                                      smp.ws.data_ptr(), smp.ws.numel(), None, None, smp.stream())
+            hist += out                                   # a consumer of the sampled ids inside the graph
+        assert rc == 0
+    finally:
+        os.environ.pop("RS_FORCE_PATH", None)
+    total = np.zeros(B, dtype=np.int64)
+    for i in range(replays):
+        ref_out, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref, penalties=pen_ref,
+                                         presence=0.1, repetition=0.2, decay=0.9)
+        print("graph replay", i, path, pen_on, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), ref_out), "replay %d" % i
+        total += ref_out
+        scratch = torch.randn(1 << 20, device="cuda").sum().item()      # eager work between replays
+        assert scratch == scratch
+    assert np.array_equal(hist.cpu().numpy(), total)
+    assert np.array_equal(st.cpu().numpy().view(np.uint32).reshape(B, 16), rng_ref)
+    if pen_on:
+        assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32))
+    assert smp.status() == 0
+
+
 def test_chi_square_one_million_draws(torch_cuda, oracle):
     """1,048,576 Philox-driven draws of one row against the exact renormalised weights w_i / S."""
     torch = torch_cuda
