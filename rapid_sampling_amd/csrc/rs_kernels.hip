@@ -1464,14 +1464,20 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
         if ((R == 1 || R == 2 || R == 4 || R == 8 || R == 16 || R == 32) && R <= maxR && parts(R) <= (uint32_t)kMaxParts)
             return {R, parts(R)};
     }
-    const uint64_t want[2] = {512, 64};
-    for (uint64_t w : want)
-        for (int R = maxR; R >= 1; R /= 2)
-            if (parts(R) <= (uint32_t)kMaxParts && (uint64_t)B * parts(R) >= w) return {R, parts(R)};
+    // Measured on MI355X: a cluster works best with at most ~64 workgroups (each exchange costs
+    // more the more peers poll), slices of 32 float4 per thread only pay for rows of a quarter
+    // million tokens and more (the variant spills), and a call wants a few hundred workgroups in
+    // flight -- 256 for small batches, where latency counts, 512 beyond.
+    int minR = maxR;
     for (int R = 1; R <= maxR; R *= 2)
-        if (parts(R) <= (uint32_t)kMaxParts) return {R, parts(R)};
-    return {maxR, parts(maxR)};
+        if (parts(R) <= 64u) { minR = R; break; }
+    const int topR = (V4 >= 65536u || minR > 16) ? maxR : (maxR < 16 ? maxR : 16);
+    const uint64_t want = B <= 16 ? 256 : 512;
+    for (int R = topR; R >= minR; R /= 2)
+        if ((uint64_t)B * parts(R) >= want) return {R, parts(R)};
+    return {minR, parts(minR)};
 }
+
 
 // Streaming geometry: workgroups of 256 threads with 16 float4 each: slices of 16384 tokens.
 constexpr int kStreamR = 16, kStreamNT = 256, kStreamSliceLog2 = 14;
