@@ -147,6 +147,7 @@ __device__ __forceinline__ uint32_t rebase_bits(uint32_t b, uint32_t delta)
 
 struct Found {               // result of a histogram scan (uniform over the workgroup)
     u128     mass_above;
+    u128     local_above;    // level 1 only: mass of this workgroup's own tokens above the bin
     uint32_t bin;            // index of the first bin (largest e first) at which the kept set becomes sufficient
     uint32_t cnt_above;      // tokens in bins before it (plus the carried offset)
     uint32_t cnt_bin;        // tokens in it
@@ -348,55 +349,57 @@ __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G,
     return 0;
 }
 
-// Scan s.g from index `top` downwards (largest e first) and find the first
-// bin at which (cnt0 + count so far >= top_k) or (mass0 + mass so far >= P).
-// With `first` the total mass of the histogram is the row total D and P is
-// derived from it here.  Thread t owns digits 2t and 2t+1 (index = top -
-// digit); the exponent of level-1 bin idx is idx >> 2.
-__device__ __forceinline__ Found hist_find512(Lds &s, uint64_t top_k, float top_p, int lane, int wave)
+// Scan the level-1 histogram s.g from the top (index 511, largest e) down to
+// index 348 (e = 2^-40) and find the first bin at which (count so far >=
+// top_k) or (mass so far >= P).  The total mass of the histogram is the row
+// total D, and P = ceil(top_p * D) is derived from it here.  The 164 bins fit
+// one wave (lane l owns indices 511-3l, 510-3l, 509-3l), so the scan needs no
+// LDS exchange; the exponent of bin idx is idx >> 2.  With LOCAL the wave also
+// scans this workgroup's own histogram s.hm and returns its mass above the
+// boundary bin in local_above.
+template <bool LOCAL>
+__device__ __forceinline__ Found hist_find_level1(Lds &s, uint64_t top_k, float top_p, int lane, int wave)
 {
-    constexpr int PER = kNB / kThreads;
-    const int t = threadIdx.x;
-    uint32_t c[PER]; u128 m[PER];
-    uint32_t cs = 0; u128 ms = 0;
+    if (wave == 0) {
+        uint32_t c[3]; u128 m[3], hl[3];
+        uint32_t cs = 0; u128 ms = 0, hs = 0;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-        const uint32_t idx = kTop1 - (uint32_t)(t * PER + i);
-        const uint64_t w = idx >= kBin0 ? s.g[idx] : 0ull;  // nothing lives below 2^-40 (what s.g holds there is stale)
-        c[i] = pack_count(w);
-        m[i] = w ? pack_mass(w, idx >> 2) : (u128)0;
-        cs += c[i]; ms += m[i];
-    }
-    // inclusive scan over threads
-    const u128 mi = wave_inclusive_scan(ms);
-    const uint32_t ci = wave_inclusive_scan(cs);
-    __syncthreads();
-    if (lane == kWave - 1) { s.q128[wave] = mi; s.u32[wave] = ci; }
-    __syncthreads();
-    u128 moff = 0, mtot = 0;
-    uint32_t coff = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-        if (w < wave) { moff += s.q128[w]; coff += s.u32[w]; }
-        mtot += s.q128[w];
-    }
-    if (t == 0) { s.D = mtot; s.P = ceil_mul(top_p, mtot); }
-    __syncthreads();
-    const u128 P = s.P;
-    uint64_t rcnt = (uint64_t)coff + ci - cs;            // count before my first bin
-    u128 rm = moff + mi - ms;                            // mass before my first bin
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-        const bool before = rcnt >= top_k || rm >= P;
-        const uint64_t nc = rcnt + c[i];
-        const u128 nm = rm + m[i];
-        const bool after = nc >= top_k || nm >= P;
-        if (!before && after) {
-            s.found.bin = kTop1 - (uint32_t)(t * PER + i);
-            s.found.cnt_above = (uint32_t)rcnt; s.found.cnt_bin = c[i];
-            s.found.mass_above = rm;
+        for (int i = 0; i < 3; ++i) {
+            const int idx = (int)kTop1 - 3 * lane - i;
+            const uint64_t w = idx >= (int)kBin0 ? s.g[idx] : 0ull;
+            c[i] = pack_count(w);
+            m[i] = w ? pack_mass(w, (uint32_t)idx >> 2) : (u128)0;
+            cs += c[i]; ms += m[i];
+            if (LOCAL) {
+                const uint64_t h = idx >= (int)kBin0 ? s.hm[idx] : 0ull;
+                hl[i] = h ? pack_mass(h, (uint32_t)idx >> 2) : (u128)0;
+                hs += hl[i];
+            }
         }
-        rcnt = nc; rm = nm;
+        const u128 mi = wave_inclusive_scan(ms);
+        const uint32_t ci = wave_inclusive_scan(cs);
+        u128 hrun = 0;
+        if (LOCAL) hrun = wave_inclusive_scan(hs) - hs;
+        const u128 D = lane63(mi);
+        const u128 P = ceil_mul(top_p, D);
+        if (lane == 0) { s.D = D; s.P = P; }
+        uint64_t rcnt = (uint64_t)ci - cs;               // count before my first bin
+        u128 rm = mi - ms;                               // mass before my first bin
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const bool before = rcnt >= top_k || rm >= P;
+            const uint64_t nc = rcnt + c[i];
+            const u128 nm = rm + m[i];
+            const bool after = nc >= top_k || nm >= P;
+            if (!before && after) {
+                s.found.bin = kTop1 - (uint32_t)(3 * lane + i);
+                s.found.cnt_above = (uint32_t)rcnt; s.found.cnt_bin = c[i];
+                s.found.mass_above = rm;
+                s.found.local_above = hrun;
+            }
+            rcnt = nc; rm = nm;
+            if (LOCAL) hrun += hl[i];
+        }
     }
     __syncthreads();
     return s.found;
@@ -659,11 +662,11 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
     const uint64_t top_k = (uint64_t)p.top_k;
 
     // ---- 3. radix selection of the threshold -------------------------------
-    Found f = hist_find512(s, top_k, p.top_p, lane, wave);
+    Found f = hist_find_level1<true>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
     const uint32_t exb = f.bin >> 2;                     // exponent of every token still in play
     // my own tokens: mass in the bins above the boundary, count in the boundary bin
-    u128 amass = local_mass_above(s, f.bin, kTop1, true, 0u, lane, wave);
+    u128 amass = f.local_above;
     uint32_t mycnt = pack_count(s.hm[f.bin]);
     // bit patterns of the tokens still undistinguished: [lo, lo + span]
     uint32_t lo = f.bin << 21;
@@ -758,8 +761,9 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         } else a_mine = tid == 0 ? amass : (u128)0;
         __syncthreads();
 
-        // resolve the remaining digits on the gathered tokens, in LDS
-        for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels; ++lv) {
+        // resolve the remaining digits on the gathered tokens, in LDS; a single token left in
+        // the range is the threshold itself
+        for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels && f.cnt_bin > 1u; ++lv) {
             const uint32_t dsh = level_shift(lv);
             lds_hist_zero(s, 128);
             __syncthreads();
@@ -771,6 +775,14 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
             f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
             lo |= f.bin << dsh;
             span = (1u << dsh) - 1u;
+        }
+        if (span != 0u) {
+            for (uint32_t i = tid; i < ncand; i += kThreads) {
+                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
+                if (b - lo <= span) s.bc32[6] = b;
+            }
+            __syncthreads();
+            lo = s.bc32[6];
         }
     }
     // every digit is known: the threshold is the one value left in [lo, lo + span]
@@ -1279,7 +1291,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     }
     __syncthreads();
     const uint64_t top_k = (uint64_t)p.top_k;
-    Found f = hist_find512(s, top_k, p.top_p, lane, wave);
+    Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
     const uint32_t exb = f.bin >> 2;
 
@@ -1348,7 +1360,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
 
     // remaining digits of the threshold, on the gathered tokens
     uint32_t lo = f.bin << 21, span = (1u << 21) - 1u;
-    for (uint32_t lv = 2; lv <= (uint32_t)kLevels; ++lv) {
+    for (uint32_t lv = 2; lv <= (uint32_t)kLevels && f.cnt_bin > 1u; ++lv) {
         const uint32_t dsh = level_shift(lv);
         lds_hist_zero(s, 128);
         __syncthreads();
@@ -1360,6 +1372,14 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
         f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
         lo |= f.bin << dsh;
         span = (1u << dsh) - 1u;
+    }
+    if (span != 0u) {                                    // a single token left in the range: the threshold itself
+        for (uint32_t i = tid; i < total; i += kThreads) {
+            const uint32_t b = (uint32_t)(t.list[i] >> 32);
+            if (b - lo <= span) s.bc32[6] = b;
+        }
+        __syncthreads();
+        lo = s.bc32[6];
     }
     const uint32_t thr = lo;
     if (tid == 0) {
