@@ -18,6 +18,7 @@ stream the kernel runs on).  Next to it, in the same JSON line:
              top_p 0.95; algorithmic bytes = 4*V per sampled row; the time
              is that of the whole call (its three launches), averaged over
              back-to-back calls between two HIP events
+  configs    time per call and rows/s of the other BASELINE configurations
   cpu_baseline  the CPU oracle (single thread) on a bounded sample of the
              headline workload; cpu_torch is torch-CPU softmax/sort/cumsum/
              multinomial on the same row with its thread count
@@ -233,7 +234,10 @@ def main():
         ach = bytes_btv / (t_btv * 1e-6) / 1e9
         result["roofline"] = {
             "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(ach / HBM_PEAK_GBS, 4),
+            # HBM bytes per call from the FETCH_SIZE / WRITE_SIZE counter runs of this same command
+            # (profiles/bench_kernels_hbm_traffic_pmc.md), not measured live
+            "traffic": 562926592,
             "workload": "(B,T,V)=(128,4,1048576) N(0,1.5), top_k 1024, top_p 0.95: 128 sampled rows of 4 MiB, "
                         "stride T*V, algorithmic bytes 4*V per row = 512 MiB per call",
             "us_per_call": round(t_btv, 2), "rows_per_s": round(Bb / (t_btv * 1e-6), 1),
@@ -252,6 +256,39 @@ def main():
             torch.cuda.synchronize()
             del dst
         del big, flat
+
+    # ---- the other BASELINE configurations (parity cases; time and rows/s only) ----
+    def timed_rows(fn, B, steps=200):
+        t = block_time_us(torch, fn, steps, 10)
+        return {"us_per_call": round(t, 2), "rows_per_s": round(B / (t * 1e-6), 1)}
+
+    g1 = torch.Generator(device=dev)
+    g1.manual_seed(0)
+    c1 = torch.rand((1, 131072), generator=g1, device=dev)
+    st1 = sample.setup_rand(0, 1)
+    g3 = torch.Generator(device=dev)
+    g3.manual_seed(4)
+    c3 = torch.randn((64, 152064), generator=g3, device=dev) * 2.0
+    c3.scatter_add_(1, torch.randint(0, 152064, (64, 16), generator=g3, device=dev),
+                    torch.full((64, 16), 10.0, device=dev))
+    st3 = sample.setup_rand(3, 64)
+    g4 = torch.Generator(device=dev)
+    g4.manual_seed(40)
+    c4 = torch.randn((32, 131072), generator=g4, device=dev) * 1.5
+    pen4 = torch.where(torch.rand((32, 131072), generator=g4, device=dev) < 0.02,
+                       torch.empty((32, 131072), device=dev).exponential_(1.0, generator=g4),
+                       torch.zeros((), device=dev))
+    st4 = sample.setup_rand(4, 32)
+    result["configs"] = {
+        "C1 B=1 V=131072 U[0,1) top_p 0.5": timed_rows(
+            lambda: sample.batch_sampling_temperature_topk_topp(c1, st1, 1.0, -1, 0.5), 1),
+        "C3 B=64 V=152064 N(0,2)+spikes T 0.8 top_k 50 top_p 0.9": timed_rows(
+            lambda: sample.batch_sampling_temperature_topk_topp(c3, st3, 0.8, 50, 0.9), 64),
+        "C4 B=32 V=131072 penalties, 256 chained calls on fixed logits": timed_rows(
+            lambda: sample.batch_sampling_repetition_temperature_topk_topp(c4, pen4, st4, 0.1, 0.1, 0.95,
+                                                                           0.8, 50, 0.9), 32, steps=256),
+    }
+    del c1, c3, c4, pen4
 
     # ---- CPU baselines ------------------------------------------------------
     if not args.skip_cpu:

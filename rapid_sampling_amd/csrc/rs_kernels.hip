@@ -960,15 +960,25 @@ template <int R, bool PEN>
 __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
 {
     __shared__ Lds s;
+    if (p.G == 1) {
+        // one workgroup per row: nobody waits for anybody, the hardware's ids will do
+        if (threadIdx.x == 0) s.abort = 0;
+        __syncthreads();
+        sample_slice<R, PEN>(p, s, blockIdx.x, 0u);
+        return;
+    }
     if (threadIdx.x == 0) {
         s.abort = 0;
-        s.bc32[0] = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        // every workgroup of the launch takes exactly one ticket: after the last one the counter
+        // is not touched again, and is put back for the next call
+        if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);
+        s.bc32[0] = t;
     }
     __syncthreads();
     const uint32_t ticket = s.bc32[0];
     const uint32_t row = ticket / p.G;
-    if (!sample_slice<R, PEN>(p, s, row, ticket - row * p.G)) return;
-    leave_launch(p.hdr);
+    sample_slice<R, PEN>(p, s, row, ticket - row * p.G);
 }
 
 // The launch that follows the streaming pass: workgroups work through the
