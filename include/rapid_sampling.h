@@ -82,6 +82,11 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
  * streaming path, about 0.7 bytes per token (stashes of the largest tokens
  * of each slice of 16384 tokens); under a fifth of the reference's scratch
  * for large V.  It does not grow with T.
+ *
+ * One workspace may serve calls of different shapes if it is at least
+ * rs_workspace_bytes(largest B, largest V) of those calls and the same
+ * (pointer, size) pair is passed every time: per-row records are addressed from
+ * its end, per-slice data from its front.
  */
 int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes);
 

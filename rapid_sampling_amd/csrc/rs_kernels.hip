@@ -60,7 +60,13 @@ struct alignas(256) WsHeader {
 };
 
 // Per-row record.  Everything a call reads before writing it is zero when the
-// call starts: the call itself re-zeroes what it used before it ends.
+// call starts: the call itself re-zeroes what it used before it ends.  The
+// records sit at the END of the workspace, row r at ctl_end[-1 - r], so that
+// a row's record is at the same address whatever B and V a call has; the
+// streaming path's per-slice data, which is written before it is read and
+// never cleaned, grows from the front.  The two do not meet as long as the
+// workspace is at least rs_workspace_bytes(largest B, largest V) of the calls
+// that share it.
 struct alignas(256) RowCtl {
     uint32_t unused0;
     uint32_t done;        // workgroups finished with this row
@@ -72,6 +78,7 @@ struct alignas(256) RowCtl {
     uint64_t A[2 * kMaxParts];  // per workgroup: a 124-bit mass as two words of 62 bits, each | kValid
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
     uint64_t h[kLevels + 1][kNB];   // cluster histograms, packed (see kPackOne); one spare for the re-framed level 1
+    uint64_t rowhist[kNB];          // streaming path: the row's bins by absolute octave (mod 128), summed over its slices
 };
 
 struct Params {
@@ -83,7 +90,7 @@ struct Params {
     rs_row_diag *diag;         // or null
     uint32_t    *e_bits;       // or null
     WsHeader    *hdr;
-    RowCtl      *ctl;
+    RowCtl      *ctl_end;      // one past the record of row 0; row r is ctl_end[-1 - r]
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
     int64_t      row_stride;
@@ -524,7 +531,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         philox4x32_10(st[2], st[3], st[4], st[5], st[0], st[1], o);
         s.bc64[5] = ((uint64_t)o[0] << 32) | o[1];
     }
-    RowCtl *rc = p.ctl + row;
+    RowCtl *rc = p.ctl_end - 1 - row;
 
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const uint32_t base4 = part * (uint32_t)(kThreads * R) + (uint32_t)tid;
@@ -1035,8 +1042,6 @@ struct PartHdr {
 
 struct StreamView {
     PartHdr  *hdr;        // [B][G]
-    uint64_t *rowhist;    // [B][512]  packed bins by absolute octave mod 128, summed over the row's slices with
-                          //           device atomics; zero between calls
     uint64_t *stash;      // [B][G][kStashCap]   bits(e, slice frame) << 32 | index, by descending bin
     uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
     uint32_t *need;       // [B]  rows left to the cluster kernel
@@ -1123,7 +1128,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     if (tid < kSB) {
         const uint64_t w = s.hm[tid];
         const float mm = M - 128.0f * __builtin_floorf(M * 0.0078125f);          // M mod 128, exact
-        if (w) a_add(&v.rowhist[(size_t)row * kNB + (((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u)], w);
+        if (w) a_add(&(p.ctl_end - 1 - row)->rowhist[((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u], w);
     }
 
     // What to stash: the bins from the top down to the first one at which the count reaches
@@ -1265,7 +1270,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t G = v.G, row = blockIdx.x;
     const PartHdr *hdrs = v.hdr + (size_t)row * G;
-    uint64_t *rowhist = v.rowhist + (size_t)row * kNB;
+    uint64_t *rowhist = (p.ctl_end - 1 - row)->rowhist;
 
     if (tid == 0) { s.abort = 0; t.fail = 0; s.ctr = 0; }
     PartHdr ph;
@@ -1514,30 +1519,33 @@ constexpr int kStreamR = 16, kStreamNT = 256, kStreamSliceLog2 = 14;
 static_assert(kStreamR * kStreamNT * 4 == 1 << kStreamSliceLog2, "slice size");
 static uint32_t stream_parts(int32_t V) { return ((uint32_t)V / 4 + kStreamNT * kStreamR - 1) / (kStreamNT * kStreamR); }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-struct StreamLayout { size_t hdr, hist, cum, stash, need, end; };
+struct StreamLayout { size_t hdr, cum, stash, need, end; };
 static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
 {
     const size_t parts = (size_t)B * stream_parts(V);
     StreamLayout l;
     l.hdr = align256(base);
-    l.hist = align256(l.hdr + parts * sizeof(PartHdr));
-    l.cum = align256(l.hist + (size_t)B * kNB * sizeof(uint64_t));
+    l.cum = align256(l.hdr + parts * sizeof(PartHdr));
     l.stash = align256(l.cum + parts * kSB * sizeof(uint32_t));
     l.need = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
     l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
     return l;
 }
 
-// The streaming path (three launches, no waits) pays off when a call moves a
-// few hundred MB and top_k bounds the kept set; below that the single launch
-// of the cluster kernel wins.  RS_FORCE_PATH=cluster|stream overrides (tests).
+// The streaming path (three launches, no waits) needs top_k to bound the kept
+// set.  Measured on MI355X it then matches or beats the cluster kernel from
+// about half a million tokens per call upwards (back to back: 18-19 us for
+// small calls against 17-29 us, 2-3 times faster for large ones); below that
+// the single launch wins by a microsecond.  RS_FORCE_PATH=cluster|stream
+// overrides (tests).
 static bool choose_stream(int32_t B, int32_t V, int32_t top_k, bool pen, bool want_e, const Geometry &g)
 {
     const bool eligible = !pen && !want_e && top_k <= kStreamK;
     const char *force = getenv("RS_FORCE_PATH");
     if (force && force[0] == 'c') return false;
     if (force && force[0] == 's') return eligible;
-    return eligible && g.G >= 4 && (uint64_t)B * (uint64_t)V >= (1ull << 25);
+    (void)g;
+    return eligible && (uint64_t)B * (uint64_t)V >= (1ull << 19);
 }
 
 template <bool PEN>
@@ -1616,7 +1624,7 @@ int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes)
     if (!bytes) return RS_ERR_NULL;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
-    *bytes = stream_layout(B, V, sizeof(WsHeader) + (size_t)B * sizeof(RowCtl)).end;
+    *bytes = stream_layout(B, V, sizeof(WsHeader)).end + (size_t)B * sizeof(RowCtl);
     return RS_OK;
 }
 
@@ -1670,17 +1678,17 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     p.logits = logits; p.penalties = penalties; p.out = out;
     p.rng = (uint32_t *)rng_state; p.inj_u = injected_u; p.diag = diag; p.e_bits = e_bits;
     p.hdr = (WsHeader *)workspace;
-    p.ctl = (RowCtl *)((char *)workspace + sizeof(WsHeader));
+    p.ctl_end = (RowCtl *)((char *)workspace + (workspace_bytes & ~(size_t)255));
     p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
     p.need = nullptr; p.stash_k = (uint32_t)top_k;
     dim3 grid((uint32_t)B * g.G);
     if (choose_stream(B, V, top_k, pen, e_bits != nullptr, g)) {
-        const StreamLayout l = stream_layout(B, V, sizeof(WsHeader) + (size_t)B * sizeof(RowCtl));
+        const StreamLayout l = stream_layout(B, V, sizeof(WsHeader));
         char *w = (char *)workspace;
         StreamView v;
-        v.hdr = (PartHdr *)(w + l.hdr); v.rowhist = (uint64_t *)(w + l.hist); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
+        v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.need = (uint32_t *)(w + l.need); v.G = stream_parts(V);
         p.stash_k = (uint32_t)top_k < 128u ? (uint32_t)top_k : min((uint32_t)top_k, max(128u, 8u * (uint32_t)top_k / v.G));
         hipStream_t st = (hipStream_t)stream;

@@ -27,19 +27,27 @@ void *current_stream(const at::Tensor &t)
     return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
 }
 
-// One zero-initialised workspace per (device, stream), grown on demand.  The
-// kernels leave it clean, so it is never cleared again; calls that share it
-// are ordered by the stream.  Takes the place of the reference's per-call
-// `probs` scratch (sampling.cu:488,1014).
-at::Tensor &workspace_for(const at::Tensor &like, void *stream, size_t bytes)
+// One zero-initialised workspace per (device, stream), sized for the largest B
+// and the largest V seen so far (the two maxima separately: that is what lets
+// calls of different shapes share it).  The kernels leave it clean, so it is
+// never cleared again; calls that share it are ordered by the stream.  Takes
+// the place of the reference's per-call `probs` scratch (sampling.cu:488,1014).
+at::Tensor &workspace_for(const at::Tensor &like, void *stream, int64_t B, int64_t V)
 {
+    struct Entry { at::Tensor ws; int64_t B = 0, V = 0; };
     static std::mutex mu;
-    static std::map<std::pair<int, void *>, at::Tensor> cache;
+    static std::map<std::pair<int, void *>, Entry> cache;
     std::lock_guard<std::mutex> lock(mu);
-    at::Tensor &ws = cache[{(int)like.device().index(), stream}];
-    if (!ws.defined() || (size_t)ws.numel() < bytes)
-        ws = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
-    return ws;
+    Entry &e = cache[{(int)like.device().index(), stream}];
+    if (!e.ws.defined() || B > e.B || V > e.V) {
+        e.B = std::max(e.B, B);
+        e.V = std::max(e.V, V);
+        size_t bytes = 0;
+        rs_workspace_bytes((int32_t)e.B, (int32_t)e.V, &bytes);
+        e.ws = at::Tensor();          // release the old one first
+        e.ws = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
+    }
+    return e.ws;
 }
 
 void throw_for(int code, int64_t B, int64_t T, int64_t V, double temperature)
@@ -137,7 +145,7 @@ at::Tensor run(const at::Tensor &logits, const Shape &s, at::Tensor *penalties, 
     void *stream = current_stream(logits);
     size_t bytes = 0;
     throw_for(rs_workspace_bytes((int32_t)s.B, (int32_t)s.V, &bytes), s.B, s.T, s.V, temperature);
-    at::Tensor &ws = workspace_for(logits, stream, bytes);
+    at::Tensor &ws = workspace_for(logits, stream, s.B, s.V);
     auto out = at::empty({s.B}, at::TensorOptions().dtype(at::kInt).device(logits.device()));
     rs_row_diag *diag = nullptr;
     uint32_t *ebits = nullptr;

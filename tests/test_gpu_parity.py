@@ -238,6 +238,25 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
     assert np.array_equal(res["stream"]["out"][rows], ref_out)
 
 
+def test_one_workspace_many_shapes(torch_cuda, oracle):
+    """Calls of different (B, V, top_k) -- and so of different paths and layouts -- on one workspace sized
+    for the largest B and the largest V: what one call leaves behind must not disturb the next."""
+    torch = torch_cuda
+    from tests import capi
+    smp = capi.Sampler(64, 151936)
+    seq = [(8, 151936, 100, 1.0, "n"), (64, 151936, -1, 0.3, "u"), (3, 32768, 50, 0.9, "n"), (64, 151936, 100, 0.9, "n"),
+           (1, 151936, -1, 0.5, "u"), (40, 65536, 1000, 1.0, "n"), (64, 4096, -1, 0.9, "u"), (8, 151936, 100, 1.0, "n")]
+    for i, (B, V, k_in, p_in, kind) in enumerate(seq):
+        lg_np = H.logits_uniform(B, V, seed=200 + i) if kind == "u" else H.logits_normal(B, V, 2.0, seed=200 + i)
+        rc, c, k, p = capi.normalize(1.0, k_in, p_in, V, B, 1)
+        u_np = H.uniforms(B, 300 + i)
+        ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np)
+        print("shape", i, B, V, k, p, flush=True)
+        res = smp.sample(torch.from_numpy(lg_np).cuda(), c, k, p, uniforms=torch.from_numpy(u_np).cuda())
+        _check(res, ref_out, ref_diag, "shape %d" % i)
+        assert smp.status() == 0
+
+
 def test_penalty_path_single_step(torch_cuda, oracle):
     from tests import capi
     B, V = 8, 32768
