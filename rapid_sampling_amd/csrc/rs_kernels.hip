@@ -363,8 +363,9 @@ __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G,
 // one wave (lane l owns indices 511-3l, 510-3l, 509-3l), so the scan needs no
 // LDS exchange; the exponent of bin idx is idx >> 2.  With LOCAL the wave also
 // scans this workgroup's own histogram s.hm and returns its mass above the
-// boundary bin in local_above.
-template <bool LOCAL>
+// boundary bin in local_above.  With GIVEN_P the histogram is that of a
+// subset of the row which is complete above some value: D and P are left alone.
+template <bool LOCAL, bool GIVEN_P = false>
 __device__ __forceinline__ Found hist_find_level1(Lds &s, uint64_t top_k, float top_p, int lane, int wave)
 {
     if (wave == 0) {
@@ -387,9 +388,17 @@ __device__ __forceinline__ Found hist_find_level1(Lds &s, uint64_t top_k, float 
         const uint32_t ci = wave_inclusive_scan(cs);
         u128 hrun = 0;
         if (LOCAL) hrun = wave_inclusive_scan(hs) - hs;
-        const u128 D = lane63(mi);
-        const u128 P = ceil_mul(top_p, D);
-        if (lane == 0) { s.D = D; s.P = P; }
+        u128 P;
+        if (GIVEN_P) {
+            // the histogram holds only part of the row: P stands as it is, and the scan may end
+            // without the set becoming sufficient (bin 0 then)
+            P = s.P;
+            if (lane == 0) s.found.bin = 0;
+        } else {
+            const u128 D = lane63(mi);
+            P = ceil_mul(top_p, D);
+            if (lane == 0) { s.D = D; s.P = P; }
+        }
         uint64_t rcnt = (uint64_t)ci - cs;               // count before my first bin
         u128 rm = mi - ms;                               // mass before my first bin
 #pragma unroll
@@ -1037,7 +1046,8 @@ struct PartHdr {
     uint32_t mkey;        // fkey(max x of the slice)
     uint32_t cov;         // the stash holds every token of the slice with bin - 348 >= cov
     uint32_t n;           // entries in the stash
-    uint32_t pad;
+    uint32_t cut;         // the stash holds every token of the slice with bits(e) >= cut (slice frame); cut lies in
+                          // bin cov or, when only part of a bin fitted, in bin cov - 1
 };
 
 struct StreamView {
@@ -1053,8 +1063,9 @@ struct LdsA {
     uint32_t gidx[kStashCap];    // and the index of their first token
     uint64_t hm[kSB];
     uint32_t off[kSB];
+    uint32_t sub[128];           // level-2 counts inside a boundary bin too large for the stash
     uint32_t u32[16];
-    uint32_t cov, n;
+    uint32_t cov, n, cut, over;
 };
 
 template <int R, int NT>     // NT threads, each with R float4 of the slice
@@ -1149,7 +1160,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         const uint32_t ci = wave_inclusive_scan(cs);
         uint32_t run = ci - cs;
         const uint32_t total = lane63(ci);
-        if (lane == 0 && total < Ks) { s.cov = 0u; s.n = total; }       // a short slice: all of it (total < top_k <= cap)
+        if (lane == 0) s.over = 0xFFFFFFFFu;
+        if (lane == 0 && total < Ks) { s.cov = 0u; s.n = total; s.cut = kBin0 << 21; }   // a short slice: all of it
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             const int b = kSB - 1 - 3 * lane - i;
@@ -1159,15 +1171,47 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
                 v.cum[((size_t)row * G + part) * kSB + b] = nx;
             }
             if (run < Ks && nx >= Ks) {
-                if (nx <= (uint32_t)kStashCap) { s.cov = (uint32_t)b; s.n = nx; }
-                else { s.cov = (uint32_t)b + 1u; s.n = run; }
+                if (nx <= (uint32_t)kStashCap) { s.cov = (uint32_t)b; s.n = nx; s.cut = ((uint32_t)b + kBin0) << 21; }
+                else { s.cov = (uint32_t)b + 1u; s.n = run; s.cut = ((uint32_t)b + 1u + kBin0) << 21; s.over = (uint32_t)b; }
             }
             run = nx;
         }
     }
+    if (tid < 128) s.sub[tid] = 0;
     __syncthreads();
+    if (s.over != 0xFFFFFFFFu) {
+        // The bin in which the count reaches stash_k does not fit (a flat distribution: thousands of
+        // tokens within a quarter octave).  Look at its next 7 bits and take the sub-bins from the top
+        // down to the one at which the count reaches stash_k, as far as they fit.
+        const uint32_t ob = s.over + kBin0, above = s.n;
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t b = eb[j * 4 + q];
+                if ((b >> 21) == ob) atomicAdd(&s.sub[(b >> 14) & 127u], 1u);
+            }
+        __syncthreads();
+        if (wave == 0) {
+            const uint32_t Ks = p.stash_k;
+            const uint32_t c0 = s.sub[127 - 2 * lane], c1 = s.sub[126 - 2 * lane];
+            const uint32_t ci = wave_inclusive_scan(c0 + c1);
+            const uint32_t r0 = above + ci - c0 - c1, r1 = r0 + c0, r2 = r1 + c1;
+            // first sub-bin at which the count reaches stash_k (there is one: the whole bin reaches it)
+            if (r0 < Ks && r1 >= Ks) {
+                const bool fits = r1 <= (uint32_t)kStashCap;
+                s.n = fits ? r1 : r0;
+                s.cut = (ob << 21) + ((127u - 2u * (uint32_t)lane + (fits ? 0u : 1u)) << 14);
+            } else if (r1 < Ks && r2 >= Ks) {
+                const bool fits = r2 <= (uint32_t)kStashCap;
+                s.n = fits ? r2 : r1;
+                s.cut = (ob << 21) + ((126u - 2u * (uint32_t)lane + (fits ? 0u : 1u)) << 14);
+            }
+        }
+        __syncthreads();
+    }
     const uint32_t cov = s.cov, n = s.n;
-    const uint32_t cut = (cov + kBin0) << 21;
+    const uint32_t cut = s.cut;
 
     // Candidates (bits >= cut) are at most n <= kStashCap, so at most that many float4 groups
     // hold one.  Each thread copies its groups with a candidate into LDS at an offset from a scan
@@ -1211,7 +1255,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     }
     if (tid == 0) {
         PartHdr ph;
-        ph.mkey = k; ph.cov = cov; ph.n = n; ph.pad = 0;
+        ph.mkey = k; ph.cov = cov; ph.n = n; ph.cut = cut;
         v.hdr[(size_t)row * G + part] = ph;
     }
 }
@@ -1274,7 +1318,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
 
     if (tid == 0) { s.abort = 0; t.fail = 0; s.ctr = 0; }
     PartHdr ph;
-    ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.pad = 0;
+    ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.cut = 0;
     if ((uint32_t)tid < G) ph = hdrs[tid];
     const uint64_t h0 = rowhist[tid], h1 = rowhist[tid + kThreads];
     rowhist[tid] = 0; rowhist[tid + kThreads] = 0;                   // left clean for the next call
@@ -1308,10 +1352,10 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     const uint64_t top_k = (uint64_t)p.top_k;
     Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
-    const uint32_t exb = f.bin >> 2;
 
-    // what each stash must hold, and whether it does
-    const uint32_t total = f.cnt_above + f.cnt_bin;
+    // Plan A: every stash reaches down to the row's boundary bin.  Then exactly the tokens at or
+    // above that bin are taken, a prefix of each stash whose length is one cumulative count.
+    uint32_t total = f.cnt_above + f.cnt_bin;
     uint32_t mtake = 0;
     bool bad = mixed || total > (uint32_t)kFinCap;
     if ((uint32_t)tid < G) {
@@ -1323,24 +1367,39 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
         else if (mtake && ((int)ph.cov > lb || mtake > ph.n)) bad = true;
     }
     if (bad) t.fail = 1;
-    // prefix of the takes
-    uint32_t inc = wave_inclusive_scan(mtake);
-    __syncthreads();
-    if (lane == kWave - 1) s.u32[wave] = inc;
-    __syncthreads();
-    for (int w = 0; w < wave; ++w) inc += s.u32[w];
-    t.take[tid] = inc;
-    __syncthreads();
+    auto take_prefix = [&](uint32_t mine) {                           // inclusive prefix over the slices, into t.take
+        uint32_t inc = wave_inclusive_scan(mine);
+        __syncthreads();
+        if (lane == kWave - 1) s.u32[wave] = inc;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) inc += s.u32[w];
+        t.take[tid] = inc;
+        __syncthreads();
+    };
+    take_prefix(mtake);
+    bool subset = false;                                               // plan B in force
+    uint32_t cutrow = 0;
     if (t.fail || t.take[kThreads - 1] != total) {
-        // not resolvable from the stashes: leave the row to the cluster kernel
-        if (tid == 0) {
-            const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
-            v.need[slot] = row;
+        // Plan B (flat distributions: the boundary bin holds thousands of tokens, but top_k is small):
+        // take the stashes whole.  Together they hold every token of the row at or above
+        // cutrow = the largest of the slices' cuts, so a threshold found among those is the row's.
+        uint32_t mycut = 0;
+        if ((uint32_t)tid < G) mycut = rebase_bits(ph.cut, dl);
+        cutrow = block_max_u32(s, mycut, lane, wave);
+        take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
+        total = t.take[kThreads - 1];
+        if (mixed || total > (uint32_t)kFinCap || total == 0u) {
+            // not resolvable from the stashes: leave the row to the cluster kernel
+            if (tid == 0) {
+                const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
+                v.need[slot] = row;
+            }
+            return;
         }
-        return;
+        subset = true;
     }
 
-    // gather the tokens at or above the boundary bin, re-based to the row's frame
+    // gather the tokens, re-based to the row's frame
     {
         constexpr int kBatch = 4;
         for (uint32_t i0 = tid; i0 < total; i0 += kBatch * kThreads) {
@@ -1365,13 +1424,35 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
             for (int u = 0; u < kBatch; ++u) {
                 const uint32_t i = i0 + (uint32_t)u * kThreads;
                 if (i < total) {
-                    const uint32_t b = (uint32_t)(e[u] >> 32) - (t.delta[sl[u]] << 23);
+                    uint32_t b = rebase_bits((uint32_t)(e[u] >> 32), t.delta[sl[u]]);
+                    if (b < cutrow) b = 0;                             // plan B: below the complete part; 0 matches nothing
                     t.list[i] = ((uint64_t)b << 32) | (uint32_t)e[u];
                 }
             }
         }
     }
     __syncthreads();
+    uint32_t exb = f.bin >> 2;
+    if (subset) {
+        // level 1 again, on the gathered tokens alone
+        for (int b = tid; b < kSB; b += kThreads) s.g[kBin0 + b] = 0;
+        __syncthreads();
+        for (uint32_t i = tid; i < total; i += kThreads) {
+            const uint32_t b = (uint32_t)(t.list[i] >> 32);
+            if (b) atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[b >> 21]), (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
+        }
+        __syncthreads();
+        f = hist_find_level1<false, true>(s, top_k, p.top_p, lane, wave);
+        if (f.bin == 0u) {
+            // even all of them are neither top_k tokens nor top_p of the mass
+            if (tid == 0) {
+                const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
+                v.need[slot] = row;
+            }
+            return;
+        }
+        exb = f.bin >> 2;
+    }
 
     // remaining digits of the threshold, on the gathered tokens
     uint32_t lo = f.bin << 21, span = (1u << 21) - 1u;

@@ -238,6 +238,36 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
     assert np.array_equal(res["stream"]["out"][rows], ref_out)
 
 
+def test_streaming_path_flat_distributions(torch_cuda, oracle):
+    """Flat rows with a small top_k: the bin in which the count reaches top_k holds thousands of tokens, so
+    a slice refines its cut inside that bin and the finish works on the whole stashes (the reference's
+    benchmark generators, /root/reference/bench.py:66-72: zeros, U[0,1), N(0,1)/2, N(0,1)*3, U[0,1)*4)."""
+    from tests import capi
+    V = 65536 + 8192
+    rng = np.random.default_rng(5)
+    lg = np.zeros((7, V), dtype=np.float32)
+    lg[1] = rng.random(V, dtype=np.float32)
+    lg[2] = rng.standard_normal(V, dtype=np.float32) / 2
+    lg[3] = rng.standard_normal(V, dtype=np.float32) * 3
+    lg[4] = rng.random(V, dtype=np.float32) * 4
+    lg[5] = rng.random(V, dtype=np.float32) * 1e-3                      # everything within a thousandth of an octave
+    lg[6] = np.round(rng.random(V, dtype=np.float32) * 64) / 64         # 65 distinct values: ties of a thousand tokens
+    for (k, p) in [(100, 0.9), (10, 1.0), (1000, 0.3), (1, 1.0), (1024, 1.0)]:
+        _run_case(torch_cuda, oracle, capi, lg, 1.0, k, p, u_np=H.uniforms(7, 41), what="flat k=%s p=%s" % (k, p))
+    os.environ["RS_FORCE_PATH"] = "stream"
+    try:
+        rc, c, k, p = capi.normalize(1.0, 100, 0.9, V, 7, 1)
+        res = capi.Sampler(7, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p,
+                                        uniforms=torch_cuda.from_numpy(H.uniforms(7, 41)).cuda())
+        rounds = res["diag"]["rounds"]
+        assert all(rounds[i] == 0 for i in (1, 2, 3, 4, 6)), rounds     # finished from the stashes
+        # handed on: all equal (a tie of every token), and a row so flat that even a level-2 sub-bin
+        # holds more tokens than a stash
+        assert rounds[0] >= 1 and rounds[5] >= 1, rounds
+    finally:
+        os.environ.pop("RS_FORCE_PATH", None)
+
+
 def test_one_workspace_many_shapes(torch_cuda, oracle):
     """Calls of different (B, V, top_k) -- and so of different paths and layouts -- on one workspace sized
     for the largest B and the largest V: what one call leaves behind must not disturb the next."""
