@@ -68,12 +68,10 @@ struct alignas(256) WsHeader {
 // workspace is at least rs_workspace_bytes(largest B, largest V) of the calls
 // that share it.
 struct alignas(256) RowCtl {
-    uint32_t unused0;
     uint32_t done;        // workgroups finished with this row
-    uint32_t unused1;
     uint32_t cursor;      // fill of cand[]
     uint32_t index_p1;    // sampled token + 1, once known
-    uint32_t pad[3];
+    uint32_t pad[5];
     uint32_t mx[kMaxParts];     // per workgroup: fkey(max x of its slice), 0 = not yet written
     uint64_t A[2 * kMaxParts];  // per workgroup: a 124-bit mass as two words of 62 bits, each | kValid
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
@@ -452,15 +450,15 @@ __device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint3
     return s.found;
 }
 
-// Mass of this workgroup's own tokens in the bins above index `bin` (larger
-// e), from s.hm, summed over the workgroup.  level1: exponent = index >> 2,
-// else the shared exponent ex.
-__device__ __forceinline__ u128 local_mass_above(Lds &s, uint32_t bin, uint32_t top, bool level1, uint32_t ex, int lane, int wave)
+// Mass of this workgroup's own tokens in the bins above index `bin` of a
+// 128-bin level (larger e), from s.hm, summed over the workgroup.  All tokens
+// of the level share the exponent ex.
+__device__ __forceinline__ u128 local_mass_above(Lds &s, uint32_t bin, uint32_t ex, int lane, int wave)
 {
     u128 a = 0;
-    for (uint32_t b = bin + 1 + threadIdx.x; b <= top; b += kThreads) {
+    for (uint32_t b = bin + 1 + threadIdx.x; b <= kTopN; b += kThreads) {
         const uint64_t w = s.hm[b];
-        if (w) a += pack_mass(w, level1 ? b >> 2 : ex);
+        if (w) a += pack_mass(w, ex);
     }
     return block_sum_u128(s, a, lane, wave);
 }
@@ -713,7 +711,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         }
         hx = levels - 1; hx_nb = 128;
         f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
-        amass += local_mass_above(s, f.bin, kTopN, false, exb, lane, wave);
+        amass += local_mass_above(s, f.bin, exb, lane, wave);
         mycnt = pack_count(s.hm[f.bin]);
         lo |= f.bin << dsh;
         span = (1u << dsh) - 1u;
@@ -1316,7 +1314,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     const PartHdr *hdrs = v.hdr + (size_t)row * G;
     uint64_t *rowhist = (p.ctl_end - 1 - row)->rowhist;
 
-    if (tid == 0) { s.abort = 0; t.fail = 0; s.ctr = 0; }
+    if (tid == 0) { s.abort = 0; t.fail = 0; }
     PartHdr ph;
     ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.cut = 0;
     if ((uint32_t)tid < G) ph = hdrs[tid];
