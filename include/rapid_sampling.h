@@ -78,7 +78,7 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
 /*
  * Size of the workspace rs_sample needs for a batch of B rows of V tokens.
  * Replaces the reference's per-call `probs` scratch tensor of B*V floats
- * (sampling.cu:488,1014): a fixed record per row (about 35 KB) plus, for the
+ * (sampling.cu:488,1014): a fixed record per row (about 38 KB) plus, for the
  * streaming path, about 0.7 bytes per token (stashes of the largest tokens
  * of each slice of 16384 tokens); under a fifth of the reference's scratch
  * for large V.  It does not grow with T.
