@@ -49,6 +49,7 @@ constexpr int      kNB        = 512;          // bins per histogram: level 1 use
 constexpr int      kLevels    = 4;            // 10 + 7 + 7 + 7 bits
 constexpr int      kCap       = 1024;         // tokens of a boundary bin that are gathered
 constexpr uint64_t kSpinLimit = 200000000ull; // 2 s of the 100 MHz wall clock
+
 constexpr uint64_t kValid     = 1ull << 63;   // marks a written exchange word
 
 struct alignas(256) WsHeader {
@@ -56,8 +57,16 @@ struct alignas(256) WsHeader {
     uint32_t finished;    // workgroups that have left the running launch
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows the streaming pass handed to the cluster kernel
-    uint32_t pad[60];
+    uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
+    uint32_t pad[59];
 };
+
+// How long a workgroup waits for its peers before it gives up (wall-clock ticks).
+__device__ __forceinline__ uint64_t spin_limit(const WsHeader *hdr)
+{
+    const uint32_t t = hdr->spin_ticks;
+    return t ? (uint64_t)t << 10 : kSpinLimit;
+}
 
 // Per-row record.  Everything a call reads before writing it is zero when the
 // call starts: the call itself re-zeroes what it used before it ends.  The
@@ -233,7 +242,7 @@ struct SpinGuard {
     // call by every thread once per polling round, before the round's __syncthreads
     __device__ __forceinline__ void tick(Lds &s, WsHeader *hdr)
     {
-        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
+        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(hdr)) {
             a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
             s.abort = 1;
         }
@@ -917,7 +926,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 const uint64_t t0 = wall_clock64();
                 uint32_t spins = 0, v;
                 while ((v = a_load(&rc->index_p1)) == 0u) {
-                    if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > kSpinLimit) {
+                    if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(p.hdr)) {
                         a_store(&p.hdr->error, (int32_t)RS_ERR_DEVICE);
                         s.abort = 1;
                         break;
@@ -1711,7 +1720,19 @@ int rs_workspace_init(void *ws, size_t bytes, void *stream)
 {
     if (!ws) return RS_ERR_NULL;
     if (bytes < sizeof(WsHeader) || ((uintptr_t)ws & 255)) return RS_ERR_WORKSPACE;
-    return hipMemsetAsync(ws, 0, bytes, (hipStream_t)stream) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+    if (hipMemsetAsync(ws, 0, bytes, (hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
+    // test hook: RS_SPIN_LIMIT_MS shortens the bound of the waits (default 2000 ms)
+    if (const char *ms = getenv("RS_SPIN_LIMIT_MS")) {
+        const long v = atol(ms);
+        if (v > 0 && v < 40000) {
+            const uint32_t ticks = (uint32_t)((uint64_t)v * 100000ull >> 10);      // 100 MHz wall clock
+            WsHeader *h = (WsHeader *)ws;
+            if (hipMemcpyAsync(&h->spin_ticks, &ticks, sizeof ticks, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess)
+                return RS_ERR_LAUNCH;
+            if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;   // `ticks` is on the stack
+        }
+    }
+    return RS_OK;
 }
 
 int rs_workspace_status(const void *ws, int32_t *status, void *stream)

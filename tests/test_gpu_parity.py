@@ -400,6 +400,38 @@ def test_hip_graph_decode_loop(torch_cuda, oracle, path, pen_on):
     assert smp.status() == 0
 
 
+def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
+    """A workspace that was never cleaned (here: filled with ones behind its header) holds histograms that
+    never add up.  The workgroups must give up after the bound of their waits (shortened to 20 ms through
+    the test hook of rs_workspace_init), leave a sticky RS_ERR_DEVICE and end normally; after
+    rs_workspace_init the same workspace works again."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 2, 65536
+    lg_np = H.logits_normal(B, V, 2.0, seed=80)
+    rc, c, k, p = capi.normalize(1.0, -1, 0.9, V, B, 1)
+    u_np = H.uniforms(B, 81)
+    ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np)
+    smp = capi.Sampler(B, V)
+    lg, u = torch.from_numpy(lg_np).cuda(), torch.from_numpy(u_np).cuda()
+    os.environ["RS_SPIN_LIMIT_MS"] = "20"
+    try:
+        assert capi.lib().rs_workspace_init(smp.ws.data_ptr(), smp.ws.numel(), smp.stream()) == 0
+        smp.ws[256:] = 1
+        torch.cuda.synchronize()
+        print("poisoned workspace, expecting a bounded wait to give up", flush=True)
+        res = smp.sample(lg, c, k, p, uniforms=u, want_diag=False)
+        assert res["rc"] == 0                       # the launch itself is fine
+        assert smp.status() == -9                   # RS_ERR_DEVICE, sticky
+        assert capi.lib().rs_workspace_init(smp.ws.data_ptr(), smp.ws.numel(), smp.stream()) == 0
+        assert smp.status() == 0
+        res = smp.sample(lg, c, k, p, uniforms=u)
+        _check(res, ref_out, ref_diag, "after re-initialisation")
+        assert smp.status() == 0
+    finally:
+        os.environ.pop("RS_SPIN_LIMIT_MS", None)
+
+
 def test_chi_square_one_million_draws(torch_cuda, oracle):
     """1,048,576 Philox-driven draws of one row against the exact renormalised weights w_i / S."""
     torch = torch_cuda
