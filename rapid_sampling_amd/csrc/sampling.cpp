@@ -17,6 +17,7 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <vector>
 
 #include "rapid_sampling.h"
 
@@ -34,7 +35,8 @@ void *current_stream(const at::Tensor &t)
 // the place of the reference's per-call `probs` scratch (sampling.cu:488,1014).
 at::Tensor &workspace_for(const at::Tensor &like, void *stream, int64_t B, int64_t V)
 {
-    struct Entry { at::Tensor ws; int64_t B = 0, V = 0; };
+    // `retired` keeps outgrown workspaces alive: a captured HIP graph may still point into one
+    struct Entry { at::Tensor ws; int64_t B = 0, V = 0; std::vector<at::Tensor> retired; };
     static std::mutex mu;
     static std::map<std::pair<int, void *>, Entry> cache;
     std::lock_guard<std::mutex> lock(mu);
@@ -44,7 +46,7 @@ at::Tensor &workspace_for(const at::Tensor &like, void *stream, int64_t B, int64
         e.V = std::max(e.V, V);
         size_t bytes = 0;
         rs_workspace_bytes((int32_t)e.B, (int32_t)e.V, &bytes);
-        e.ws = at::Tensor();          // release the old one first
+        if (e.ws.defined()) e.retired.push_back(e.ws);
         e.ws = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
     }
     return e.ws;
