@@ -400,6 +400,46 @@ def test_hip_graph_decode_loop(torch_cuda, oracle, path, pen_on):
     assert smp.status() == 0
 
 
+def test_python_module_drop_in_calls(torch_cuda, oracle):
+    """The reference's three functions through the PyTorch extension (the drop-in surface), not the C ABI:
+    setup_rand + both sampling calls, (V,), (B,V) and (B,T,V) logits, penalties in place, shapes changing
+    from call to call (the module's workspace cache grows), all against the oracle's Philox stream."""
+    torch = torch_cuda
+    import rapid_sampling_amd as sample
+    seed = 20240607
+    for (shape, k_in, p_in, temp) in [((5, 32768), 50, 0.9, 0.8), ((3, 4, 65536), -1, 0.7, 1.0), ((131072,), 20, 1.0, 1.3),
+                                      ((70, 8192), 1000, 0.95, 1.0), ((5, 32768), 50, 0.9, 0.8)]:
+        V = shape[-1]
+        B = shape[0] if len(shape) > 1 else 1
+        T = shape[1] if len(shape) == 3 else 1
+        lg_np = H.logits_normal(B * T, V, 2.0, seed=V % 1000 + B).reshape(shape)
+        c, k, p = oracle.normalize(temp, k_in, p_in, V, B, T)
+        states = sample.setup_rand(seed, B)
+        rng_ref = oracle.rng_init(seed, B)
+        lg = torch.from_numpy(lg_np).cuda()
+        for call in range(3):
+            ref_out, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref)
+            out = sample.batch_sampling_temperature_topk_topp(lg, states, temp, k_in, p_in)
+            assert out.dtype == torch.int32 and tuple(out.shape) == (B,)
+            assert np.array_equal(out.cpu().numpy(), ref_out), (shape, call)
+        # the penalty call continues the same Philox stream and updates penalties in place
+        pen_ref = H.penalties_sparse(B, V, seed=7)
+        pen = torch.from_numpy(pen_ref.copy()).cuda()
+        for call in range(2):
+            ref_out, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref, penalties=pen_ref,
+                                             presence=0.3, repetition=0.1, decay=0.99)
+            out = sample.batch_sampling_repetition_temperature_topk_topp(lg, pen, states, 0.3, 0.1, 0.99,
+                                                                         temp, k_in, p_in)
+            assert np.array_equal(out.cpu().numpy(), ref_out), (shape, "pen", call)
+        assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32))
+        # keyword call with injected uniforms
+        u_np = H.uniforms(B, 5)
+        ref_out, _ = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np)
+        out = sample.batch_sampling_temperature_topk_topp(logits=lg, states=states, temperature=temp, top_k=k_in,
+                                                          top_p=p_in, uniforms=torch.from_numpy(u_np).cuda())
+        assert np.array_equal(out.cpu().numpy(), ref_out)
+
+
 def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
     """A workspace that was never cleaned (here: filled with ones behind its header) holds histograms that
     never add up.  The workgroups must give up after the bound of their waits (shortened to 20 ms through
