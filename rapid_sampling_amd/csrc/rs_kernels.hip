@@ -1047,7 +1047,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
 constexpr int      kSB       = 164;           // level-1 bins in use: indices 348..511
 constexpr int      kStashCap = 1280;          // stash entries per slice (at least kStreamK)
 constexpr int      kStreamK  = 1024;          // largest top_k the streaming path takes
-constexpr int      kFinCap   = 4096;          // tokens the finishing workgroup can hold
+constexpr int      kFinCap   = 8192;          // tokens the finishing workgroup can hold at most (64 KB of LDS)
 
 struct PartHdr {
     uint32_t mkey;        // fkey(max x of the slice)
@@ -1063,6 +1063,7 @@ struct StreamView {
     uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
     uint32_t *need;       // [B]  rows left to the cluster kernel
     uint32_t  G;          // slices per row
+    uint32_t  list_cap;   // entries of the finishing workgroup's token list (a power of two up to kFinCap)
 };
 
 struct LdsA {
@@ -1178,7 +1179,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
                 v.cum[((size_t)row * G + part) * kSB + b] = nx;
             }
             if (run < Ks && nx >= Ks) {
-                if (nx <= (uint32_t)kStashCap) { s.cov = (uint32_t)b; s.n = nx; s.cut = ((uint32_t)b + kBin0) << 21; }
+                // the whole bin if that stays close to stash_k, else only part of it (found below)
+                if (nx <= min((uint32_t)kStashCap, Ks + max(64u, Ks >> 2))) { s.cov = (uint32_t)b; s.n = nx; s.cut = ((uint32_t)b + kBin0) << 21; }
                 else { s.cov = (uint32_t)b + 1u; s.n = run; s.cut = ((uint32_t)b + 1u + kBin0) << 21; s.over = (uint32_t)b; }
             }
             run = nx;
@@ -1187,9 +1189,10 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     if (tid < 128) s.sub[tid] = 0;
     __syncthreads();
     if (s.over != 0xFFFFFFFFu) {
-        // The bin in which the count reaches stash_k does not fit (a flat distribution: thousands of
-        // tokens within a quarter octave).  Look at its next 7 bits and take the sub-bins from the top
-        // down to the one at which the count reaches stash_k, as far as they fit.
+        // The bin in which the count reaches stash_k holds far more tokens than asked for (a flat
+        // distribution: hundreds or thousands of tokens within a quarter octave).  Look at its next
+        // 7 bits and take the sub-bins from the top down to the one at which the count reaches
+        // stash_k, as far as they fit.
         const uint32_t ob = s.over + kBin0, above = s.n;
 #pragma unroll
         for (int j = 0; j < R; ++j)
@@ -1268,7 +1271,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
 }
 
 struct LdsB {
-    uint64_t list[kFinCap];      // gathered tokens, row frame: bits << 32 | index
+    uint64_t *list;              // gathered tokens, row frame: bits << 32 | index (dynamic LDS, v.list_cap entries)
     uint64_t blo[kMaxParts], bhi[kMaxParts];
     uint64_t small[128];
     uint32_t delta[kMaxParts];   // octaves between the row's frame and slice g's
@@ -1318,6 +1321,8 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
 {
     __shared__ Lds s;
     __shared__ LdsB t;
+    extern __shared__ __align__(16) unsigned char finish_dyn[];
+    t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t G = v.G, row = blockIdx.x;
     const PartHdr *hdrs = v.hdr + (size_t)row * G;
@@ -1364,7 +1369,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     // above that bin are taken, a prefix of each stash whose length is one cumulative count.
     uint32_t total = f.cnt_above + f.cnt_bin;
     uint32_t mtake = 0;
-    bool bad = mixed || total > (uint32_t)kFinCap;
+    bool bad = mixed || total > v.list_cap;
     if ((uint32_t)tid < G) {
         const int lb = (int)(f.bin - kBin0) + 4 * (int)dl;            // boundary bin in the slice's frame
         if (dl >= 64u) mtake = 0;                                      // the whole slice is clamped; the boundary bin
@@ -1395,7 +1400,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
         cutrow = block_max_u32(s, mycut, lane, wave);
         take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
         total = t.take[kThreads - 1];
-        if (mixed || total > (uint32_t)kFinCap || total == 0u) {
+        if (mixed || total > v.list_cap || total == 0u) {
             // not resolvable from the stashes: leave the row to the cluster kernel
             if (tid == 0) {
                 const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
@@ -1602,15 +1607,18 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
 }
 
 
-// Streaming geometry: workgroups of 256 threads with 16 float4 each: slices of 16384 tokens.
-constexpr int kStreamR = 16, kStreamNT = 256, kStreamSliceLog2 = 14;
-static_assert(kStreamR * kStreamNT * 4 == 1 << kStreamSliceLog2, "slice size");
-static uint32_t stream_parts(int32_t V) { return ((uint32_t)V / 4 + kStreamNT * kStreamR - 1) / (kStreamNT * kStreamR); }
+// Streaming geometry: workgroups of 256 threads; slices of 16384 tokens (16 float4 per thread), or
+// of 4096 tokens (4 float4) for calls of up to kStreamSmall tokens in rows of up to 262144, where a
+// shorter slice shortens the one wave of workgroups the whole pass consists of (longer rows would
+// be cut into more slices than a finishing workgroup handles quickly).
+constexpr int kStreamNT = 256;
+constexpr uint64_t kStreamSmall = 1ull << 22;
+static int stream_r(int32_t B, int32_t V) { return (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144 ? 4 : 16; }
+static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 struct StreamLayout { size_t hdr, cum, stash, need, end; };
-static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
+static StreamLayout stream_layout(int32_t B, size_t parts, size_t base)
 {
-    const size_t parts = (size_t)B * stream_parts(V);
     StreamLayout l;
     l.hdr = align256(base);
     l.cum = align256(l.hdr + parts * sizeof(PartHdr));
@@ -1619,13 +1627,25 @@ static StreamLayout stream_layout(int32_t B, int32_t V, size_t base)
     l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
     return l;
 }
+// Bytes of per-slice data a workspace for (B, V) sets aside: enough for the long slices of (B, V)
+// itself and for the short slices of any call of at most B rows that takes them (at most
+// kStreamSmall tokens: fewer than kStreamSmall / 4096 + B slices), so that the size grows with
+// B and with V and a workspace for the largest B and V serves every smaller call.
+static size_t stream_bytes(int32_t B, int32_t V)
+{
+    const size_t longs = stream_layout(B, (size_t)B * stream_parts(V, 16), sizeof(WsHeader)).end;
+    size_t small_parts = (size_t)B * stream_parts(V, 4);
+    const size_t cap = (size_t)(kStreamSmall / 4096) + (size_t)B;
+    if (small_parts > cap) small_parts = cap;
+    const size_t shorts = stream_layout(B, small_parts, sizeof(WsHeader)).end;
+    return longs > shorts ? longs : shorts;
+}
 
 // The streaming path (three launches, no waits) needs top_k to bound the kept
-// set.  Measured on MI355X it then matches or beats the cluster kernel from
-// about half a million tokens per call upwards (back to back: 18-19 us for
-// small calls against 17-29 us, 2-3 times faster for large ones); below that
-// the single launch wins by a microsecond.  RS_FORCE_PATH=cluster|stream
-// overrides (tests).
+// set.  Measured on MI355X it then beats the cluster kernel from 131072
+// tokens per call upwards (back to back: 15-17 us for small calls against
+// 16-31 us, 2-3 times faster for large ones); below that the single launch
+// wins by up to a microsecond.  RS_FORCE_PATH=cluster|stream overrides (tests).
 static bool choose_stream(int32_t B, int32_t V, int32_t top_k, bool pen, bool want_e, const Geometry &g)
 {
     const bool eligible = !pen && !want_e && top_k <= kStreamK;
@@ -1633,7 +1653,7 @@ static bool choose_stream(int32_t B, int32_t V, int32_t top_k, bool pen, bool wa
     if (force && force[0] == 'c') return false;
     if (force && force[0] == 's') return eligible;
     (void)g;
-    return eligible && (uint64_t)B * (uint64_t)V >= (1ull << 19);
+    return eligible && (uint64_t)B * (uint64_t)V >= (1ull << 17);
 }
 
 template <bool PEN>
@@ -1712,7 +1732,7 @@ int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes)
     if (!bytes) return RS_ERR_NULL;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
-    *bytes = stream_layout(B, V, sizeof(WsHeader)).end + (size_t)B * sizeof(RowCtl);
+    *bytes = stream_bytes(B, V) + (size_t)B * sizeof(RowCtl);
     return RS_OK;
 }
 
@@ -1785,15 +1805,29 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     p.need = nullptr; p.stash_k = (uint32_t)top_k;
     dim3 grid((uint32_t)B * g.G);
     if (choose_stream(B, V, top_k, pen, e_bits != nullptr, g)) {
-        const StreamLayout l = stream_layout(B, V, sizeof(WsHeader));
-        char *w = (char *)workspace;
+        const int sr = stream_r(B, V);
         StreamView v;
+        v.G = stream_parts(V, sr);
+        const StreamLayout l = stream_layout(B, (size_t)B * v.G, sizeof(WsHeader));
+        char *w = (char *)workspace;
         v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
-        v.need = (uint32_t *)(w + l.need); v.G = stream_parts(V);
+        v.need = (uint32_t *)(w + l.need);
         p.stash_k = (uint32_t)top_k < 128u ? (uint32_t)top_k : min((uint32_t)top_k, max(128u, 8u * (uint32_t)top_k / v.G));
         hipStream_t st = (hipStream_t)stream;
-        hipLaunchKernelGGL((stream_kernel<kStreamR, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
-        hipLaunchKernelGGL((finish_kernel<kStreamSliceLog2>), dim3((uint32_t)B), dim3(kThreads), 0, st, p, v);
+        // The finishing workgroup's list: twice what a well-behaved row needs (its top_k tokens and
+        // a boundary bin, or every stash whole), as a power of two; a row that needs more is handed
+        // on.  Kept small where it can be: the list is LDS, and LDS decides how many rows finish at once.
+        const uint32_t est = 2u * max((uint32_t)top_k + 512u, v.G * (p.stash_k + 64u));
+        v.list_cap = 2048u;
+        while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
+        const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
+        if (sr == 4) {
+            hipLaunchKernelGGL((stream_kernel<4, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
+            hipLaunchKernelGGL((finish_kernel<12>), dim3((uint32_t)B), dim3(kThreads), dyn, st, p, v);
+        } else {
+            hipLaunchKernelGGL((stream_kernel<16, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
+            hipLaunchKernelGGL((finish_kernel<14>), dim3((uint32_t)B), dim3(kThreads), dyn, st, p, v);
+        }
         if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
         p.need = v.need;               // the cluster kernel follows for the rows the finish left over
         if (grid.x > 1024u) grid.x = 1024u / g.G * g.G > 0 ? 1024u / g.G * g.G : g.G;

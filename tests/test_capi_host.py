@@ -78,18 +78,25 @@ def test_limits_accept_the_extremes():
     assert capi.normalize(1000.0, 1, 1.0, 4)[0] == 0
 
 
-def test_workspace_size_is_independent_of_t_and_bounded():
-    """rs_workspace_bytes takes (B, V) only -- T never enters -- grows with B, and stays well below the
-    reference's per-call scratch of B*V floats (sampling.cu:488,1014) plus a fixed record per row."""
+def test_workspace_size_is_independent_of_t_monotone_and_bounded():
+    """rs_workspace_bytes takes (B, V) only -- T never enters.  It grows with B and with V (so that a
+    workspace for the largest B and the largest V serves every smaller call), and stays well below the
+    reference's per-call scratch of B*V floats (sampling.cu:488,1014) apart from a fixed reserve of 12 MB
+    and a record per row."""
+    Bs, Vs = (1, 2, 3, 7, 64, 128, 1000), (4, 4096, 32768, 131072, 152064, 1048576)
     sizes = {}
-    for B in (1, 2, 3, 128):
-        for V in (4, 131072, 1048576):
+    for B in Bs:
+        for V in Vs:
             rc, n = capi.workspace_bytes(B, V)
             assert rc == 0 and n % 256 == 0
-            assert n <= 4096 + B * (65536 + 0.3 * 4 * V)
+            assert n <= 12 * 2 ** 20 + B * (65536 + 0.3 * 4 * V)
             sizes[B, V] = n
-    for V in (4, 131072, 1048576):
-        assert sizes[1, V] < sizes[2, V] < sizes[3, V] < sizes[128, V]
+    for i, B in enumerate(Bs):
+        for j, V in enumerate(Vs):
+            if i:
+                assert sizes[Bs[i - 1], V] < sizes[B, V]
+            if j:
+                assert sizes[B, Vs[j - 1]] <= sizes[B, V]
     assert capi.workspace_bytes(0, 8)[0] == -2 and capi.workspace_bytes(1, 6)[0] == -1
 
 
