@@ -80,8 +80,9 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
  * Replaces the reference's per-call `probs` scratch tensor of B*V floats
  * (sampling.cu:488,1014): a fixed record per row (about 38 KB) plus, for the
  * streaming path, about 0.7 bytes per token (stashes of the largest tokens
- * of each slice of 16384 tokens), at least 11 MB; under a fifth of the
- * reference's scratch for large V.  It does not grow with T.
+ * of each slice; up to 2.7 bytes per token for the first 4M tokens, where
+ * slices are shorter); under a fifth of the reference's scratch for large V.
+ * It does not grow with T.
  *
  * One workspace may serve calls of different shapes if it is at least
  * rs_workspace_bytes(largest B, largest V) of those calls and the same
