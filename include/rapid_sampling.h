@@ -95,6 +95,8 @@ int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes);
  * Zero a freshly allocated workspace (device memory, 256-byte aligned).  Call
  * once after allocation, and again after a call reported RS_ERR_DEVICE;
  * rs_sample leaves the workspace ready for the next call on the same stream.
+ * The first call for a workspace address also allocates 64 bytes of pinned
+ * host memory (see rs_workspace_policy), kept until the process ends.
  */
 int rs_workspace_init(void *workspace_device, size_t bytes, void *stream);
 
@@ -103,6 +105,18 @@ int rs_workspace_init(void *workspace_device, size_t bytes, void *stream);
  * `stream`).  *status is RS_OK or RS_ERR_DEVICE.
  */
 int rs_workspace_status(const void *workspace_device, int32_t *status, void *stream);
+
+/*
+ * Diagnostic: how calls WITHOUT a bounding top_k (top_k > 1024 or disabled, top_p < 1) are
+ * currently routed on this workspace.  Such a call may be attempted on the
+ * wait-free path, which works when the nucleus is small; the finishing kernel
+ * reports each attempt to a word of pinned host memory that rs_sample reads,
+ * without waiting, before the next call.  *state: -1 the workspace was not set
+ * up by rs_workspace_init (never attempted), 0 attempts are made, 1 the last
+ * attempt handed most rows on: calls go to the general kernel, one in 64 tries
+ * again.  Results do not depend on the routing.  No counterpart in the reference.
+ */
+int rs_workspace_policy(const void *workspace_device, int32_t *state);
 
 /*
  * setup_rand (sampling.cu:136-144): initialise B records of RNG state for
@@ -139,7 +153,8 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  * top_k <= 1024 (a wait-free pass over the logits, a per-row finish, and the
  * general kernel for rows the finish hands on); results are identical either
  * way.  Two environment variables exist for tests: RS_FORCE_R (1..32, float4
- * per thread of the general kernel) and RS_FORCE_PATH (cluster | stream).
+ * per thread of the general kernel) and RS_FORCE_PATH (cluster | stream |
+ * optimistic).
  */
 int rs_sample(const float *logits_device, int64_t row_stride,
               float *penalties_device, int32_t *out_device,

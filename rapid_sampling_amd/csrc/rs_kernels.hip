@@ -37,6 +37,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "rapid_sampling.h"
 #include "rs_device.h"
 
@@ -58,7 +61,10 @@ struct alignas(256) WsHeader {
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows the streaming pass handed to the cluster kernel
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
-    uint32_t pad[59];
+    uint32_t fin_rows;    // rows the finishing kernel is through with (attempts without a bounding top_k only)
+    uint32_t pad0;
+    int32_t *hint;        // pinned host word the finishing kernel reports such an attempt to, or null
+    uint32_t pad[54];
 };
 
 // How long a workgroup waits for its peers before it gives up (wall-clock ticks).
@@ -1064,6 +1070,7 @@ struct StreamView {
     uint32_t *need;       // [B]  rows left to the cluster kernel
     uint32_t  G;          // slices per row
     uint32_t  list_cap;   // entries of the finishing workgroup's token list (a power of two up to kFinCap)
+    uint32_t  attempt;    // 1: top_k does not bound the kept set; report how the rows fared
 };
 
 struct LdsA {
@@ -1317,14 +1324,10 @@ __device__ __forceinline__ uint32_t bucket_step(Lds &s, LdsB &t, uint32_t nlist,
 }
 
 template <int SLICE_LOG2>     // log2 of the tokens per slice of the view
-__global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const StreamView v)
+__device__ __forceinline__ void finish_row(const Params &p, const StreamView &v, Lds &s, LdsB &t, const uint32_t row)
 {
-    __shared__ Lds s;
-    __shared__ LdsB t;
-    extern __shared__ __align__(16) unsigned char finish_dyn[];
-    t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const uint32_t G = v.G, row = blockIdx.x;
+    const uint32_t G = v.G;
     const PartHdr *hdrs = v.hdr + (size_t)row * G;
     uint64_t *rowhist = (p.ctl_end - 1 - row)->rowhist;
 
@@ -1544,6 +1547,30 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     }
 }
 
+template <int SLICE_LOG2>
+__global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const StreamView v)
+{
+    __shared__ Lds s;
+    __shared__ LdsB t;
+    extern __shared__ __align__(16) unsigned char finish_dyn[];
+    t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value
+    finish_row<SLICE_LOG2>(p, v, s, t, blockIdx.x);
+    // An attempt without a bounding top_k: the workgroup that is through last tells the host (a
+    // word of pinned memory it looks at before its next call) whether most rows had to be handed
+    // on -- then such calls are better not attempted for a while.
+    if (v.attempt && threadIdx.x == 0) {
+        wait_vmem();                                         // my row's entry in the list, if any, is counted
+        const uint32_t n = __hip_atomic_fetch_add(&p.hdr->fin_rows, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        if (n == gridDim.x - 1) {
+            a_store(&p.hdr->fin_rows, 0u);
+            int32_t *hint = p.hdr->hint;
+            if (hint)
+                __hip_atomic_store(hint, a_load(&p.hdr->n_need) * 2u > gridDim.x ? 1 : 0, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+    }
+}
+
 // Launch-plus-one-read floor: same grid, each row read once, one int out.
 template <int R>
 __global__ void __launch_bounds__(kThreads) floor_kernel(const float *logits, int64_t row_stride, int32_t *out,
@@ -1641,19 +1668,56 @@ static size_t stream_bytes(int32_t B, int32_t V)
     return longs > shorts ? longs : shorts;
 }
 
-// The streaming path (three launches, no waits) needs top_k to bound the kept
-// set.  Measured on MI355X it then beats the cluster kernel from 131072
-// tokens per call upwards (back to back: 15-17 us for small calls against
-// 16-31 us, 2-3 times faster for large ones); below that the single launch
-// wins by up to a microsecond.  RS_FORCE_PATH=cluster|stream overrides (tests).
-static bool choose_stream(int32_t B, int32_t V, int32_t top_k, bool pen, bool want_e, const Geometry &g)
+// Without a bounding top_k (nucleus sampling alone) the streaming path is an attempt: it works
+// when the nucleus is small (peaked distributions: the usual case with language models) and is a
+// wasted pass when it is not (flat ones).  How the last attempt on a workspace fared is reported by
+// the finishing kernel into a word of pinned host memory, which rs_sample looks at -- without
+// waiting for anything -- before the next call: after a failed attempt such calls go straight to
+// the cluster kernel, and one in 64 tries again.  Workspaces never given to rs_workspace_init have
+// no such word and are never used for attempts.
+struct Hint { int32_t *word; uint32_t calls; };
+static std::mutex g_hint_mu;
+static std::unordered_map<const void *, Hint> g_hints;
+
+static Hint *hint_of(const void *ws, bool create)
 {
-    const bool eligible = !pen && !want_e && top_k <= kStreamK;
+    std::lock_guard<std::mutex> lock(g_hint_mu);
+    auto it = g_hints.find(ws);
+    if (it != g_hints.end()) return &it->second;
+    if (!create) return nullptr;
+    int32_t *word = nullptr;
+    if (hipHostMalloc((void **)&word, 64, hipHostMallocDefault) != hipSuccess || !word) return nullptr;
+    *word = 0;
+    Hint h;
+    h.word = word; h.calls = 0;
+    return &g_hints.emplace(ws, h).first->second;
+}
+
+// The streaming path (three launches, no waits) is certain to work when top_k
+// bounds the kept set.  Measured on MI355X it then beats the cluster kernel
+// from 131072 tokens per call upwards (back to back: 15-17 us for small calls
+// against 16-31 us, 2-3 times faster for large ones); below that the single
+// launch wins by up to a microsecond.  RS_FORCE_PATH=cluster|stream|optimistic
+// overrides (tests).
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2 };
+static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pen, bool want_e, const void *ws, hipStream_t st)
+{
+    if (pen || want_e) return kPathCluster;
+    const bool bounded = top_k <= kStreamK;
     const char *force = getenv("RS_FORCE_PATH");
-    if (force && force[0] == 'c') return false;
-    if (force && force[0] == 's') return eligible;
-    (void)g;
-    return eligible && (uint64_t)B * (uint64_t)V >= (1ull << 17);
+    if (force && force[0] == 'c') return kPathCluster;
+    if (force && force[0] == 's') return bounded ? kPathStream : kPathCluster;
+    if (force && force[0] == 'o') return bounded ? kPathStream : kPathAttempt;
+    if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
+    if (bounded) return kPathStream;
+    if (!(top_p < 1.0f)) return kPathCluster;                  // everything is kept: nothing a stash could hold
+    Hint *h = hint_of(ws, false);
+    if (!h) return kPathCluster;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone)
+        return kPathCluster;                                    // a captured choice could not follow the reports
+    const bool failing = *(volatile int32_t *)h->word != 0;
+    return (!failing || (++h->calls & 63u) == 0u) ? kPathAttempt : kPathCluster;
 }
 
 template <bool PEN>
@@ -1741,6 +1805,14 @@ int rs_workspace_init(void *ws, size_t bytes, void *stream)
     if (!ws) return RS_ERR_NULL;
     if (bytes < sizeof(WsHeader) || ((uintptr_t)ws & 255)) return RS_ERR_WORKSPACE;
     if (hipMemsetAsync(ws, 0, bytes, (hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
+    // the word of pinned host memory attempts are reported to (see choose_path)
+    if (Hint *hint = hint_of(ws, true)) {
+        *hint->word = 0;
+        hint->calls = 0;
+        WsHeader *h = (WsHeader *)ws;
+        if (hipMemcpyAsync(&h->hint, &hint->word, sizeof hint->word, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess)
+            return RS_ERR_LAUNCH;
+    }
     // test hook: RS_SPIN_LIMIT_MS shortens the bound of the waits (default 2000 ms)
     if (const char *ms = getenv("RS_SPIN_LIMIT_MS")) {
         const long v = atol(ms);
@@ -1763,6 +1835,14 @@ int rs_workspace_status(const void *ws, int32_t *status, void *stream)
     if (hipMemcpyAsync(&e, &h->error, sizeof e, hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
     if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
     *status = e;
+    return RS_OK;
+}
+
+int rs_workspace_policy(const void *ws, int32_t *state)
+{
+    if (!ws || !state) return RS_ERR_NULL;
+    const Hint *h = hint_of(ws, false);
+    *state = h ? (*(volatile int32_t *)h->word != 0 ? 1 : 0) : -1;
     return RS_OK;
 }
 
@@ -1804,7 +1884,8 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     p.top_k = top_k; p.top_p = top_p;
     p.need = nullptr; p.stash_k = (uint32_t)top_k;
     dim3 grid((uint32_t)B * g.G);
-    if (choose_stream(B, V, top_k, pen, e_bits != nullptr, g)) {
+    const int path = choose_path(B, V, top_k, top_p, pen, e_bits != nullptr, workspace, (hipStream_t)stream);
+    if (path != kPathCluster) {
         const int sr = stream_r(B, V);
         StreamView v;
         v.G = stream_parts(V, sr);
@@ -1812,14 +1893,18 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         char *w = (char *)workspace;
         v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.need = (uint32_t *)(w + l.need);
-        p.stash_k = (uint32_t)top_k < 128u ? (uint32_t)top_k : min((uint32_t)top_k, max(128u, 8u * (uint32_t)top_k / v.G));
+        // without a bounding top_k the stashes are sized as for top_k = kStreamK: enough for a nucleus
+        // of up to about a thousand tokens
+        const uint32_t kk = min((uint32_t)top_k, (uint32_t)kStreamK);
+        p.stash_k = kk < 128u ? kk : min(kk, max(128u, 8u * kk / v.G));
         hipStream_t st = (hipStream_t)stream;
         // The finishing workgroup's list: twice what a well-behaved row needs (its top_k tokens and
         // a boundary bin, or every stash whole), as a power of two; a row that needs more is handed
         // on.  Kept small where it can be: the list is LDS, and LDS decides how many rows finish at once.
-        const uint32_t est = 2u * max((uint32_t)top_k + 512u, v.G * (p.stash_k + 64u));
+        const uint32_t est = 2u * max(kk + 512u, v.G * (p.stash_k + 64u));
         v.list_cap = 2048u;
         while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
+        v.attempt = path == kPathAttempt ? 1u : 0u;
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (sr == 4) {
             hipLaunchKernelGGL((stream_kernel<4, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);

@@ -8,6 +8,7 @@
 // include/rapid_sampling.h.  PyTorch supplies device memory and the current
 // stream, nothing else.
 #include <torch/extension.h>
+#include <hip/hip_runtime_api.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
@@ -47,7 +48,17 @@ at::Tensor &workspace_for(const at::Tensor &like, void *stream, int64_t B, int64
         size_t bytes = 0;
         rs_workspace_bytes((int32_t)e.B, (int32_t)e.V, &bytes);
         if (e.ws.defined()) e.retired.push_back(e.ws);
-        e.ws = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        const bool capturing = hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
+        if (capturing) {
+            // a memset must not be recorded into a graph: clear with a fill kernel, and do without
+            // the routing reports rs_workspace_init would set up
+            e.ws = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
+        } else {
+            e.ws = at::empty({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
+            const int rc = rs_workspace_init(e.ws.data_ptr(), bytes, stream);
+            if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
+        }
     }
     return e.ws;
 }

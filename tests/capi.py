@@ -35,6 +35,8 @@ def lib():
                                         C.POINTER(f32), C.POINTER(i32), C.POINTER(f32)]
         L.rs_workspace_bytes.restype = C.c_int
         L.rs_workspace_bytes.argtypes = [i32, i32, C.POINTER(sz)]
+        L.rs_workspace_policy.restype = C.c_int
+        L.rs_workspace_policy.argtypes = [vp, C.POINTER(C.c_int32)]
         L.rs_workspace_init.restype = C.c_int
         L.rs_workspace_init.argtypes = [vp, sz, vp]
         L.rs_workspace_status.restype = C.c_int

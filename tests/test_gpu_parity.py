@@ -68,8 +68,9 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
         _check(res2, ref_out, ref_diag, what + " (second call)")
         if pen_np is None:
             # the wait-free streaming path (taken for top_k <= 1024; rows it cannot finish go on to
-            # the cluster kernel), then the cluster path again on the workspace it leaves behind
-            for path in ("stream", "cluster"):
+            # the cluster kernel), the same attempted whatever top_k is, then the cluster path again
+            # on the workspace these leave behind
+            for path in ("stream", "optimistic", "cluster"):
                 os.environ["RS_FORCE_PATH"] = path
                 res3 = smp.sample(lg, c, k, p, uniforms=u)
                 _check(res3, ref_out, ref_diag, what + " (path %s)" % path)
@@ -438,6 +439,57 @@ def test_python_module_drop_in_calls(torch_cuda, oracle):
         out = sample.batch_sampling_temperature_topk_topp(logits=lg, states=states, temperature=temp, top_k=k_in,
                                                           top_p=p_in, uniforms=torch.from_numpy(u_np).cuda())
         assert np.array_equal(out.cpu().numpy(), ref_out)
+
+
+def test_nucleus_only_calls_are_routed_by_reports(torch_cuda, oracle):
+    """top_k disabled, top_p < 1: the wait-free path is an attempt.  On a workspace set up by
+    rs_workspace_init it is made; peaked rows finish on it (diag.rounds == 0).  After a call whose rows
+    mostly had to be handed on (flat rows) the report word says so and the next calls go straight to the
+    general kernel; a workspace that was only zeroed is never used for attempts.  Every result equals the
+    oracle's whatever the route."""
+    torch = torch_cuda
+    import ctypes as C
+    from tests import capi
+    B, V = 16, 65536
+    peaked = H.logits_normal(B, V, 3.0, seed=90)
+    flat = H.logits_uniform(B, V, seed=91)
+    rc, c, k, p = capi.normalize(1.0, -1, 0.3, V, B, 1)
+    assert k == V
+    u_np = H.uniforms(B, 92)
+    u = torch.from_numpy(u_np).cuda()
+    ref_peaked = oracle.sample_batch(peaked, c, k, p, injected_u=u_np)
+    ref_flat = oracle.sample_batch(flat, c, k, p, injected_u=u_np)
+    lg_peaked, lg_flat = torch.from_numpy(peaked).cuda(), torch.from_numpy(flat).cuda()
+
+    def policy(smp):
+        st = C.c_int32(-5)
+        assert capi.lib().rs_workspace_policy(smp.ws.data_ptr(), C.byref(st)) == 0
+        return st.value
+
+    plain = capi.Sampler(B, V)                           # zeroed by torch: no report word
+    assert policy(plain) == -1
+    res = plain.sample(lg_peaked, c, k, p, uniforms=u)
+    _check(res, *ref_peaked, "zeroed workspace")
+    assert (res["diag"]["rounds"] >= 1).all()            # general kernel
+
+    smp = capi.Sampler(B, V)
+    assert capi.lib().rs_workspace_init(smp.ws.data_ptr(), smp.ws.numel(), smp.stream()) == 0
+    assert policy(smp) == 0
+    res = smp.sample(lg_peaked, c, k, p, uniforms=u)
+    _check(res, *ref_peaked, "attempt on peaked rows")
+    assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
+    res = smp.sample(lg_flat, c, k, p, uniforms=u)       # attempted, every row handed on
+    _check(res, *ref_flat, "attempt on flat rows")
+    assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 1
+    for i in range(3):                                   # no further attempts for now, peaked or not
+        res = smp.sample(lg_peaked, c, k, p, uniforms=u)
+        _check(res, *ref_peaked, "after a failed attempt %d" % i)
+        assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 1
+    for i in range(70):                                  # one call in 64 tries again and finds peaked rows
+        res = smp.sample(lg_peaked, c, k, p, uniforms=u, want_diag=False)
+        assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
+    assert policy(smp) == 0
+    assert smp.status() == 0
 
 
 def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
