@@ -1033,6 +1033,28 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
     leave_launch(p.hdr);
 }
 
+// The same for a launch of one workgroup per slice of every row of the batch:
+// each takes one ticket, those beyond the list leave at once.  Used behind an
+// attempt, after which the list may hold every row.
+template <int R>
+__global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list_once_kernel(const Params p)
+{
+    __shared__ Lds s;
+    const uint32_t n = a_load(&p.hdr->n_need);
+    if (n == 0u) return;                                         // nothing left over: no ticket was taken
+    if (threadIdx.x == 0) {
+        s.abort = 0;
+        const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
+        if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);     // the last ticket of the launch
+        s.bc32[0] = t;
+    }
+    __syncthreads();
+    const uint32_t ticket = s.bc32[0];
+    const uint32_t slot = ticket / p.G;
+    if (slot >= n) return;
+    sample_slice<R, false>(p, s, p.need[slot], ticket - slot * p.G);
+}
+
 // ---------------------------------------------------------- streaming path --
 // For large batches with a small top_k the cluster kernel's exchanges cost
 // more than the data movement.  The streaming path has no waits at all:
@@ -1125,6 +1147,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         }
     }
     if (tid < kSB) s.hm[tid] = 0;
+    if (blockIdx.x == 0 && tid == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
     uint32_t k = wave_max_u32(fkey(lmax));
     if (lane == 0) s.u32[wave] = k;
     __syncthreads();
@@ -1736,8 +1759,19 @@ static hipError_t launch_sample(int R, dim3 grid, hipStream_t st, const Params &
     return hipGetLastError();
 }
 
-static hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p)
+static hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p, bool once)
 {
+    if (once) {
+        switch (R) {
+        case 1:  hipLaunchKernelGGL((sample_list_once_kernel<1>),  grid, dim3(kThreads), 0, st, p); break;
+        case 2:  hipLaunchKernelGGL((sample_list_once_kernel<2>),  grid, dim3(kThreads), 0, st, p); break;
+        case 4:  hipLaunchKernelGGL((sample_list_once_kernel<4>),  grid, dim3(kThreads), 0, st, p); break;
+        case 8:  hipLaunchKernelGGL((sample_list_once_kernel<8>),  grid, dim3(kThreads), 0, st, p); break;
+        case 16: hipLaunchKernelGGL((sample_list_once_kernel<16>), grid, dim3(kThreads), 0, st, p); break;
+        default: hipLaunchKernelGGL((sample_list_once_kernel<32>), grid, dim3(kThreads), 0, st, p); break;
+        }
+        return hipGetLastError();
+    }
     switch (R) {
     case 1:  hipLaunchKernelGGL((sample_list_kernel<1>),  grid, dim3(kThreads), 0, st, p); break;
     case 2:  hipLaunchKernelGGL((sample_list_kernel<2>),  grid, dim3(kThreads), 0, st, p); break;
@@ -1915,9 +1949,13 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         }
         if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
         p.need = v.need;               // the cluster kernel follows for the rows the finish left over
-        if (grid.x > 1024u) grid.x = 1024u / g.G * g.G > 0 ? 1024u / g.G * g.G : g.G;
+        // Workgroups for the rows handed on.  Few rows are expected when top_k bounds the kept set: a
+        // small grid whose workgroups take tickets until the list is exhausted.  After an attempt it
+        // may be all of them: one workgroup per slice of every row, as in the cluster kernel; those
+        // beyond the list leave at once.
+        if (path == kPathStream && grid.x > 1024u) grid.x = 1024u / g.G * g.G > 0 ? 1024u / g.G * g.G : g.G;
     }
-    const hipError_t e = p.need ? launch_list(g.R, grid, (hipStream_t)stream, p)
+    const hipError_t e = p.need ? launch_list(g.R, grid, (hipStream_t)stream, p, path == kPathAttempt)
                        : pen ? launch_sample<true>(g.R, grid, (hipStream_t)stream, p)
                              : launch_sample<false>(g.R, grid, (hipStream_t)stream, p);
     return e == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
