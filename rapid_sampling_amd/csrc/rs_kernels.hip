@@ -1935,7 +1935,8 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         // The finishing workgroup's list: twice what a well-behaved row needs (its top_k tokens and
         // a boundary bin, or every stash whole), as a power of two; a row that needs more is handed
         // on.  Kept small where it can be: the list is LDS, and LDS decides how many rows finish at once.
-        const uint32_t est = 2u * max(kk + 512u, v.G * (p.stash_k + 64u));
+        const uint32_t whole = v.G * (p.stash_k + 64u);            // every stash whole; of no use beyond kFinCap
+        const uint32_t est = 2u * max(kk + 512u, whole <= (uint32_t)kFinCap ? whole : 0u);
         v.list_cap = 2048u;
         while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
         v.attempt = path == kPathAttempt ? 1u : 0u;
