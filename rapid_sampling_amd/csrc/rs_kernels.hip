@@ -1303,9 +1303,10 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
 struct LdsB {
     uint64_t *list;              // gathered tokens, row frame: bits << 32 | index (dynamic LDS, v.list_cap entries)
     uint64_t blo[kMaxParts], bhi[kMaxParts];
-    uint64_t small[128];
+    uint64_t small[64];
     uint32_t delta[kMaxParts];   // octaves between the row's frame and slice g's
     uint32_t take[kMaxParts];    // inclusive prefix of the entries taken from each stash
+    uint64_t rand64;
     uint32_t nsmall, bucket, fail;
 };
 
@@ -1359,9 +1360,26 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.cut = 0;
     if ((uint32_t)tid < G) ph = hdrs[tid];
     const uint64_t h0 = rowhist[tid], h1 = rowhist[tid + kThreads];
+    // the first lane of wave 1 draws the row's random number while wave 0 scans the histogram;
+    // the state is advanced only once the row is certain to be finished here
+    const bool drawer = tid == kWave && !p.inj_u;
+    uint32_t *rng_st = p.rng + (size_t)row * 16;
+    uint32_t rs[6] = {0u, 0u, 0u, 0u, 0u, 0u};
+    if (drawer) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) rs[i] = rng_st[i];
+    }
     rowhist[tid] = 0; rowhist[tid + kThreads] = 0;                   // left clean for the next call
-    const uint32_t kmax = block_max_u32(s, ph.mkey, lane, wave);
-    const uint32_t kmin = ~block_max_u32(s, (uint32_t)tid < G ? ~ph.mkey : 0u, lane, wave);
+    uint32_t kmax, kmin;
+    {
+        const uint32_t a = wave_max_u32(ph.mkey), b = wave_max_u32((uint32_t)tid < G ? ~ph.mkey : 0u);
+        if (lane == 0) { s.u32[wave] = a; s.u32[kWaves + wave] = b; }
+        __syncthreads();
+        kmax = s.u32[0]; kmin = s.u32[kWaves];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) { kmax = max(kmax, s.u32[w]); kmin = max(kmin, s.u32[kWaves + w]); }
+        kmin = ~kmin;
+    }
     const float xmax = fkey_inv(kmax);
     const float M = __builtin_floorf(xmax);
     // frames further apart than this may have put different octaves into one bin
@@ -1387,6 +1405,11 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         if (tid == 0) s.g[kBin0] += (uint64_t)low << 43;
     }
     __syncthreads();
+    if (drawer) {
+        uint32_t o[4];
+        philox4x32_10(rs[2], rs[3], rs[4], rs[5], rs[0], rs[1], o);
+        t.rand64 = ((uint64_t)o[0] << 32) | o[1];
+    }
     const uint64_t top_k = (uint64_t)p.top_k;
     Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
@@ -1516,18 +1539,12 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         lo = s.bc32[6];
     }
     const uint32_t thr = lo;
+    if (drawer) {                                        // the row is finished here: this draw is used up
+        rng_st[2] = rs[2] + 1u;
+        if (rs[2] + 1u == 0u) rng_st[3] = rs[3] + 1u;
+    }
     if (tid == 0) {
-        uint64_t rand64 = 0;
-        if (!p.inj_u) {
-            uint32_t *st = p.rng + (size_t)row * 16;
-            uint32_t o[4];
-            philox4x32_10(st[2], st[3], st[4], st[5], st[0], st[1], o);
-            rand64 = ((uint64_t)o[0] << 32) | o[1];
-            const uint32_t lo32 = st[2] + 1;
-            st[2] = lo32;
-            if (lo32 == 0) st[3] += 1;
-        }
-        const Target tg = tie_and_target(p, row, rand64, xmax, D, P, thr, f.cnt_above, f.cnt_bin, f.mass_above, 0u, true);   // rounds = 0: no cluster histogram
+        const Target tg = tie_and_target(p, row, p.inj_u ? 0ull : t.rand64, xmax, D, P, thr, f.cnt_above, f.cnt_bin, f.mass_above, 0u, true);   // rounds = 0: no cluster histogram
         s.bc64[1] = tg.w_tie; s.bc128[0] = tg.r;
     }
     __syncthreads();
@@ -1537,32 +1554,63 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
 
     // inverse CDF in index order: slice, then run of tokens, then token
     constexpr uint32_t sh_slice = SLICE_LOG2;
-    constexpr uint32_t sh_run = sh_slice - 8;                                  // 256 runs of at most 128 tokens
-    static_assert(SLICE_LOG2 >= 8 && SLICE_LOG2 <= 15, "runs must fit the final all-pairs step");
+    constexpr uint32_t sh_run = sh_slice - 8;                                  // 256 runs of at most 64 tokens
+    static_assert(SLICE_LOG2 >= 8 && SLICE_LOG2 <= 14, "runs must fit the final all-pairs step");
     const uint32_t ga = bucket_step(s, t, total, sh_slice, 0u, 0xFFFFFFFFu, r, weight, lane, wave);
-    const uint32_t lo_a = ga << sh_slice;
-    const uint32_t gb = bucket_step(s, t, total, sh_run, lo_a, lo_a + (1u << sh_slice), r, weight, lane, wave);
-    const uint32_t lo_b = lo_a + (gb << sh_run);
-    if (tid == 0) t.nsmall = 0;
-    __syncthreads();
-    for (uint32_t i = tid; i < total; i += kThreads) {
-        const uint64_t e = t.list[i];
-        const uint32_t idx = (uint32_t)e;
-        if (idx >= lo_b && idx < lo_b + (1u << sh_run) && weight((uint32_t)(e >> 32))) {
-            const uint32_t o = atomicAdd(&t.nsmall, 1u);
-            if (o < 128u) t.small[o] = e;
+    constexpr uint32_t kPairs = 64;
+    uint32_t lo_b = ga << sh_slice, len_b = 1u << sh_slice;
+    // the kept tokens of that slice: few enough for the all-pairs step as they are, as a rule;
+    // otherwise the slice is narrowed to one of its 256 runs first
+    auto collect = [&]() {
+        if (tid == 0) t.nsmall = 0;
+        __syncthreads();
+        for (uint32_t i = tid; i < total; i += kThreads) {
+            const uint64_t e = t.list[i];
+            const uint32_t idx = (uint32_t)e;
+            if (idx - lo_b < len_b && weight((uint32_t)(e >> 32))) {
+                const uint32_t o = atomicAdd(&t.nsmall, 1u);
+                if (o < kPairs) t.small[o] = e;
+            }
         }
+        __syncthreads();
+        return t.nsmall;
+    };
+    uint32_t nkept = collect();
+    if (nkept > kPairs) {
+        __syncthreads();                                                       // everyone has read the count
+        const uint32_t gb = bucket_step(s, t, total, sh_run, lo_b, lo_b + len_b, r, weight, lane, wave);
+        lo_b += gb << sh_run; len_b = 1u << sh_run;
+        nkept = collect();
+    }
+    // all pairs: every kept token of the range adds up the weights at or before it in index order;
+    // the four waves take a quarter of the addends each
+    static_assert(kWaves == 4 && offsetof(Lds, cand) % 16 == 0 && sizeof(s.cand) >= 64 * 16 + 4 * 64 * 16, "records and partial sums live in s.cand");
+    const uint32_t ns = min(nkept, kPairs);
+    uint4 *rec = reinterpret_cast<uint4 *>(s.cand);                             // weight (x, y), index (z)
+    u128 *partial = reinterpret_cast<u128 *>(s.cand) + kPairs;
+    uint64_t me = 0, wme = 0;
+    if ((uint32_t)tid < ns) {
+        me = t.small[tid];
+        wme = weight((uint32_t)(me >> 32));
+        rec[tid] = make_uint4((uint32_t)wme, (uint32_t)(wme >> 32), (uint32_t)me, 0u);
     }
     __syncthreads();
-    const uint32_t ns = min(t.nsmall, 128u);
-    if ((uint32_t)tid < ns) {
-        const uint64_t me = t.small[tid];
-        const uint64_t wme = weight((uint32_t)(me >> 32));
-        u128 upto = 0;
-        for (uint32_t j = 0; j < ns; ++j) {
-            const uint64_t o = t.small[j];
-            if ((uint32_t)o <= (uint32_t)me) upto += weight((uint32_t)(o >> 32));
+    {
+        const uint32_t per = (ns + 3u) >> 2, j0 = (uint32_t)wave * per, j1 = min(ns, j0 + per);
+        const uint32_t mine = (uint32_t)lane < ns ? rec[lane].z : 0u;
+        uint64_t lo32 = 0, hi32 = 0;                                              // halves summed apart: no carries
+#pragma unroll 4
+        for (uint32_t j = j0; j < j1; ++j) {
+            const uint4 o = rec[j];
+            const bool c = o.z <= mine;
+            lo32 += c ? o.x : 0u;
+            hi32 += c ? o.y : 0u;
         }
+        partial[wave * (int)kPairs + lane] = (u128)lo32 + ((u128)hi32 << 32);
+    }
+    __syncthreads();
+    if ((uint32_t)tid < ns) {
+        const u128 upto = partial[tid] + partial[kPairs + tid] + partial[2 * kPairs + tid] + partial[3 * kPairs + tid];
         if (upto - wme < r && r <= upto) {
             p.out[row] = (int32_t)(uint32_t)me;
             if (p.diag) p.diag[row].index = (int32_t)(uint32_t)me;
