@@ -33,22 +33,28 @@ constexpr uint32_t kEMinBits = 0x2B800000u;               // bit pattern of 2^-4
 // exp2f(x - max) at sampling.cu:235; the common factor 2^(max - M) cancels in
 // every probability).  n = floor(x) and f = x - n are exact; 2^f is a degree-5
 // Horner polynomial with positive coefficients (monotone, poly(1) < 2); the
-// exponent n - M is added to the exponent field and the result is clamped
-// from below at 2^-40.  The significand depends on x alone, so a slice can
-// use its own M and be re-based later by an exponent shift.
+// result is scaled by 2^(n - M), n - M <= 0, and clamped from below at 2^-40.
+// The significand depends on x alone, so a slice can use its own M and be
+// re-based later by an exponent shift.
+//
+// This is the inner loop of every kernel, and the vector ALU is what bounds
+// the streaming pass once the logits arrive fast enough, so the instruction
+// count is kept down by hand: the Horner steps with a literal addend are
+// written as v_fmaak_f32 (the compiler otherwise spends a move per step on
+// some of them), and the scaling is v_cvt_i32_f32 (which saturates) +
+// v_ldexp_f32 (exact; anything below 2^-40, zero included, ends at the clamp).
 __device__ __forceinline__ uint32_t e_bits_of(float x, float M)
 {
     const float n = __builtin_floorf(x);
     const float f = x - n;
-    float p = 0x1.e974fap-10f;
-    p = __builtin_fmaf(p, f, 0x1.277856p-7f);
-    p = __builtin_fmaf(p, f, 0x1.c91ce6p-5f);
-    p = __builtin_fmaf(p, f, 0x1.ebdb56p-3f);
-    p = __builtin_fmaf(p, f, 0x1.62e4bap-1f);
+    float p = __builtin_fmaf(0x1.e974fap-10f, f, 0x1.277856p-7f);
+    asm("v_fmaak_f32 %0, %1, %2, 0x3d648e73" : "=v"(p) : "v"(p), "v"(f));      // p * f + 0x1.c91ce6p-5
+    asm("v_fmaak_f32 %0, %1, %2, 0x3e75edab" : "=v"(p) : "v"(p), "v"(f));      // p * f + 0x1.ebdb56p-3
+    asm("v_fmaak_f32 %0, %1, %2, 0x3f31725d" : "=v"(p) : "v"(p), "v"(f));      // p * f + 0x1.62e4bap-1
     p = __builtin_fmaf(p, f, 1.0f);
-    const float k = fmaxf(n - M, -41.0f);
-    const uint32_t b = __float_as_uint(p) + ((uint32_t)(int)k << 23);
-    return max(b, kEMinBits);
+    int k;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(k) : "v"(n - M));
+    return __float_as_uint(fmaxf(__builtin_ldexpf(p, k), 0x1p-40f));
 }
 
 // Exact weight of a token from the bit pattern of e (2^-40 <= e < 2):
