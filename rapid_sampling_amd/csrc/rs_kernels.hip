@@ -598,7 +598,8 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
             }
             probe = __builtin_fmaf(x[0], x[1], probe);
             probe = __builtin_fmaf(x[2], x[3], probe);
-            if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
+            // slots past the end of the row hold its last group again (same slice): harmless here
+            lmax = fmaxf(fmaxf(lmax, x[0]), fmaxf(x[1], fmaxf(x[2], x[3])));
         }
         const bool special = __builtin_amdgcn_classf(probe, kSpecial);
         if (special) {
@@ -1123,22 +1124,21 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     const float4 *lg = reinterpret_cast<const float4 *>(p.logits + (int64_t)row * p.row_stride);
 
     uint32_t eb[R * 4];                                 // x, then bits(e)
-#pragma unroll
-    for (int j = 0; j < R; ++j) {
-        const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
-        eb[j * 4 + 0] = __float_as_uint(l.x * p.c); eb[j * 4 + 1] = __float_as_uint(l.y * p.c);
-        eb[j * 4 + 2] = __float_as_uint(l.z * p.c); eb[j * 4 + 3] = __float_as_uint(l.w * p.c);
-    }
-    // x = l * c is the definition unless a NaN or Inf shows up (see sample_kernel)
+    // x = l * c is the definition unless a NaN or Inf shows up (see sample_kernel).  Slots past the
+    // end of the row read its last group again: harmless for the maximum and the probe, and they
+    // are set aside before the histogram.
     constexpr int kSpecial = 0x207;
     float probe = 0.0f;
     float lmax = -3.402823466e+38f;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-        probe = __builtin_fmaf(__uint_as_float(eb[j * 4]), __uint_as_float(eb[j * 4 + 1]), probe);
-        probe = __builtin_fmaf(__uint_as_float(eb[j * 4 + 2]), __uint_as_float(eb[j * 4 + 3]), probe);
-        if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(__uint_as_float(eb[j * 4]), __uint_as_float(eb[j * 4 + 1])),
-                                             fmaxf(__uint_as_float(eb[j * 4 + 2]), __uint_as_float(eb[j * 4 + 3]))));
+        const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
+        const float x0 = l.x * p.c, x1 = l.y * p.c, x2 = l.z * p.c, x3 = l.w * p.c;
+        probe = __builtin_fmaf(x0, x1, probe);
+        probe = __builtin_fmaf(x2, x3, probe);
+        lmax = fmaxf(fmaxf(lmax, x0), fmaxf(x1, fmaxf(x2, x3)));
+        eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
+        eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
     }
     if (__builtin_amdgcn_classf(probe, kSpecial)) {
         lmax = -3.402823466e+38f;
