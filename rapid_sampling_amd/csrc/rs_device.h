@@ -57,6 +57,22 @@ __device__ __forceinline__ uint32_t e_bits_of(float x, float M)
     return __float_as_uint(fmaxf(__builtin_ldexpf(p, k), 0x1p-40f));
 }
 
+// The same without the clamp: whatever lies below 2^-40 (zero included) stands for 2^-40.  For
+// code that can tell such tokens by their bin and saves the instruction.
+__device__ __forceinline__ uint32_t e_bits_raw(float x, float M)
+{
+    const float n = __builtin_floorf(x);
+    const float f = x - n;
+    float p = __builtin_fmaf(0x1.e974fap-10f, f, 0x1.277856p-7f);
+    asm("v_fmaak_f32 %0, %1, %2, 0x3d648e73" : "=v"(p) : "v"(p), "v"(f));
+    asm("v_fmaak_f32 %0, %1, %2, 0x3e75edab" : "=v"(p) : "v"(p), "v"(f));
+    asm("v_fmaak_f32 %0, %1, %2, 0x3f31725d" : "=v"(p) : "v"(p), "v"(f));
+    p = __builtin_fmaf(p, f, 1.0f);
+    int k;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(k) : "v"(n - M));
+    return __float_as_uint(__builtin_ldexpf(p, k));
+}
+
 // Exact weight of a token from the bit pattern of e (2^-40 <= e < 2):
 // W = e * 2^63 = significand24 << (exponent - 87), in [2^23, 2^64).
 __device__ __forceinline__ uint64_t w_of_bits(uint32_t b)

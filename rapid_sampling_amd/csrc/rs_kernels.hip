@@ -1101,14 +1101,27 @@ struct StreamView {
     uint32_t  attempt;    // 1: top_k does not bound the kept set; report how the rows fared
 };
 
+// Lanes of a wave that add to one LDS address are served one after the other, and rows often put
+// most of their tokens into a few bins.  So each bin is kept in kRep copies (lane l adds to copy
+// l % kRep), and e is not clamped at 2^-40 before it is counted: the histogram spans all 512
+// values of bits >> 21, the tokens below 2^-40 -- often most of a row -- spread over the bins
+// below kBin0 by their own exponents, and those bins hand their counts to bin kBin0 afterwards
+// (such a token weighs 2^-40 exactly: a count and no fraction bits).  The histogram is done with
+// before the candidates are staged, and shares their memory.
+constexpr int kRep = 8;
 struct LdsA {
-    uint4    grp[kStashCap];     // float4 groups that hold a candidate: bits of their 4 tokens
-    uint32_t gidx[kStashCap];    // and the index of their first token
-    uint64_t hm[kSB];
+    union {
+        uint64_t hm[kNB * kRep];     // the slice's bins by bits >> 21
+        struct {
+            uint4    grp[kStashCap];     // float4 groups that hold a candidate: bits of their 4 tokens
+            uint32_t gidx[kStashCap];    // and the index of their first token
+        };
+    };
     uint32_t off[kSB];
     uint32_t sub[128];           // level-2 counts inside a boundary bin too large for the stash
     uint32_t u32[16];
     uint32_t cov, n, cut, over;
+    uint32_t low;                // tokens of the slice below 2^-40
 };
 
 template <int R, int NT>     // NT threads, each with R float4 of the slice
@@ -1151,7 +1164,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    if (tid < kSB) s.hm[tid] = 0;
+    for (int i = tid; i < kNB * kRep; i += NT) s.hm[i] = 0;
+    if (tid == 0) s.low = 0;
     if (blockIdx.x == 0 && tid == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
     uint32_t k = wave_max_u32(fkey(lmax));
     if (lane == 0) s.u32[wave] = k;
@@ -1160,15 +1174,16 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     for (int w = 0; w < (NT / kWave); ++w) k = max(k, s.u32[w]);
     const float M = __builtin_floorf(fkey_inv(k));
 
-    // e in the slice's frame and its histogram; slots past the end of the row become 0, below any cut
+    // e in the slice's frame, not yet clamped at 2^-40, and its histogram; slots past the end of
+    // the row become 0
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         if (j < nv) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const uint32_t b = e_bits_of(__uint_as_float(eb[j * 4 + q]), M);
+                const uint32_t b = e_bits_raw(__uint_as_float(eb[j * 4 + q]), M);
                 eb[j * 4 + q] = b;
-                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) - kBin0]),
+                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) * kRep + (lane & (kRep - 1))]),
                           (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
             }
         } else {
@@ -1176,11 +1191,28 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         }
     }
     __syncthreads();
+    {
+        // the tokens below 2^-40: counted into bin kBin0
+        uint32_t low = 0;
+        for (int i = tid; i < (int)kBin0 * kRep; i += NT) low += pack_count(s.hm[i]);
+        low = wave_sum(low);
+        if (lane == 0 && low) {
+            atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[kBin0 * kRep]), (unsigned long long)low << 43);
+            atomicAdd(&s.low, low);
+        }
+    }
+    __syncthreads();
     // Add the slice's bins to the row's, which are kept by absolute octave (mod 128, 4 bins each):
     // bin t of this frame is octave M - 40 + t/4.  Slices of one row may use different frames; as
     // long as their maxima lie within 87 octaves of each other no two octaves in use coincide.
+    auto bin_total = [&](int b) {
+        uint64_t w = 0;
+#pragma unroll
+        for (int c = 0; c < kRep; ++c) w += s.hm[((int)kBin0 + b) * kRep + c];
+        return w;
+    };
     if (tid < kSB) {
-        const uint64_t w = s.hm[tid];
+        const uint64_t w = bin_total(tid);
         const float mm = M - 128.0f * __builtin_floorf(M * 0.0078125f);          // M mod 128, exact
         if (w) a_add(&(p.ctl_end - 1 - row)->rowhist[((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u], w);
     }
@@ -1197,7 +1229,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             const int b = kSB - 1 - 3 * lane - i;
-            c3[i] = b >= 0 ? pack_count(s.hm[b]) : 0u;
+            c3[i] = b >= 0 ? pack_count(bin_total(b)) : 0u;
             cs += c3[i];
         }
         const uint32_t ci = wave_inclusive_scan(cs);
@@ -1236,6 +1268,9 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
                 const uint32_t b = eb[j * 4 + q];
                 if ((b >> 21) == ob) atomicAdd(&s.sub[(b >> 14) & 127u], 1u);
             }
+        // in the lowest bin, the tokens below 2^-40 (not counted above: their bits say another bin)
+        // all weigh 2^-40 exactly
+        if (ob == kBin0 && tid == 0 && s.low) atomicAdd(&s.sub[0], s.low);
         __syncthreads();
         if (wave == 0) {
             const uint32_t Ks = p.stash_k;
@@ -1257,6 +1292,17 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     }
     const uint32_t cov = s.cov, n = s.n;
     const uint32_t cut = s.cut;
+    // From here on the bits in the registers are compared with the cut.  Above 2^-40 they are what
+    // they should be; if the cut lies at 2^-40 itself (the stash takes all of a slice, tokens
+    // down there included) they are clamped first.
+    if (cut == kEMinBits) {
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+            if (j < nv) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) eb[j * 4 + q] = max(eb[j * 4 + q], kEMinBits);
+            }
+    }
 
     // Candidates (bits >= cut) are at most n <= kStashCap, so at most that many float4 groups
     // hold one.  Each thread copies its groups with a candidate into LDS at an offset from a scan
