@@ -107,14 +107,19 @@ int rs_workspace_init(void *workspace_device, size_t bytes, void *stream);
 int rs_workspace_status(const void *workspace_device, int32_t *status, void *stream);
 
 /*
- * Diagnostic: how calls WITHOUT a bounding top_k (top_k > 1024 or disabled, top_p < 1) are
- * currently routed on this workspace.  Such a call may be attempted on the
- * wait-free path, which works when the nucleus is small; the finishing kernel
- * reports each attempt to a word of pinned host memory that rs_sample reads,
- * without waiting, before the next call.  *state: -1 the workspace was not set
- * up by rs_workspace_init (never attempted), 0 attempts are made, 1 the last
- * attempt handed most rows on: calls go to the general kernel, one in 64 tries
- * again.  Results do not depend on the routing.  No counterpart in the reference.
+ * Diagnostic: how calls that could take the wait-free streaming path are
+ * currently routed on this workspace.  A row that path cannot finish is handed
+ * to the general kernel in a further launch, and a call whose rows mostly end
+ * that way has wasted a pass: with a bounding top_k (<= 1024) that takes
+ * unusual rows (ties of thousands of tokens, slices of a row more than 87
+ * octaves apart), without one (top_p < 1 alone) a flat distribution.  Each
+ * streaming call reports "most rows handed on: yes/no" to a word of pinned
+ * host memory that rs_sample reads, without waiting, before the next call.
+ * *state: -1 the workspace was not set up by rs_workspace_init (calls with a
+ * bounding top_k always stream, calls without never do); otherwise bit 0 set:
+ * calls without a bounding top_k currently go to the general kernel, bit 1
+ * set: so do calls with one; in both cases one call in 64 streams again.
+ * Results do not depend on the routing.  No counterpart in the reference.
  */
 int rs_workspace_policy(const void *workspace_device, int32_t *state);
 

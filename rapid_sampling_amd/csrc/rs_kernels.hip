@@ -61,9 +61,8 @@ struct alignas(256) WsHeader {
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows the streaming pass handed to the cluster kernel
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
-    uint32_t fin_rows;    // rows the finishing kernel is through with (attempts without a bounding top_k only)
-    uint32_t pad0;
-    int32_t *hint;        // pinned host word the finishing kernel reports such an attempt to, or null
+    uint32_t pad0[2];
+    int32_t *hint;        // two words of pinned host memory the streaming path reports to, or null
     uint32_t pad[54];
 };
 
@@ -106,6 +105,7 @@ struct Params {
     RowCtl      *ctl_end;      // one past the record of row 0; row r is ctl_end[-1 - r]
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
+    uint32_t     report;       // which of the two report words a streaming call writes: 0 top_k bounds the kept set, 1 not
     int64_t      row_stride;
     int32_t      B, V;
     uint32_t     G;            // workgroups per row
@@ -1016,6 +1016,19 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     sample_slice<R, PEN>(p, s, row, ticket - row * p.G);
 }
 
+// The launch that follows the streaming pass knows how many rows were handed on.  Its first
+// workgroup tells the host -- a word of pinned memory that rs_sample looks at, without waiting,
+// before its next call -- whether that was most of them: such calls are then better served by
+// the cluster kernel alone for a while.
+__device__ __forceinline__ void report_streaming(const Params &p, uint32_t handed_on)
+{
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        int32_t *hint = p.hdr->hint;
+        if (hint)
+            __hip_atomic_store(hint + p.report, handed_on * 2u > (uint32_t)p.B ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
 // The launch that follows the streaming pass: workgroups work through the
 // rows on its list, taking tickets until the list is exhausted.
 template <int R>
@@ -1023,7 +1036,9 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
 {
     __shared__ Lds s;
     const uint32_t G = p.G;
-    if (a_load(&p.hdr->n_need) == 0u) return;                    // nothing left over: no ticket was taken
+    const uint32_t n = a_load(&p.hdr->n_need);
+    report_streaming(p, n);
+    if (n == 0u) return;                                         // nothing left over: no ticket was taken
     for (;;) {
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -1047,6 +1062,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
 {
     __shared__ Lds s;
     const uint32_t n = a_load(&p.hdr->n_need);
+    report_streaming(p, n);
     if (n == 0u) return;                                         // nothing left over: no ticket was taken
     if (threadIdx.x == 0) {
         s.abort = 0;
@@ -1098,7 +1114,6 @@ struct StreamView {
     uint32_t *need;       // [B]  rows left to the cluster kernel
     uint32_t  G;          // slices per row
     uint32_t  list_cap;   // entries of the finishing workgroup's token list (a power of two up to kFinCap)
-    uint32_t  attempt;    // 1: top_k does not bound the kept set; report how the rows fared
 };
 
 // Lanes of a wave that add to one LDS address are served one after the other, and rows often put
@@ -1677,20 +1692,6 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     extern __shared__ __align__(16) unsigned char finish_dyn[];
     t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value
     finish_row<SLICE_LOG2>(p, v, s, t, blockIdx.x);
-    // An attempt without a bounding top_k: the workgroup that is through last tells the host (a
-    // word of pinned memory it looks at before its next call) whether most rows had to be handed
-    // on -- then such calls are better not attempted for a while.
-    if (v.attempt && threadIdx.x == 0) {
-        wait_vmem();                                         // my row's entry in the list, if any, is counted
-        const uint32_t n = __hip_atomic_fetch_add(&p.hdr->fin_rows, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        if (n == gridDim.x - 1) {
-            a_store(&p.hdr->fin_rows, 0u);
-            int32_t *hint = p.hdr->hint;
-            if (hint)
-                __hip_atomic_store(hint, a_load(&p.hdr->n_need) * 2u > gridDim.x ? 1 : 0, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_SYSTEM);
-        }
-    }
 }
 
 // Launch-plus-one-read floor: same grid, each row read once, one int out.
@@ -1762,6 +1763,7 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
 // be cut into more slices than a finishing workgroup handles quickly).
 constexpr int kStreamNT = 256;
 constexpr uint64_t kStreamSmall = 1ull << 22;
+constexpr uint32_t kListGrid = 256;            // workgroups of the launch for the rows handed on (they loop)
 static int stream_r(int32_t B, int32_t V) { return (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144 ? 4 : 16; }
 static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -1790,14 +1792,19 @@ static size_t stream_bytes(int32_t B, int32_t V)
     return longs > shorts ? longs : shorts;
 }
 
-// Without a bounding top_k (nucleus sampling alone) the streaming path is an attempt: it works
-// when the nucleus is small (peaked distributions: the usual case with language models) and is a
-// wasted pass when it is not (flat ones).  How the last attempt on a workspace fared is reported by
-// the finishing kernel into a word of pinned host memory, which rs_sample looks at -- without
-// waiting for anything -- before the next call: after a failed attempt such calls go straight to
-// the cluster kernel, and one in 64 tries again.  Workspaces never given to rs_workspace_init have
-// no such word and are never used for attempts.
-struct Hint { int32_t *word; uint32_t calls; };
+// The streaming path works when the kept set is small next to the row and the slices of a row
+// share a frame; a row for which it does not is handed to the cluster kernel in a third launch,
+// and a call whose rows mostly end that way has wasted a pass.  With a bounding top_k that takes
+// unusual rows (ties of thousands of tokens, slices more than 87 octaves apart); without one
+// (nucleus sampling alone) it is simply a flat distribution, so such a call is an attempt.  The
+// launch for the rows handed on reports "most of them: yes/no" into a word of pinned host memory
+// that belongs to the workspace, one word for calls with a bounding top_k and one for calls
+// without, and rs_sample looks at the word -- without waiting for anything; a stale value only
+// delays the switch -- before it chooses the path of the next call: after a call that handed
+// most rows on, calls of that kind go straight to the cluster kernel and one in 64 streams again.
+// Workspaces never given to rs_workspace_init have no such words: with a bounding top_k they
+// always stream, without one they never do.
+struct Hint { int32_t *word; uint32_t calls[2]; };
 static std::mutex g_hint_mu;
 static std::unordered_map<const void *, Hint> g_hints;
 
@@ -1809,18 +1816,16 @@ static Hint *hint_of(const void *ws, bool create)
     if (!create) return nullptr;
     int32_t *word = nullptr;
     if (hipHostMalloc((void **)&word, 64, hipHostMallocDefault) != hipSuccess || !word) return nullptr;
-    *word = 0;
+    word[0] = 0; word[1] = 0;
     Hint h;
-    h.word = word; h.calls = 0;
+    h.word = word; h.calls[0] = 0; h.calls[1] = 0;
     return &g_hints.emplace(ws, h).first->second;
 }
 
-// The streaming path (three launches, no waits) is certain to work when top_k
-// bounds the kept set.  Measured on MI355X it then beats the cluster kernel
-// from 131072 tokens per call upwards (back to back: 15-17 us for small calls
-// against 16-31 us, 2-3 times faster for large ones); below that the single
-// launch wins by up to a microsecond.  RS_FORCE_PATH=cluster|stream|optimistic
-// overrides (tests).
+// Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
+// kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
+// times faster for large ones); below that the single launch wins by up to a microsecond.
+// RS_FORCE_PATH=cluster|stream|optimistic overrides (tests).
 enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2 };
 static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pen, bool want_e, const void *ws, hipStream_t st)
 {
@@ -1831,15 +1836,14 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (force && force[0] == 's') return bounded ? kPathStream : kPathCluster;
     if (force && force[0] == 'o') return bounded ? kPathStream : kPathAttempt;
     if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
-    if (bounded) return kPathStream;
-    if (!(top_p < 1.0f)) return kPathCluster;                  // everything is kept: nothing a stash could hold
+    if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // everything is kept: nothing a stash could hold
+    const int yes = bounded ? kPathStream : kPathAttempt, kind = bounded ? 0 : 1;
     Hint *h = hint_of(ws, false);
-    if (!h) return kPathCluster;
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone)
-        return kPathCluster;                                    // a captured choice could not follow the reports
-    const bool failing = *(volatile int32_t *)h->word != 0;
-    return (!failing || (++h->calls & 63u) == 0u) ? kPathAttempt : kPathCluster;
+    if (!h || hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone)
+        return bounded ? kPathStream : kPathCluster;            // a captured choice could not follow the reports
+    const bool failing = *(volatile int32_t *)(h->word + kind) != 0;
+    return (!failing || (++h->calls[kind] & 63u) == 0u) ? yes : kPathCluster;
 }
 
 template <bool PEN>
@@ -1940,8 +1944,8 @@ int rs_workspace_init(void *ws, size_t bytes, void *stream)
     if (hipMemsetAsync(ws, 0, bytes, (hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
     // the word of pinned host memory attempts are reported to (see choose_path)
     if (Hint *hint = hint_of(ws, true)) {
-        *hint->word = 0;
-        hint->calls = 0;
+        hint->word[0] = 0; hint->word[1] = 0;
+        hint->calls[0] = 0; hint->calls[1] = 0;
         WsHeader *h = (WsHeader *)ws;
         if (hipMemcpyAsync(&h->hint, &hint->word, sizeof hint->word, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess)
             return RS_ERR_LAUNCH;
@@ -1975,7 +1979,7 @@ int rs_workspace_policy(const void *ws, int32_t *state)
 {
     if (!ws || !state) return RS_ERR_NULL;
     const Hint *h = hint_of(ws, false);
-    *state = h ? (*(volatile int32_t *)h->word != 0 ? 1 : 0) : -1;
+    *state = h ? (((volatile int32_t *)h->word)[1] != 0 ? 1 : 0) | (((volatile int32_t *)h->word)[0] != 0 ? 2 : 0) : -1;
     return RS_OK;
 }
 
@@ -2015,7 +2019,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
-    p.need = nullptr; p.stash_k = (uint32_t)top_k;
+    p.need = nullptr; p.stash_k = (uint32_t)top_k; p.report = 0;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, e_bits != nullptr, workspace, (hipStream_t)stream);
     if (path != kPathCluster) {
@@ -2038,7 +2042,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         const uint32_t est = 2u * max(kk + 512u, whole <= (uint32_t)kFinCap ? whole : 0u);
         v.list_cap = 2048u;
         while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
-        v.attempt = path == kPathAttempt ? 1u : 0u;
+        p.report = path == kPathAttempt ? 1u : 0u;
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (sr == 4) {
             hipLaunchKernelGGL((stream_kernel<4, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
@@ -2053,7 +2057,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         // small grid whose workgroups take tickets until the list is exhausted.  After an attempt it
         // may be all of them: one workgroup per slice of every row, as in the cluster kernel; those
         // beyond the list leave at once.
-        if (path == kPathStream && grid.x > 1024u) grid.x = 1024u / g.G * g.G > 0 ? 1024u / g.G * g.G : g.G;
+        if (path == kPathStream && grid.x > kListGrid) grid.x = kListGrid / g.G * g.G > 0 ? kListGrid / g.G * g.G : g.G;
     }
     const hipError_t e = p.need ? launch_list(g.R, grid, (hipStream_t)stream, p, path == kPathAttempt)
                        : pen ? launch_sample<true>(g.R, grid, (hipStream_t)stream, p)

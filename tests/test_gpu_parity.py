@@ -441,7 +441,7 @@ def test_python_module_drop_in_calls(torch_cuda, oracle):
         assert np.array_equal(out.cpu().numpy(), ref_out)
 
 
-def test_nucleus_only_calls_are_routed_by_reports(torch_cuda, oracle):
+def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     """top_k disabled, top_p < 1: the wait-free path is an attempt.  On a workspace set up by
     rs_workspace_init it is made; peaked rows finish on it (diag.rounds == 0).  After a call whose rows
     mostly had to be handed on (flat rows) the report word says so and the next calls go straight to the
@@ -490,6 +490,31 @@ def test_nucleus_only_calls_are_routed_by_reports(torch_cuda, oracle):
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
     assert policy(smp) == 0
     assert smp.status() == 0
+
+    # The same for calls WITH a bounding top_k, which stream unless told otherwise: rows that are one
+    # tie of all their tokens cannot be finished from the stashes and are handed on, the report says
+    # so (bit 1), the next calls skip the streaming pass, and one in 64 streams again.
+    ties = np.zeros((B, V), dtype=np.float32)
+    rc, c, k, p = capi.normalize(1.0, 10, 1.0, V, B, 1)
+    ref_ties = oracle.sample_batch(ties, c, k, p, injected_u=u_np)
+    ref_peaked = oracle.sample_batch(peaked, c, k, p, injected_u=u_np)
+    lg_ties = torch.from_numpy(ties).cuda()
+    res = smp.sample(lg_peaked, c, k, p, uniforms=u)
+    _check(res, *ref_peaked, "bounded, peaked rows")
+    assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
+    res = smp.sample(lg_ties, c, k, p, uniforms=u)       # streamed, every row handed on
+    _check(res, *ref_ties, "bounded, rows of ties")
+    assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 2
+    res = smp.sample(lg_peaked, c, k, p, uniforms=u)     # not streamed
+    _check(res, *ref_peaked, "bounded, after rows of ties")
+    assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 2
+    for i in range(70):
+        res = smp.sample(lg_peaked, c, k, p, uniforms=u, want_diag=False)
+        assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
+    assert policy(smp) == 0
+    res = plain.sample(lg_ties, c, k, p, uniforms=u)     # no report words: streams whatever happened before
+    _check(res, *ref_ties, "bounded, zeroed workspace")
+    assert policy(plain) == -1 and plain.status() == 0 and smp.status() == 0
 
 
 def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
