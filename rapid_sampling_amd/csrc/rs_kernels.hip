@@ -174,6 +174,7 @@ struct Found {               // result of a histogram scan (uniform over the wor
     uint32_t pad;
 };
 
+constexpr int kRepC = 4;
 struct Lds {
     u128     q128[kWaves * 2];
     u128     bc128[4];
@@ -182,6 +183,9 @@ struct Lds {
     u128     D, P;
     Found    found;
     uint64_t hm[kNB];        // this workgroup's histogram
+    uint64_t hr[kNB * kRepC]; // level 1 while it is being counted: kRepC copies of each bin (lane l adds to copy
+                             // l % kRepC), since lanes that add to one LDS address are served one after the other
+                             // and rows often put most of their tokens into a few bins
     uint64_t g[kNB];         // the cluster's histogram
     uint64_t cand[kCap];
     uint64_t bc64[8];
@@ -622,7 +626,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
             }
         }
         kmax_row = block_max_u32(s, fkey(lmax), lane, wave);            // of this slice, for now
-        lds_hist_zero(s, kNB);
+        for (int b = tid; b < kNB * kRepC; b += kThreads) s.hr[b] = 0;
         if (tid == 0) { s.bc32[3] = 0; s.bc32[4] = 0; }
         // every workgroup posts its key (never 0 for a finite x) in its own slot
         if (G > 1 && tid == 0) a_store(&rc->mx[part], kmax_row);
@@ -643,9 +647,18 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const uint32_t b = eb[j * 4 + k];
-                lds_hist_add(s, ((b >> 21) + pos0) & 511u, b);
+                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hr[(((b >> 21) + pos0) & 511u) * kRepC + (lane & (kRepC - 1))]),
+                          (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
             }
         }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < kNB / kThreads; ++h) {
+        uint64_t w = 0;
+#pragma unroll
+        for (int c = 0; c < kRepC; ++c) w += s.hr[(tid + h * kThreads) * kRepC + c];
+        s.hm[tid + h * kThreads] = w;
     }
     uint32_t hx = 0;                                     // cluster histogram last summed
     uint32_t hx_nb = kNB;                                // and its size
