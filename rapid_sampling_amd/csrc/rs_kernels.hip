@@ -1124,6 +1124,7 @@ struct StreamView {
     PartHdr  *hdr;        // [B][G]
     uint64_t *stash;      // [B][G][kStashCap]   bits(e, slice frame) << 32 | index, by descending bin
     uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
+    uint64_t *shist;      // [B][G][kSB]   the slice's own bins (slice frame), as it added them to the row's
     uint32_t *need;       // [B]  rows left to the cluster kernel
     uint32_t  G;          // slices per row
     uint32_t  list_cap;   // entries of the finishing workgroup's token list (a power of two up to kFinCap)
@@ -1242,6 +1243,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     if (tid < kSB) {
         const uint64_t w = bin_total(tid);
         const float mm = M - 128.0f * __builtin_floorf(M * 0.0078125f);          // M mod 128, exact
+        v.shist[((size_t)row * G + part) * kSB + tid] = w;                        // kept for rows whose slices lie far apart
         if (w) a_add(&(p.ctl_end - 1 - row)->rowhist[((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u], w);
     }
 
@@ -1384,6 +1386,7 @@ struct LdsB {
     uint64_t blo[kMaxParts], bhi[kMaxParts];
     uint64_t small[64];
     uint32_t delta[kMaxParts];   // octaves between the row's frame and slice g's
+    uint32_t m4[kMaxParts];      // 4 (M mod 128) of slice g's frame: where its bins sit among the row's positions
     uint32_t take[kMaxParts];    // inclusive prefix of the entries taken from each stash
     uint64_t rand64;
     uint32_t nsmall, bucket, fail;
@@ -1468,6 +1471,8 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         const float d = M - __builtin_floorf(fkey_inv(ph.mkey));      // >= 0, a whole number or huge
         dl = d >= 64.0f ? 64u : (uint32_t)d;
         t.delta[tid] = dl;
+        const float Mg = __builtin_floorf(fkey_inv(ph.mkey));
+        t.m4[tid] = (uint32_t)(int)(Mg - 128.0f * __builtin_floorf(Mg * 0.0078125f)) * 4u;
     }
     // the row's level-1 histogram in the row's frame: bin r (octave M - 40 + r/4) sits at absolute
     // position 4 (M mod 128) + r - 160; the other 348 positions hold tokens below 2^-40 of this
@@ -1482,6 +1487,27 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         for (int b = tid; b < (int)kBin0; b += kThreads) s.g[b] = 0;
         low = block_sum_u32(s, low, lane, wave);
         if (tid == 0) s.g[kBin0] += (uint64_t)low << 43;
+        __syncthreads();
+        if (mixed) {
+            // Slices whose maxima lie 88 octaves or more apart may have put different octaves into
+            // one position.  Every token of a slice 41 octaves or more below the row's frame weighs
+            // 2^-40 there, whatever its bin: what such a slice added is taken out again, bin by bin
+            // (its own bins are on record), and its tokens are counted into the lowest bin.  The
+            // slices that remain lie within 40 octaves of each other.
+            for (uint32_t i = (uint32_t)tid; i < G * (uint32_t)kSB; i += kThreads) {
+                const uint32_t g = i / (uint32_t)kSB, r = i - g * (uint32_t)kSB;
+                if (t.delta[g] >= 41u) {
+                    const uint64_t w = v.shist[((size_t)row * G + g) * kSB + r];
+                    if (w) {
+                        const uint32_t rr = (t.m4[g] + r - m4) & 511u;
+                        if (rr < (uint32_t)kSB) {
+                            atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[kBin0 + rr]), 0ull - (unsigned long long)w);
+                            atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[kBin0]), (unsigned long long)pack_count(w) << 43);
+                        }
+                    }
+                }
+            }
+        }
     }
     __syncthreads();
     if (drawer) {
@@ -1497,7 +1523,7 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     // above that bin are taken, a prefix of each stash whose length is one cumulative count.
     uint32_t total = f.cnt_above + f.cnt_bin;
     uint32_t mtake = 0;
-    bool bad = mixed || total > v.list_cap;
+    bool bad = total > v.list_cap;
     if ((uint32_t)tid < G) {
         const int lb = (int)(f.bin - kBin0) + 4 * (int)dl;            // boundary bin in the slice's frame
         if (dl >= 64u) mtake = 0;                                      // the whole slice is clamped; the boundary bin
@@ -1528,7 +1554,7 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         cutrow = block_max_u32(s, mycut, lane, wave);
         take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
         total = t.take[kThreads - 1];
-        if (mixed || total > v.list_cap || total == 0u) {
+        if (total > v.list_cap || total == 0u) {
             // not resolvable from the stashes: leave the row to the cluster kernel
             if (tid == 0) {
                 const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
@@ -1780,13 +1806,14 @@ constexpr uint32_t kListGrid = 256;            // workgroups of the launch for t
 static int stream_r(int32_t B, int32_t V) { return (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144 ? 4 : 16; }
 static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-struct StreamLayout { size_t hdr, cum, stash, need, end; };
+struct StreamLayout { size_t hdr, cum, shist, stash, need, end; };
 static StreamLayout stream_layout(int32_t B, size_t parts, size_t base)
 {
     StreamLayout l;
     l.hdr = align256(base);
     l.cum = align256(l.hdr + parts * sizeof(PartHdr));
-    l.stash = align256(l.cum + parts * kSB * sizeof(uint32_t));
+    l.shist = align256(l.cum + parts * kSB * sizeof(uint32_t));
+    l.stash = align256(l.shist + parts * kSB * sizeof(uint64_t));
     l.need = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
     l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
     return l;
@@ -2042,6 +2069,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         const StreamLayout l = stream_layout(B, (size_t)B * v.G, sizeof(WsHeader));
         char *w = (char *)workspace;
         v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
+        v.shist = (uint64_t *)(w + l.shist);
         v.need = (uint32_t *)(w + l.need);
         // without a bounding top_k the stashes are sized as for top_k = kStreamK: enough for a nucleus
         // of up to about a thousand tokens

@@ -190,9 +190,11 @@ def test_streaming_path_mixed_rows(torch_cuda, oracle):
                                          uniforms=torch_cuda.from_numpy(H.uniforms(10, 91)).cuda())
         rounds = res["diag"]["rounds"]
         assert rounds[0] == 0 and rounds[1] == 0 and rounds[8] == 0 and rounds[9] == 0, rounds
-        # handed on: slices whose maxima are more than 87 octaves apart (rows 2, 3, 5, 6) and
-        # a tie of all 69632 tokens, too large to gather (row 4)
-        assert all(rounds[i] >= 1 for i in (2, 3, 4, 5, 6)), rounds
+        # slices whose maxima are more than 87 octaves apart (rows 2, 3, 5, 6): what the far ones put
+        # into the row's bins is taken out again, and the row is finished all the same
+        assert all(rounds[i] == 0 for i in (2, 3, 5, 6)), rounds
+        # handed on: a tie of all 69632 tokens, too large to gather
+        assert rounds[4] >= 1, rounds
     finally:
         os.environ.pop("RS_FORCE_PATH", None)
 
