@@ -1137,7 +1137,10 @@ struct StreamView {
 // below kBin0 by their own exponents, and those bins hand their counts to bin kBin0 afterwards
 // (such a token weighs 2^-40 exactly: a count and no fraction bits).  The histogram is done with
 // before the candidates are staged, and shares their memory.
-constexpr int kRep = 8;
+// Eight copies for long slices; two for the short slices of small calls, where clearing and
+// folding the copies would cost more than the few tokens of a thread.
+template <int R> constexpr int stream_copies() { return R >= 8 ? 8 : 2; }
+template <int kRep>
 struct LdsA {
     union {
         uint64_t hm[kNB * kRep];     // the slice's bins by bits >> 21
@@ -1156,7 +1159,8 @@ struct LdsA {
 template <int R, int NT>     // NT threads, each with R float4 of the slice
 __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Params p, const StreamView v)
 {
-    __shared__ LdsA s;
+    constexpr int kRep = stream_copies<R>();
+    __shared__ LdsA<kRep> s;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t G = v.G;
     const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
