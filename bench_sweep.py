@@ -11,10 +11,16 @@ multinomial), timed the same way.
     python bench_sweep.py                 # a cross-section of the grid, about a minute
     python bench_sweep.py --full          # the reference's whole grid (7200 points)
     python bench_sweep.py --out sweep.jsonl
+    python bench_sweep.py --json results.json --cpu-baseline
 
 One JSON line per point: shape, parameters, logit generator, microseconds per call for both
 (median of call + synchronize, and back-to-back device time between two events), speed-up.
 A summary line with the geometric-mean speed-up and the slowest points ends the run.
+--json writes one file in the layout of the reference's result file (bench.py:98-138:
+benchmark_config / results / summary, times in seconds, medians of call + synchronize), with
+`median_torch_gpu_time` in the place of `median_flashinfer_time`; --cpu-baseline adds
+`median_torch_cpu_time` (the same PyTorch formulation on the host's cores) for points of up to
+2^21 logits.
 """
 import argparse
 import json
@@ -79,6 +85,8 @@ def main():
     ap.add_argument("--out", default=None, help="write the JSON lines here as well")
     ap.add_argument("--reps", type=int, default=5, help="timed call+sync repetitions per point (reference: 5)")
     ap.add_argument("--b2b", type=int, default=20, help="back-to-back calls between two events")
+    ap.add_argument("--json", default=None, help="write a result file in the reference's layout (bench.py:121-138)")
+    ap.add_argument("--cpu-baseline", action="store_true", help="time the PyTorch formulation on the CPU too (small points)")
     args = ap.parse_args()
 
     import torch
@@ -122,6 +130,15 @@ def main():
                                "speedup_call_sync": round(t_sync / o_sync, 2),
                                "speedup_back_to_back": round(t_b2b / o_b2b, 2),
                                "GBps": round(B * V * 4 / o_b2b / 1e3, 1)}
+                        if args.cpu_baseline and B * V <= (1 << 21):
+                            lc = logits.cpu()
+                            ts = []
+                            for _ in range(3):
+                                t0 = time.perf_counter()
+                                torch_baseline(torch, lc, 1.0, top_k, top_p)
+                                ts.append((time.perf_counter() - t0) * 1e6)
+                            rec["torch_cpu_us"] = round(statistics.median(ts), 1)
+                            rec["torch_cpu_threads"] = torch.get_num_threads()
                         line = json.dumps(rec)
                         print(line, flush=True)
                         if out:
@@ -141,6 +158,26 @@ def main():
     if out:
         out.write(line + "\n")
         out.close()
+    if args.json:
+        results = []
+        for r in rows:
+            e = {"batch_size": r["B"], "vocab_size": r["V"], "top_p": r["top_p"], "top_k": r["top_k"],
+                 "logit_type": r["logits"],
+                 "median_torch_gpu_time": r["torch_us_call_sync"] * 1e-6,
+                 "median_my_kernel_time": r["us_call_sync"] * 1e-6,
+                 "speedup_ratio": r["torch_us_call_sync"] / r["us_call_sync"]}
+            if "torch_cpu_us" in r:
+                e["median_torch_cpu_time"] = r["torch_cpu_us"] * 1e-6
+            results.append(e)
+        with open(args.json, "w") as f:
+            json.dump({"benchmark_config": {"batch_sizes": Bs, "vocab_sizes": Vs, "top_ps": ps, "top_ks": ks,
+                                            "logit_types": kinds, "runs_per_setting": args.reps, "temperature": 1.0},
+                       "results": results,
+                       "summary": {"total_combinations": len(results),
+                                   "fastest_kernel_count": {
+                                       "torch_gpu": sum(1 for r in results if r["speedup_ratio"] < 1.0),
+                                       "your_kernel": sum(1 for r in results if r["speedup_ratio"] >= 1.0)}}},
+                      f, indent=2)
 
 
 if __name__ == "__main__":
