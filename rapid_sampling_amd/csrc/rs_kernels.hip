@@ -2078,7 +2078,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         // without a bounding top_k the stashes are sized as for top_k = kStreamK: enough for a nucleus
         // of up to about a thousand tokens
         const uint32_t kk = min((uint32_t)top_k, (uint32_t)kStreamK);
-        p.stash_k = kk < 128u ? kk : min(kk, max(128u, 8u * kk / v.G));
+        p.stash_k = min(kk, max(32u, 8u * kk / v.G));            // eight times a slice's share of the row's top_k
         hipStream_t st = (hipStream_t)stream;
         // The finishing workgroup's list: twice what a well-behaved row needs (its top_k tokens and
         // a boundary bin, or every stash whole), as a power of two; a row that needs more is handed
