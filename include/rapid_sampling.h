@@ -79,9 +79,10 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
  * Size of the workspace rs_sample needs for a batch of B rows of V tokens.
  * Replaces the reference's per-call `probs` scratch tensor of B*V floats
  * (sampling.cu:488,1014): a fixed record per row (about 38 KB) plus, for the
- * streaming path, about 0.7 bytes per token (stashes of the largest tokens
- * of each slice; up to 2.7 bytes per token for the first 4M tokens, where
- * slices are shorter); under a fifth of the reference's scratch for large V.
+ * streaming path, about 0.8 bytes per token (stashes of the largest tokens,
+ * counts and bins of each slice; up to 3.2 bytes per token for the first 4M
+ * tokens, where slices are shorter); a fifth of the reference's scratch for
+ * large V.
  * It does not grow with T.
  *
  * One workspace may serve calls of different shapes if it is at least
@@ -154,9 +155,10 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  *
  * Calls that share a workspace must be ordered on one stream.
  *
- * The call is one kernel launch, or three for large batches with
- * top_k <= 1024 (a wait-free pass over the logits, a per-row finish, and the
- * general kernel for rows the finish hands on); results are identical either
+ * The call is one kernel launch, or three for calls of at least 2^17 tokens
+ * without penalties whose kept set is expected to be small (a wait-free pass
+ * over the logits, a per-row finish, and the general kernel for rows the
+ * finish hands on; see rs_workspace_policy); results are identical either
  * way.  Two environment variables exist for tests: RS_FORCE_R (1..32, float4
  * per thread of the general kernel) and RS_FORCE_PATH (cluster | stream |
  * optimistic).
