@@ -28,7 +28,8 @@
 //     Any top_k / top_p, penalties, any batch.
 //
 //   streaming path (stream_kernel, finish_kernel, sample_list_kernel): for
-//     calls that move hundreds of MB with top_k <= 1024.  No workgroup waits
+//     calls of 2^17 tokens and more without penalties whose kept set is small
+//     next to the row (top_k <= 1024, or a small nucleus).  No workgroup waits
 //     for another: one pass over the logits leaves per-row histograms and
 //     per-slice stashes of the largest tokens, a small kernel finishes each
 //     row from them, and rows it cannot finish that way go through the
@@ -1091,22 +1092,24 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
 }
 
 // ---------------------------------------------------------- streaming path --
-// For large batches with a small top_k the cluster kernel's exchanges cost
-// more than the data movement.  The streaming path has no waits at all:
+// When the kept set is small next to the row the cluster kernel's exchanges
+// cost more than the data movement.  The streaming path has no waits at all:
 //
 //   stream_kernel   one workgroup per slice.  It reads the slice once, takes
 //                   its OWN maximum as the frame (the significand of e does
 //                   not depend on the frame, so a slice's histogram is the
-//                   row's up to a shift of whole octaves), writes its level-1
-//                   histogram and stashes its top_k largest tokens -- the
-//                   row's top_k tokens are among them -- ordered by bin.
-//   finish_kernel   one workgroup per row.  It shifts the slice histograms
-//                   into the row's frame and adds them, finds the boundary
-//                   bin, pulls the few stashed tokens at or above it, resolves
-//                   the threshold on them and picks.  A row whose stashes do
-//                   not reach down to the boundary bin (top_p cuts deeper
-//                   than any slice's top_k, or a huge tie) is put on a list,
-//                   and the cluster kernel then runs for the listed rows.
+//                   row's up to a shift of whole octaves), adds its level-1
+//                   histogram to the row's and stashes its largest tokens --
+//                   several times its share of the row's top_k -- ordered by
+//                   bin, with the exact value down to which the stash is
+//                   complete.
+//   finish_kernel   one workgroup per row.  It brings the row's histogram into
+//                   the row's frame, finds the boundary bin, pulls the stashed
+//                   tokens at or above it (or, for flat rows, the stashes
+//                   whole), resolves the threshold on them and picks.  A row
+//                   that cannot be finished from the stashes (a huge tie, a
+//                   nucleus of thousands of tokens) is put on a list, and the
+//                   cluster kernel then runs for the listed rows.
 constexpr int      kSB       = 164;           // level-1 bins in use: indices 348..511
 constexpr int      kStashCap = 1280;          // stash entries per slice (at least kStreamK)
 constexpr int      kStreamK  = 1024;          // largest top_k the streaming path takes
