@@ -271,6 +271,40 @@ def test_streaming_path_flat_distributions(torch_cuda, oracle):
         os.environ.pop("RS_FORCE_PATH", None)
 
 
+@pytest.mark.parametrize("B,V", [(6, 65536 + 4096), (20, 262144 + 4096)])
+def test_streaming_path_peaked_and_masked_rows(torch_cuda, oracle, B, V):
+    """Rows whose tokens mostly lie below 2^-40 of the maximum (wide or cold distributions, masked
+    vocabulary): the streaming kernel counts such tokens by their own exponents and folds them into
+    the lowest bin, refines a cut inside that bin with their number added analytically, and the
+    finishing kernel takes slices far below the row's frame out of the row's bins again.  Short slices
+    (first shape) and long slices (second).  Every row must equal the oracle's on every path, and all
+    but the row of ties must be finished by the streaming path itself."""
+    from tests import capi
+    rng = np.random.default_rng(123)
+    lg = np.empty((B, V), dtype=np.float32)
+    sig = [6.0, 15.0, 40.0, 100.0, 1000.0]
+    for b in range(B):
+        lg[b] = rng.standard_normal(V, dtype=np.float32) * np.float32(sig[b % len(sig)])
+    lg[1, : V // 2] = -np.inf                            # half the vocabulary masked, slices and all
+    lg[2, 1::2] = -1e9                                   # every other token masked: no slice is empty
+    lg[3, :] = -np.inf; lg[3, V - 7:] = rng.standard_normal(7)   # seven live tokens in the last, short slice
+    lg[4, 4096:8192] += 500.0                            # one short slice (a quarter of a long one) far above the rest
+    lg[5, :] = 1.0                                       # one tie
+    u = H.uniforms(B, 17)
+    for (k, p, t) in [(50, 0.9, 1.0), (1024, 1.0, 0.7), (3, 0.5, 0.05), (1000, 0.999, 4.0)]:
+        _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="peaked k=%s p=%s T=%s" % (k, p, t))
+    os.environ["RS_FORCE_PATH"] = "stream"
+    try:
+        rc, c, k, p = capi.normalize(1.0, 50, 0.9, V, B, 1)
+        res = capi.Sampler(B, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p,
+                                        uniforms=torch_cuda.from_numpy(u).cuda())
+        rounds = res["diag"]["rounds"]
+        assert all(rounds[i] == 0 for i in range(B) if i != 5), rounds
+        assert rounds[5] >= 1, rounds
+    finally:
+        os.environ.pop("RS_FORCE_PATH", None)
+
+
 def test_one_workspace_many_shapes(torch_cuda, oracle):
     """Calls of different (B, V, top_k) -- and so of different paths and layouts -- on one workspace sized
     for the largest B and the largest V: what one call leaves behind must not disturb the next."""
