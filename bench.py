@@ -249,6 +249,18 @@ def main():
                                    "achieved": round(bytes_flat / (t_flat * 1e-6) / 1e9, 1),
                                    "rows_per_s": round(Bb * Tb / (t_flat * 1e-6), 1)},
         }
+        # extension: the same rows handed over as bfloat16 (half the algorithmic bytes); (128, 1M), T = 1
+        half = big[:, Tb - 1, :].to(torch.bfloat16)
+        st_h = sample.setup_rand(1, Bb)
+
+        def call_half():
+            return sample.batch_sampling_temperature_topk_topp(half, st_h, 1.0, 1024, 0.95, accept_half=True)
+
+        t_half = block_time_us(torch, call_half, args.bandwidth_steps, 3)
+        result["roofline"]["bfloat16_logits_extension"] = {
+            "us_per_call": round(t_half, 2), "achieved": round(Bb * Vb * 2 / (t_half * 1e-6) / 1e9, 1),
+            "note": "(128,1048576) bfloat16 rows of the same values rounded, 2*V bytes per row, accept_half=True"}
+        del half
         if args.traffic_probe:
             src = big.view(-1)[: Bb * Vb]
             dst = torch.empty_like(src)

@@ -174,6 +174,28 @@ int rs_sample(const float *logits_device, int64_t row_stride,
               void *stream);
 
 /*
+ * The same call for logits stored as bfloat16 or IEEE half (RS_DTYPE_BF16,
+ * RS_DTYPE_F16; RS_DTYPE_F32 makes it rs_sample).  An extension: the reference
+ * rejects anything but float32 (sampling.cu:452-457, :976-981), and so do the
+ * drop-in Python functions unless the caller opts in.  Both formats widen to
+ * float32 exactly, so the result is that of rs_sample on the widened logits,
+ * bit for bit; rows of V elements, row_stride in elements, rows 8-byte aligned.
+ * Half the algorithmic bytes per row (2 V).
+ */
+#define RS_DTYPE_F32  0
+#define RS_DTYPE_BF16 1
+#define RS_DTYPE_F16  2
+int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row_stride,
+                    float *penalties_device, int32_t *out_device,
+                    void *rng_state_device, const float *injected_u_device,
+                    int32_t B, int32_t V,
+                    float presence_penalty, float repetition_penalty, float penalty_decay,
+                    float log2e_inv_temp, int32_t top_k, float top_p,
+                    void *workspace_device, size_t workspace_bytes,
+                    rs_row_diag *diag_device, uint32_t *e_bits_device,
+                    void *stream);
+
+/*
  * Launch-plus-one-read floor: a kernel with rs_sample's grid for (B,V) that
  * reads every logit once and max-combines one int per row into out_device
  * (which it does not clear).  Measurement aid for the B=1 latency bound; no

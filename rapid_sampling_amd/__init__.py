@@ -11,6 +11,10 @@ Drop-in for the Python API of the reference module (`sample` in
                   logits, penalties, states, presence_penalty, repetition_penalty,
                   penalty_decay, temperature, top_k, top_p)
 
+Beyond the reference: keyword names, `uniforms=` (injected draws, for tests) and
+`accept_half=True` (bfloat16 / float16 logits read as they are; by default any
+type but float32 raises the reference's error).
+
 The functions live in the compiled extension `_sample` (host layer in
 csrc/sampling.cpp, kernels in csrc/rs_kernels.hip behind the C ABI of
 include/rapid_sampling.h).  There is no Python or CPU fallback: without the

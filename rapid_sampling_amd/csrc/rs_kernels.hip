@@ -95,7 +95,7 @@ struct alignas(256) RowCtl {
 };
 
 struct Params {
-    const float *logits;
+    const void  *logits;       // fp32, or bf16 / fp16 (dtype): converted exactly on load
     float       *penalties;
     int32_t     *out;
     uint32_t    *rng;          // 16 words per row, or null
@@ -106,6 +106,7 @@ struct Params {
     RowCtl      *ctl_end;      // one past the record of row 0; row r is ctl_end[-1 - r]
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
+    int32_t      dtype;        // RS_DTYPE_* of the logits
     uint32_t     report;       // which of the two report words a streaming call writes: 0 top_k bounds the kept set, 1 not
     int64_t      row_stride;
     int32_t      B, V;
@@ -164,6 +165,32 @@ __device__ __forceinline__ uint32_t rebase_bits(uint32_t b, uint32_t delta)
 {
     const uint32_t d = delta << 23;
     return max(b, d + kEMinBits) - d;
+}
+
+// Logits arrive as fp32 or, if the caller opted in, as bf16 or fp16.  Both widen to fp32
+// exactly, so everything behind the load is the same arithmetic on the same values.
+__device__ __forceinline__ const char *logits_row(const Params &p, uint32_t row)
+{
+    return static_cast<const char *>(p.logits) + (int64_t)row * p.row_stride * (p.dtype == RS_DTYPE_F32 ? 4 : 2);
+}
+__device__ __forceinline__ void widen4(uint2 h, int dtype, uint32_t *bits)
+{
+    if (dtype == RS_DTYPE_BF16) {
+        bits[0] = h.x << 16; bits[1] = h.x & 0xFFFF0000u; bits[2] = h.y << 16; bits[3] = h.y & 0xFFFF0000u;
+    } else {
+        bits[0] = __float_as_uint((float)__builtin_bit_cast(_Float16, (uint16_t)(h.x & 0xFFFFu)));
+        bits[1] = __float_as_uint((float)__builtin_bit_cast(_Float16, (uint16_t)(h.x >> 16)));
+        bits[2] = __float_as_uint((float)__builtin_bit_cast(_Float16, (uint16_t)(h.y & 0xFFFFu)));
+        bits[3] = __float_as_uint((float)__builtin_bit_cast(_Float16, (uint16_t)(h.y >> 16)));
+    }
+}
+// group i4 (four tokens) of a row as floats, any dtype: for the rare re-reads
+__device__ __forceinline__ float4 load_logits4(const char *rowp, uint32_t i4, int dtype)
+{
+    if (dtype == RS_DTYPE_F32) return reinterpret_cast<const float4 *>(rowp)[i4];
+    uint32_t b[4];
+    widen4(reinterpret_cast<const uint2 *>(rowp)[i4], dtype, b);
+    return make_float4(__uint_as_float(b[0]), __uint_as_float(b[1]), __uint_as_float(b[2]), __uint_as_float(b[3]));
 }
 
 struct Found {               // result of a histogram scan (uniform over the workgroup)
@@ -565,7 +592,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
     // float4 slots of this thread: base4 + j*256, valid while < V4 (a prefix of j)
     const int nv = base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - base4 + kThreads - 1) / kThreads);
 
-    const float4 *lg = reinterpret_cast<const float4 *>(p.logits + (int64_t)row * p.row_stride);
+    const char *lrow = logits_row(p, row);
     float4 *pn4 = PEN ? reinterpret_cast<float4 *>(p.penalties + (int64_t)row * p.V) : nullptr;
 
     uint32_t eb[R * 4];                                 // l, then x, then bits(e)
@@ -574,13 +601,27 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
     // ---- 1. load once, scale, local max ---------------------------------
     uint32_t kmax_row;
     {
+        if (p.dtype == RS_DTYPE_F32) {
+            const float4 *lg = reinterpret_cast<const float4 *>(lrow);
 #pragma unroll
-        for (int j = 0; j < R; ++j) {
-            const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
-            const float4 l = lg[i4];
-            eb[j * 4 + 0] = __float_as_uint(l.x); eb[j * 4 + 1] = __float_as_uint(l.y);
-            eb[j * 4 + 2] = __float_as_uint(l.z); eb[j * 4 + 3] = __float_as_uint(l.w);
-            if (PEN) pen[j] = pn4[i4];
+            for (int j = 0; j < R; ++j) {
+                const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
+                const float4 l = lg[i4];
+                eb[j * 4 + 0] = __float_as_uint(l.x); eb[j * 4 + 1] = __float_as_uint(l.y);
+                eb[j * 4 + 2] = __float_as_uint(l.z); eb[j * 4 + 3] = __float_as_uint(l.w);
+                if (PEN) pen[j] = pn4[i4];
+            }
+        } else {
+            const uint2 *lh = reinterpret_cast<const uint2 *>(lrow);
+            uint2 h[R];
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
+                h[j] = lh[i4];
+                if (PEN) pen[j] = pn4[i4];
+            }
+#pragma unroll
+            for (int j = 0; j < R; ++j) widen4(h[j], p.dtype, &eb[j * 4]);
         }
         // Fast path: x = (l - pen) * c with no clean-up.  A NaN or Inf anywhere
         // in l, pen or the product shows as a NaN or Inf x, and only then do the
@@ -613,7 +654,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
 #pragma unroll
             for (int j = 0; j < R; ++j) {
                 const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
-                const float4 l = lg[i4];
+                const float4 l = load_logits4(lrow, i4, p.dtype);
                 float x0, x1, x2, x3;
                 if (PEN) {
                     x0 = sf((sf(l.x) - pen[j].x) * p.c); x1 = sf((sf(l.y) - pen[j].y) * p.c);
@@ -1159,7 +1200,7 @@ struct LdsA {
     uint32_t low;                // tokens of the slice below 2^-40
 };
 
-template <int R, int NT>     // NT threads, each with R float4 of the slice
+template <int R, int NT, int DT>     // NT threads, each with R groups of four tokens of the slice; DT the logits' type
 __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Params p, const StreamView v)
 {
     constexpr int kRep = stream_copies<R>();
@@ -1170,19 +1211,35 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const uint32_t base4 = part * (uint32_t)(NT * R) + (uint32_t)tid;
     const int nv = base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - base4 + NT - 1) / NT);
-    const float4 *lg = reinterpret_cast<const float4 *>(p.logits + (int64_t)row * p.row_stride);
+    const char *lrow = logits_row(p, row);
 
-    uint32_t eb[R * 4];                                 // x, then bits(e)
+    uint32_t eb[R * 4];                                 // l, then x, then bits(e)
     // x = l * c is the definition unless a NaN or Inf shows up (see sample_kernel).  Slots past the
     // end of the row read its last group again: harmless for the maximum and the probe, and they
     // are set aside before the histogram.
     constexpr int kSpecial = 0x207;
     float probe = 0.0f;
     float lmax = -3.402823466e+38f;
+    if constexpr (DT == RS_DTYPE_F32) {
+        const float4 *lg = reinterpret_cast<const float4 *>(lrow);
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
+            eb[j * 4 + 0] = __float_as_uint(l.x); eb[j * 4 + 1] = __float_as_uint(l.y);
+            eb[j * 4 + 2] = __float_as_uint(l.z); eb[j * 4 + 3] = __float_as_uint(l.w);
+        }
+    } else {
+        const uint2 *lh = reinterpret_cast<const uint2 *>(lrow);
+        uint2 h[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) h[j] = lh[min(base4 + (uint32_t)(j * NT), V4 - 1)];
+#pragma unroll
+        for (int j = 0; j < R; ++j) widen4(h[j], DT, &eb[j * 4]);
+    }
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-        const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
-        const float x0 = l.x * p.c, x1 = l.y * p.c, x2 = l.z * p.c, x3 = l.w * p.c;
+        const float x0 = __uint_as_float(eb[j * 4]) * p.c, x1 = __uint_as_float(eb[j * 4 + 1]) * p.c;
+        const float x2 = __uint_as_float(eb[j * 4 + 2]) * p.c, x3 = __uint_as_float(eb[j * 4 + 3]) * p.c;
         probe = __builtin_fmaf(x0, x1, probe);
         probe = __builtin_fmaf(x2, x3, probe);
         lmax = fmaxf(fmaxf(lmax, x0), fmaxf(x1, fmaxf(x2, x3)));
@@ -1193,8 +1250,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         lmax = -3.402823466e+38f;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            const float4 l = lg[min(base4 + (uint32_t)(j * NT), V4 - 1)];
-            const float x0 = sf(sf(l.x) * p.c), x1 = sf(sf(l.y) * p.c), x2 = sf(sf(l.z) * p.c), x3 = sf(sf(l.w) * p.c);
+            const float4 l = load_logits4(lrow, min(base4 + (uint32_t)(j * NT), V4 - 1), DT);
+            const float x0 = sf(l.x * p.c), x1 = sf(l.y * p.c), x2 = sf(l.z * p.c), x3 = sf(l.w * p.c);   // as at sampling.cu:553
             if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
             eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
@@ -2046,11 +2103,24 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
               void *workspace, size_t workspace_bytes,
               rs_row_diag *diag, uint32_t *e_bits, void *stream)
 {
+    return rs_sample_dtype(logits, RS_DTYPE_F32, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                           repetition, decay, log2e_inv_temp, top_k, top_p, workspace, workspace_bytes, diag, e_bits,
+                           stream);
+}
+
+int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                    void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                    float presence, float repetition, float decay,
+                    float log2e_inv_temp, int32_t top_k, float top_p,
+                    void *workspace, size_t workspace_bytes,
+                    rs_row_diag *diag, uint32_t *e_bits, void *stream)
+{
     if (!logits || !out || !workspace || (!rng_state && !injected_u)) return RS_ERR_NULL;
+    if (logits_dtype != RS_DTYPE_F32 && logits_dtype != RS_DTYPE_BF16 && logits_dtype != RS_DTYPE_F16) return RS_ERR_ARG;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
     if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
-    if (((uintptr_t)logits & 15) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
+    if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
         return RS_ERR_ALIGN;
     size_t need = 0;
     rs_workspace_bytes(B, V, &need);
@@ -2059,7 +2129,7 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
     const bool pen = penalties != nullptr;
     const Geometry g = choose_geometry(B, V, pen);
     Params p;
-    p.logits = logits; p.penalties = penalties; p.out = out;
+    p.logits = logits; p.dtype = logits_dtype; p.penalties = penalties; p.out = out;
     p.rng = (uint32_t *)rng_state; p.inj_u = injected_u; p.diag = diag; p.e_bits = e_bits;
     p.hdr = (WsHeader *)workspace;
     p.ctl_end = (RowCtl *)((char *)workspace + (workspace_bytes & ~(size_t)255));
@@ -2092,11 +2162,16 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
         while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
         p.report = path == kPathAttempt ? 1u : 0u;
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
+        const dim3 sgrid((uint32_t)B * v.G), sblock(kStreamNT);
         if (sr == 4) {
-            hipLaunchKernelGGL((stream_kernel<4, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
+            if (logits_dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_F32>), sgrid, sblock, 0, st, p, v);
+            else if (logits_dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);
+            else hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_F16>), sgrid, sblock, 0, st, p, v);
             hipLaunchKernelGGL((finish_kernel<12>), dim3((uint32_t)B), dim3(kThreads), dyn, st, p, v);
         } else {
-            hipLaunchKernelGGL((stream_kernel<16, kStreamNT>), dim3((uint32_t)B * v.G), dim3(kStreamNT), 0, st, p, v);
+            if (logits_dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<16, kStreamNT, RS_DTYPE_F32>), sgrid, sblock, 0, st, p, v);
+            else if (logits_dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<16, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);
+            else hipLaunchKernelGGL((stream_kernel<16, kStreamNT, RS_DTYPE_F16>), sgrid, sblock, 0, st, p, v);
             hipLaunchKernelGGL((finish_kernel<14>), dim3((uint32_t)B), dim3(kThreads), dyn, st, p, v);
         }
         if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;

@@ -84,17 +84,28 @@ void throw_for(int code, int64_t B, int64_t T, int64_t V, double temperature)
 
 struct Shape {
     int64_t B, T, V;
-    const float *first_row;   // logits[:, T-1, :] start
+    const void *first_row;    // logits[:, T-1, :] start
     int64_t row_stride;
+    int32_t dtype;            // RS_DTYPE_*
 };
 
 // Shapes as the reference reads them (sampling.cu:458-460, :982-984), plus the
 // checks it omits: device, unit stride of the vocabulary axis.
-Shape read_logits(const at::Tensor &logits, std::optional<int64_t> B_override)
+// The reference takes float32 logits only (sampling.cu:452-457, :976-981), and so does this unless
+// the caller passes accept_half=True: then bfloat16 and float16 logits are read as they are (they
+// widen to float32 exactly; half the bytes).
+int32_t logits_dtype(const at::Tensor &logits, bool accept_half)
 {
-    if (logits.dtype() != at::kFloat)
-        throw std::invalid_argument("Logits tensor must be of type float32 (FP32), got " +
-                                    std::string(logits.dtype().name()) + " !\n");
+    if (logits.dtype() == at::kFloat) return RS_DTYPE_F32;
+    if (accept_half && logits.dtype() == at::kBFloat16) return RS_DTYPE_BF16;
+    if (accept_half && logits.dtype() == at::kHalf) return RS_DTYPE_F16;
+    throw std::invalid_argument("Logits tensor must be of type float32 (FP32), got " +
+                                std::string(logits.dtype().name()) + " !\n");
+}
+
+Shape read_logits(const at::Tensor &logits, std::optional<int64_t> B_override, bool accept_half)
+{
+    const int32_t dtype = logits_dtype(logits, accept_half);
     if (logits.dim() < 1 || logits.dim() > 3)
         throw std::invalid_argument("Logits tensor must have shape (V,), (B, V) or (B, T, V) !\n");
     Shape s;
@@ -107,7 +118,8 @@ Shape read_logits(const at::Tensor &logits, std::optional<int64_t> B_override)
     if (s.B > rows) throw std::invalid_argument("penalties has more rows than logits !\n");
     s.row_stride = logits.dim() >= 2 ? logits.stride(0) : s.V;
     const int64_t t_stride = logits.dim() == 3 ? logits.stride(1) : 0;
-    s.first_row = logits.data_ptr<float>() + (s.T - 1) * t_stride;
+    s.first_row = static_cast<const char *>(logits.data_ptr()) + (s.T - 1) * t_stride * (int64_t)logits.element_size();
+    s.dtype = dtype;
     return s;
 }
 
@@ -168,10 +180,10 @@ at::Tensor run(const at::Tensor &logits, const Shape &s, at::Tensor *penalties, 
         diag = (rs_row_diag *)dbg->diag.data_ptr();
         ebits = (uint32_t *)dbg->e_bits.data_ptr();
     }
-    const int rc = rs_sample(s.first_row, s.row_stride, penalties ? penalties->data_ptr<float>() : nullptr,
-                             out.data_ptr<int32_t>(), inj ? nullptr : states->data_ptr(), inj,
-                             (int32_t)s.B, (int32_t)s.V, (float)presence, (float)repetition, (float)decay,
-                             c, k, p, ws.data_ptr(), (size_t)ws.numel(), diag, ebits, stream);
+    const int rc = rs_sample_dtype(s.first_row, s.dtype, s.row_stride, penalties ? penalties->data_ptr<float>() : nullptr,
+                                   out.data_ptr<int32_t>(), inj ? nullptr : states->data_ptr(), inj,
+                                   (int32_t)s.B, (int32_t)s.V, (float)presence, (float)repetition, (float)decay,
+                                   c, k, p, ws.data_ptr(), (size_t)ws.numel(), diag, ebits, stream);
     throw_for(rc, s.B, s.T, s.V, temperature);
     return out;
 }
@@ -190,9 +202,10 @@ at::Tensor setup_rand(int64_t seed, int64_t B)
 
 // sampling.cu:968-1044
 at::Tensor batch_sampling_temperature_topk_topp(at::Tensor &logits, at::Tensor &states, double temperature,
-                                                int64_t top_k, double top_p, std::optional<at::Tensor> uniforms)
+                                                int64_t top_k, double top_p, std::optional<at::Tensor> uniforms,
+                                                bool accept_half)
 {
-    const Shape s = read_logits(logits, std::nullopt);
+    const Shape s = read_logits(logits, std::nullopt, accept_half);
     return run(logits, s, nullptr, &states, 0, 0, 1, temperature, top_k, top_p, uniforms, nullptr);
 }
 
@@ -201,13 +214,11 @@ at::Tensor batch_sampling_repetition_temperature_topk_topp(at::Tensor &logits, a
                                                            at::Tensor &states, double presence_penalty,
                                                            double repetition_penalty, double penalty_decay,
                                                            double temperature, int64_t top_k, double top_p,
-                                                           std::optional<at::Tensor> uniforms)
+                                                           std::optional<at::Tensor> uniforms, bool accept_half)
 {
-    if (logits.dtype() != at::kFloat)
-        throw std::invalid_argument("Logits tensor must be of type float32 (FP32), got " +
-                                    std::string(logits.dtype().name()) + " !\n");
+    logits_dtype(logits, accept_half);                   // the reference's first check (sampling.cu:452)
     const int64_t B = penalties.dim() == 2 ? penalties.size(0) : 1;
-    const Shape s = read_logits(logits, B);
+    const Shape s = read_logits(logits, B, accept_half);
     return run(logits, s, &penalties, &states, presence_penalty, repetition_penalty, penalty_decay, temperature,
                top_k, top_p, uniforms, nullptr);
 }
@@ -217,11 +228,11 @@ at::Tensor batch_sampling_repetition_temperature_topk_topp(at::Tensor &logits, a
 std::tuple<at::Tensor, at::Tensor, at::Tensor> batch_sampling_debug(
     at::Tensor &logits, std::optional<at::Tensor> penalties, std::optional<at::Tensor> states,
     double presence_penalty, double repetition_penalty, double penalty_decay, double temperature, int64_t top_k,
-    double top_p, std::optional<at::Tensor> uniforms)
+    double top_p, std::optional<at::Tensor> uniforms, bool accept_half)
 {
     std::optional<int64_t> B;
     if (penalties) B = penalties->dim() == 2 ? penalties->size(0) : 1;
-    const Shape s = read_logits(logits, B);
+    const Shape s = read_logits(logits, B, accept_half);
     if (!uniforms && !states) throw std::invalid_argument("need states or uniforms !\n");
     Debug dbg;
     at::Tensor out = run(logits, s, penalties ? &*penalties : nullptr, states ? &*states : nullptr, presence_penalty,
@@ -232,11 +243,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> batch_sampling_debug(
 // Launch-plus-one-read floor kernel on the logits' grid (measurement aid).
 at::Tensor floor_read(at::Tensor &logits)
 {
-    const Shape s = read_logits(logits, std::nullopt);
+    const Shape s = read_logits(logits, std::nullopt, false);
     c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
     // not cleared: the kernel max-combines into it, and a second launch to zero it would be timed along
     auto out = at::empty({s.B}, at::TensorOptions().dtype(at::kInt).device(logits.device()));
-    const int rc = rs_floor_read(s.first_row, s.row_stride, out.data_ptr<int32_t>(), (int32_t)s.B, (int32_t)s.V,
+    const int rc = rs_floor_read(static_cast<const float *>(s.first_row), s.row_stride, out.data_ptr<int32_t>(), (int32_t)s.B, (int32_t)s.V,
                                  current_stream(logits));
     if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
     return out;
@@ -249,14 +260,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("batch_sampling_repetition_temperature_topk_topp", &batch_sampling_repetition_temperature_topk_topp,
           py::arg("logits"), py::arg("penalties"), py::arg("states"), py::arg("presence_penalty"),
           py::arg("repetition_penalty"), py::arg("penalty_decay"), py::arg("temperature"), py::arg("top_k"),
-          py::arg("top_p"), py::kw_only(), py::arg("uniforms") = py::none());
+          py::arg("top_p"), py::kw_only(), py::arg("uniforms") = py::none(), py::arg("accept_half") = false);
     m.def("batch_sampling_temperature_topk_topp", &batch_sampling_temperature_topk_topp, py::arg("logits"),
           py::arg("states"), py::arg("temperature"), py::arg("top_k"), py::arg("top_p"), py::kw_only(),
-          py::arg("uniforms") = py::none());
+          py::arg("uniforms") = py::none(), py::arg("accept_half") = false);
     m.def("batch_sampling_debug", &batch_sampling_debug, py::arg("logits"), py::arg("penalties"), py::arg("states"),
           py::arg("presence_penalty"), py::arg("repetition_penalty"), py::arg("penalty_decay"),
           py::arg("temperature"), py::arg("top_k"), py::arg("top_p"), py::kw_only(),
-          py::arg("uniforms") = py::none());
+          py::arg("uniforms") = py::none(), py::arg("accept_half") = false);
     m.def("floor_read", &floor_read, py::arg("logits"));
     m.attr("STATE_BYTES_PER_ROW") = RS_STATE_BYTES_PER_ROW;
     m.attr("DIAG_BYTES") = (int)sizeof(rs_row_diag);

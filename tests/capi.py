@@ -46,6 +46,9 @@ def lib():
         L.rs_sample.restype = C.c_int
         L.rs_sample.argtypes = [vp, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
                                 vp, sz, vp, vp, vp]
+        L.rs_sample_dtype.restype = C.c_int
+        L.rs_sample_dtype.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
+                                      vp, sz, vp, vp, vp]
         L.rs_floor_read.restype = C.c_int
         L.rs_floor_read.argtypes = [vp, i64, vp, i32, i32, vp]
         _lib = L
@@ -87,11 +90,13 @@ class Sampler:
 
     def sample(self, logits, c, top_k, top_p, *, rng=None, uniforms=None, penalties=None,
                presence=0.0, repetition=0.0, decay=1.0, want_diag=True, want_e=False):
-        """logits: (B,V) or (B,T,V) float32 cuda tensor.  Returns dict of cpu numpy results."""
+        """logits: (B,V) or (B,T,V) cuda tensor, float32 (rs_sample) or bfloat16 / float16
+        (rs_sample_dtype).  Returns dict of cpu numpy results."""
         torch = self.torch
+        dtype = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[logits.dtype]
         if logits.dim() == 3:
             B, T, V = logits.shape
-            ptr = logits.data_ptr() + 4 * (T - 1) * logits.stride(1)
+            ptr = logits.data_ptr() + logits.element_size() * (T - 1) * logits.stride(1)
             stride = logits.stride(0)
         else:
             B, V = logits.shape
@@ -101,13 +106,17 @@ class Sampler:
         out = torch.full((B,), -7, dtype=torch.int32, device="cuda")
         diag = torch.zeros((B, DIAG_DTYPE.itemsize), dtype=torch.uint8, device="cuda") if want_diag else None
         eb = torch.empty((B, V), dtype=torch.int32, device="cuda") if want_e else None
-        rc = lib().rs_sample(ptr, stride, penalties.data_ptr() if penalties is not None else None,
-                             out.data_ptr(), rng.data_ptr() if rng is not None else None,
-                             uniforms.data_ptr() if uniforms is not None else None,
-                             B, V, presence, repetition, decay, c, top_k, top_p,
-                             self.ws.data_ptr(), self.ws.numel(),
-                             diag.data_ptr() if diag is not None else None,
-                             eb.data_ptr() if eb is not None else None, self.stream())
+        tail = (penalties.data_ptr() if penalties is not None else None,
+                out.data_ptr(), rng.data_ptr() if rng is not None else None,
+                uniforms.data_ptr() if uniforms is not None else None,
+                B, V, presence, repetition, decay, c, top_k, top_p,
+                self.ws.data_ptr(), self.ws.numel(),
+                diag.data_ptr() if diag is not None else None,
+                eb.data_ptr() if eb is not None else None, self.stream())
+        if dtype == 0:
+            rc = lib().rs_sample(ptr, stride, *tail)
+        else:
+            rc = lib().rs_sample_dtype(ptr, dtype, stride, *tail)
         res = {"rc": rc}
         if rc != 0:
             return res

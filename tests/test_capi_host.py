@@ -167,6 +167,17 @@ def test_extension_raises_reference_errors_in_reference_order(sample):
         g(torch.zeros(2, 8), torch.zeros(2, 8), st, 0.1, 0.1, 0.9, 1e-4, -1, 0.5)
     with pytest.raises(ValueError, match=r"B must be positive"):
         sample.setup_rand(0, 0)
+    # half-precision logits are an opt-in: bfloat16 and float16 pass the first check with
+    # accept_half=True (and fail the next one here), other types never do
+    with pytest.raises(ValueError, match=r"type float32 \(FP32\), got"):
+        f(torch.zeros(2, 8, dtype=torch.bfloat16), st, 1.0, -1, 0.5)
+    with pytest.raises(ValueError, match=r"type float32 \(FP32\), got"):
+        f(torch.zeros(2, 8, dtype=torch.float64), st, 1.0, -1, 0.5, accept_half=True)
+    for dt in (torch.bfloat16, torch.float16):
+        with pytest.raises(ValueError, match="must live on the GPU"):
+            f(torch.zeros(2, 8, dtype=dt), st, 1.0, -1, 0.5, accept_half=True)
+        with pytest.raises(ValueError, match="must live on the GPU"):
+            g(torch.zeros(2, 8, dtype=dt), torch.zeros(2, 8), st, 0.1, 0.1, 0.9, 1.0, -1, 0.5, accept_half=True)
 
 
 def test_extension_accepts_keywords_like_the_readme(sample):

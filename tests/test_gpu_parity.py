@@ -33,7 +33,9 @@ def _check(res, ref_out, ref_diag, what):
 
 
 def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_np=None, u_np=None,
-              presence=0.0, repetition=0.0, decay=1.0, force_r=None, what=""):
+              presence=0.0, repetition=0.0, decay=1.0, force_r=None, what="", dtype=None):
+    """dtype: torch.bfloat16 / torch.float16 to hand the logits over in that format (logits_np must
+    then hold values that format represents exactly)."""
     if logits_np.ndim == 3:
         B, T, V = logits_np.shape
     else:
@@ -52,6 +54,9 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     try:
         smp = capi.Sampler(B, V)
         lg = torch.from_numpy(logits_np).cuda()
+        if dtype is not None:
+            lg = lg.to(dtype)
+            assert torch.equal(lg.float().cpu(), torch.from_numpy(logits_np)) or np.isnan(logits_np).any()
         pen = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
         u = torch.from_numpy(u_np).cuda()
         print("case", what, "B", B, "T", T, "V", V, "k", k, "p", p, "R", force_r, flush=True)
@@ -149,6 +154,10 @@ def test_degenerate_rows(torch_cuda, oracle):
     lg[5] = H.logits_normal(1, V, 1.0, seed=3)[0]; lg[5, :2000] = lg[5, 2000]
     for (k, p) in [(10, 0.5), (-1, 1.0), (1, 1.0), (-1, 1e-30), (V, 0.9)]:
         _run_case(torch_cuda, oracle, capi, lg, 1.0, k, p, u_np=H.uniforms(6, 17), what="degenerate k=%s p=%s" % (k, p))
+    # infinities times a factor below one (temperature above log2 e) stay infinities before the clean-up
+    # (sampling.cu:553); on the streaming path as well (forced: the call is smaller than it would take)
+    big = np.tile(lg, (1, 40))
+    _run_case(torch_cuda, oracle, capi, big, 4.0, 10, 0.9, u_np=H.uniforms(6, 18), what="degenerate T=4")
 
 
 def test_uniform_extremes(torch_cuda, oracle):
@@ -303,6 +312,36 @@ def test_streaming_path_peaked_and_masked_rows(torch_cuda, oracle, B, V):
         assert rounds[5] >= 1, rounds
     finally:
         os.environ.pop("RS_FORCE_PATH", None)
+
+
+@pytest.mark.parametrize("fmt", ["bfloat16", "float16"])
+def test_half_precision_logits(torch_cuda, oracle, fmt):
+    """Logits handed over as bfloat16 or float16 (rs_sample_dtype; an extension, the reference takes
+    float32 only): both widen to float32 exactly, so every result must equal the oracle's on the widened
+    values -- cluster path with the e bit patterns, streaming path with short and long slices, (B,T,V)
+    addressing, masked and infinite entries, the penalty kernel."""
+    torch = torch_cuda
+    from tests import capi
+    dtype = getattr(torch, fmt)
+    rng = np.random.default_rng(321)
+
+    def rounded(a):
+        return torch.from_numpy(a).to(dtype).float().numpy()
+
+    for (B, V, sigma) in [(5, 65536 + 4096, 3.0), (20, 262144 + 4096, 2.0)]:
+        lg = rounded((rng.standard_normal((B, V)) * sigma).astype(np.float32))
+        lg[1, : V // 3] = -np.inf
+        lg[2, 17] = np.inf
+        lg[3, 1::2] = rounded(np.full(1, -30000.0, dtype=np.float32))[0]
+        for (k, p, t) in [(50, 0.9, 1.0), (-1, 0.3, 0.7), (1024, 1.0, 2.0)]:
+            _run_case(torch, oracle, capi, lg, t, k, p, u_np=H.uniforms(B, 5), dtype=dtype,
+                      what="%s B=%d V=%d k=%s p=%s T=%s" % (fmt, B, V, k, p, t))
+    lg3 = rounded(rng.standard_normal((3, 4, 32768)).astype(np.float32) * 2)
+    _run_case(torch, oracle, capi, lg3, 0.8, 40, 0.95, u_np=H.uniforms(3, 6), dtype=dtype, what=fmt + " (B,T,V)")
+    lgp = rounded(rng.standard_normal((4, 131072)).astype(np.float32) * 1.5)
+    pen = (rng.random((4, 131072)) < 0.02).astype(np.float32) * rng.exponential(1.0, (4, 131072)).astype(np.float32)
+    _run_case(torch, oracle, capi, lgp, 0.8, 50, 0.9, pen_np=pen, u_np=H.uniforms(4, 7), presence=0.1, repetition=0.1,
+              decay=0.95, dtype=dtype, what=fmt + " penalties")
 
 
 def test_one_workspace_many_shapes(torch_cuda, oracle):
@@ -475,6 +514,16 @@ def test_python_module_drop_in_calls(torch_cuda, oracle):
         out = sample.batch_sampling_temperature_topk_topp(logits=lg, states=states, temperature=temp, top_k=k_in,
                                                           top_p=p_in, uniforms=torch.from_numpy(u_np).cuda())
         assert np.array_equal(out.cpu().numpy(), ref_out)
+    # half-precision logits, opted into: the result of the float32 call on the widened values
+    for dt in (torch.bfloat16, torch.float16):
+        lgh = torch.from_numpy(H.logits_normal(6, 4 * 65536, 2.0, seed=3).reshape(6, 4, 65536)).cuda().to(dt)
+        u = torch.from_numpy(H.uniforms(6, 9)).cuda()
+        st = sample.setup_rand(1, 6)
+        a = sample.batch_sampling_temperature_topk_topp(lgh, st, 0.9, 100, 0.95, uniforms=u, accept_half=True)
+        b = sample.batch_sampling_temperature_topk_topp(lgh.float(), st, 0.9, 100, 0.95, uniforms=u)
+        assert torch.equal(a, b)
+        with pytest.raises(ValueError, match="float32"):
+            sample.batch_sampling_temperature_topk_topp(lgh, st, 0.9, 100, 0.95, uniforms=u)
 
 
 def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
