@@ -344,6 +344,41 @@ def test_half_precision_logits(torch_cuda, oracle, fmt):
               decay=0.95, dtype=dtype, what=fmt + " penalties")
 
 
+def test_seeded_random_shapes_and_parameters(torch_cuda, oracle):
+    """A hundred seeded random cases -- batch, vocabulary (any multiple of 4, so most slices end ragged),
+    temperature, top_k, top_p and the kind of logits (the reference's five generators of bench.py:66-72,
+    plus rows with masked stretches and rows of few distinct values) -- each through every path."""
+    from tests import capi
+    rng = np.random.default_rng(20250101)
+    for case in range(100):
+        B = int(rng.integers(1, 24))
+        V = 4 * int(rng.integers(1, 50000)) if case % 3 else 4 * int(rng.integers(1, 2000))
+        if case % 10 == 9:
+            B, V = int(rng.integers(1, 8)), 4 * int(rng.integers(65537, 100000))      # long slices on the streaming path
+        kind = int(rng.integers(0, 7))
+        if kind == 0:
+            lg = np.zeros((B, V), dtype=np.float32)
+        elif kind == 1:
+            lg = rng.random((B, V), dtype=np.float32)
+        elif kind == 2:
+            lg = rng.standard_normal((B, V), dtype=np.float32) / np.float32(2)
+        elif kind == 3:
+            lg = rng.standard_normal((B, V), dtype=np.float32) * np.float32(3)
+        elif kind == 4:
+            lg = rng.random((B, V), dtype=np.float32) * np.float32(4)
+        elif kind == 5:
+            lg = rng.standard_normal((B, V), dtype=np.float32) * np.float32(2)
+            lo = int(rng.integers(0, V))
+            lg[:, lo: lo + int(rng.integers(1, V))] = -np.inf
+        else:
+            lg = np.round(rng.standard_normal((B, V), dtype=np.float32) * 3).astype(np.float32)
+        temp = float(rng.choice([0.05, 0.5, 0.8, 1.0, 1.3, 4.0, 100.0]))
+        top_k = int(rng.choice([-1, 1, 2, 10, 50, 100, 1000, 1024, 1025, 10000]))
+        top_p = float(rng.choice([0.0, 0.01, 0.1, 0.3, 0.5, 0.7, 0.9, 0.99, 1.0]))
+        _run_case(torch_cuda, oracle, capi, lg, temp, top_k, top_p, u_np=H.uniforms(B, 1000 + case),
+                  what="random case %d kind %d" % (case, kind))
+
+
 def test_one_workspace_many_shapes(torch_cuda, oracle):
     """Calls of different (B, V, top_k) -- and so of different paths and layouts -- on one workspace sized
     for the largest B and the largest V: what one call leaves behind must not disturb the next."""
