@@ -9,7 +9,7 @@ PyTorch formulation on the same GPU (softmax, descending sort, cumsum, top-k / t
 multinomial), timed the same way.
 
     python bench_sweep.py                 # a cross-section of the grid, about a minute
-    python bench_sweep.py --full          # the reference's whole grid (7200 points)
+    python bench_sweep.py --full          # the reference's whole grid (11500 points, ten minutes)
     python bench_sweep.py --out sweep.jsonl
     python bench_sweep.py --json results.json --cpu-baseline
 

@@ -466,6 +466,15 @@ __device__ __forceinline__ Found hist_find_level1(Lds &s, uint64_t top_k, float 
     return s.found;
 }
 
+// A boundary bin with nothing above it holds the row's largest token.  Every token of the bin
+// shares its exponent and none has a larger fraction, so a fraction sum of count times the largest
+// token's fraction proves that all of them equal it: one tie, whose value is then known without
+// looking at another digit.  `word` is the bin's packed count and fraction sum.
+__device__ __forceinline__ bool bin_is_one_tie(uint64_t word, uint32_t bin, uint32_t emax_bits)
+{
+    return (emax_bits >> 21) == bin && (word & kPackMask) == (uint64_t)pack_count(word) * (uint64_t)(emax_bits & 0x7FFFFFu);
+}
+
 // The same for a 128-bin level (all tokens share the exponent ex): one wave,
 // lane l owns indices 127-2l and 126-2l, no LDS exchange inside the scan.
 __device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint32_t cnt0, u128 mass0,
@@ -762,7 +771,15 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
     uint32_t lo = f.bin << 21;
     uint32_t span = (1u << 21) - 1u;
     uint32_t levels = 1;                                 // histogram levels summed over the cluster
-    while (f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
+    // more tokens in the boundary bin than can be gathered, all equal to the row's largest (rows of
+    // equal logits): the threshold is that value, no further level is needed
+    bool one_tie = false;
+    if (f.cnt_bin > (uint32_t)kCap && f.cnt_above == 0u) {
+        const uint32_t emax = e_bits_of(xmax, __builtin_floorf(xmax));
+        one_tie = bin_is_one_tie(s.g[f.bin], f.bin, emax);
+        if (one_tie) { lo = emax; span = 0u; }
+    }
+    while (!one_tie && f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
         ++levels;
         const uint32_t dsh = level_shift(levels);
         const uint32_t expect = f.cnt_bin;
@@ -1355,16 +1372,24 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         // 7 bits and take the sub-bins from the top down to the one at which the count reaches
         // stash_k, as far as they fit.
         const uint32_t ob = s.over + kBin0, above = s.n;
+        // a bin that is one tie of the slice's largest token (rows of equal logits) has all its
+        // tokens in one sub-bin: known without counting, which would queue them up at one address
+        const uint32_t emax = e_bits_raw(fkey_inv(k), M);
+        const uint64_t wbin = bin_total((int)s.over);
+        if (above == 0u && bin_is_one_tie(wbin, ob, emax)) {
+            if (tid == 0) s.sub[(emax >> 14) & 127u] = pack_count(wbin);
+        } else {
 #pragma unroll
-        for (int j = 0; j < R; ++j)
+            for (int j = 0; j < R; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t b = eb[j * 4 + q];
-                if ((b >> 21) == ob) atomicAdd(&s.sub[(b >> 14) & 127u], 1u);
-            }
-        // in the lowest bin, the tokens below 2^-40 (not counted above: their bits say another bin)
-        // all weigh 2^-40 exactly
-        if (ob == kBin0 && tid == 0 && s.low) atomicAdd(&s.sub[0], s.low);
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t b = eb[j * 4 + q];
+                    if ((b >> 21) == ob) atomicAdd(&s.sub[(b >> 14) & 127u], 1u);
+                }
+            // in the lowest bin, the tokens below 2^-40 (not counted above: their bits say another
+            // bin) all weigh 2^-40 exactly
+            if (ob == kBin0 && tid == 0 && s.low) atomicAdd(&s.sub[0], s.low);
+        }
         __syncthreads();
         if (wave == 0) {
             const uint32_t Ks = p.stash_k;
@@ -1582,6 +1607,29 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     const uint64_t top_k = (uint64_t)p.top_k;
     Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
+
+    // A row that is one tie of all its tokens (rows of equal logits) needs no stash at all: the
+    // threshold is the largest token's value, every token weighs the tie weight, and the token at
+    // which the running sum reaches r follows by division.
+    if (f.cnt_bin == (uint32_t)p.V && bin_is_one_tie(s.g[f.bin], f.bin, e_bits_of(xmax, M))) {
+        if (drawer) {
+            rng_st[2] = rs[2] + 1u;
+            if (rs[2] + 1u == 0u) rng_st[3] = rs[3] + 1u;
+        }
+        if (tid == 0) {
+            const uint32_t thr1 = e_bits_of(xmax, M);
+            const Target tg = tie_and_target(p, row, p.inj_u ? 0ull : t.rand64, xmax, D, P, thr1, 0u, f.cnt_bin, (u128)0, 0u, true);
+            // smallest i with (i + 1) * w_tie >= r; r <= V * w_tie
+            uint32_t lo_i = 0, hi_i = (uint32_t)p.V - 1u;
+            while (lo_i < hi_i) {
+                const uint32_t mid = (lo_i + hi_i) >> 1;
+                if ((u128)(mid + 1u) * tg.w_tie >= tg.r) hi_i = mid; else lo_i = mid + 1u;
+            }
+            p.out[row] = (int32_t)lo_i;
+            if (p.diag) p.diag[row].index = (int32_t)lo_i;
+        }
+        return;
+    }
 
     // Plan A: every stash reaches down to the row's boundary bin.  Then exactly the tokens at or
     // above that bin are taken, a prefix of each stash whose length is one cumulative count.
