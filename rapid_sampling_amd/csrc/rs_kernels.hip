@@ -658,18 +658,22 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         }
         const bool special = __builtin_amdgcn_classf(probe, kSpecial);
         if (special) {
-            // rare: fetch the logits again and apply the definition with its clean-ups
+            // Apply the definition with its clean-ups.  Without penalties that is sf of the product
+            // already in the registers (sampling.cu:553: masked vocabularies, logits at -inf, end
+            // here on every call, so nothing is fetched again); with penalties the logit itself is
+            // cleaned first (sampling.cu:220) and has to be read once more.
             lmax = -3.402823466e+38f;
 #pragma unroll
             for (int j = 0; j < R; ++j) {
-                const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
-                const float4 l = load_logits4(lrow, i4, p.dtype);
                 float x0, x1, x2, x3;
                 if (PEN) {
+                    const uint32_t i4 = min(base4 + (uint32_t)(j * kThreads), V4 - 1);
+                    const float4 l = load_logits4(lrow, i4, p.dtype);
                     x0 = sf((sf(l.x) - pen[j].x) * p.c); x1 = sf((sf(l.y) - pen[j].y) * p.c);
                     x2 = sf((sf(l.z) - pen[j].z) * p.c); x3 = sf((sf(l.w) - pen[j].w) * p.c);
                 } else {
-                    x0 = sf(l.x * p.c); x1 = sf(l.y * p.c); x2 = sf(l.z * p.c); x3 = sf(l.w * p.c);
+                    x0 = sf(__uint_as_float(eb[j * 4])); x1 = sf(__uint_as_float(eb[j * 4 + 1]));
+                    x2 = sf(__uint_as_float(eb[j * 4 + 2])); x3 = sf(__uint_as_float(eb[j * 4 + 3]));
                 }
                 if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
                 eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
@@ -1264,11 +1268,13 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
     }
     if (__builtin_amdgcn_classf(probe, kSpecial)) {
+        // the clean-up of sampling.cu:553 on the products already in the registers (masked
+        // vocabularies, logits at -inf, come through here on every call)
         lmax = -3.402823466e+38f;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            const float4 l = load_logits4(lrow, min(base4 + (uint32_t)(j * NT), V4 - 1), DT);
-            const float x0 = sf(l.x * p.c), x1 = sf(l.y * p.c), x2 = sf(l.z * p.c), x3 = sf(l.w * p.c);   // as at sampling.cu:553
+            const float x0 = sf(__uint_as_float(eb[j * 4])), x1 = sf(__uint_as_float(eb[j * 4 + 1]));
+            const float x2 = sf(__uint_as_float(eb[j * 4 + 2])), x3 = sf(__uint_as_float(eb[j * 4 + 3]));
             if (j < nv) lmax = fmaxf(lmax, fmaxf(fmaxf(x0, x1), fmaxf(x2, x3)));
             eb[j * 4 + 0] = __float_as_uint(x0); eb[j * 4 + 1] = __float_as_uint(x1);
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
