@@ -1683,36 +1683,43 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         subset = true;
     }
 
-    // gather the tokens, re-based to the row's frame
+    // gather the tokens, re-based to the row's frame: a thread takes a run of consecutive list
+    // entries, so that it looks up its first slice once and walks on from there
     {
-        constexpr int kBatch = 4;
-        for (uint32_t i0 = tid; i0 < total; i0 += kBatch * kThreads) {
+        constexpr int kBatch = 8;
+        const uint32_t per = (total + kThreads - 1u) / kThreads;
+        uint32_t i = (uint32_t)tid * per;
+        const uint32_t iend = min(total, i + per);
+        uint32_t g = 0, gbase = 0, gend = 0;
+        if (i < iend) {
+            uint32_t lo_g = 0, hi_g = G - 1;                           // first slice whose prefix exceeds i
+            while (lo_g < hi_g) {
+                const uint32_t mid = (lo_g + hi_g) >> 1;
+                if (t.take[mid] > i) hi_g = mid; else lo_g = mid + 1;
+            }
+            g = lo_g; gbase = g ? t.take[g - 1] : 0u; gend = t.take[g];
+        }
+        while (i < iend) {
             uint64_t e[kBatch];
             uint32_t sl[kBatch];
+            const uint32_t n = min((uint32_t)kBatch, iend - i);
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                const uint32_t i = i0 + (uint32_t)u * kThreads;
                 e[u] = 0; sl[u] = 0;
-                if (i < total) {
-                    uint32_t lo_g = 0, hi_g = G - 1;                   // first slice whose prefix exceeds i
-                    while (lo_g < hi_g) {
-                        const uint32_t mid = (lo_g + hi_g) >> 1;
-                        if (t.take[mid] > i) hi_g = mid; else lo_g = mid + 1;
-                    }
-                    const uint32_t j = i - (lo_g ? t.take[lo_g - 1] : 0u);
-                    e[u] = v.stash[((size_t)row * G + lo_g) * kStashCap + j];
-                    sl[u] = lo_g;
+                if ((uint32_t)u < n) {
+                    while (i + (uint32_t)u >= gend) { ++g; gbase = gend; gend = t.take[g]; }    // slices that give nothing are skipped
+                    e[u] = v.stash[((size_t)row * G + g) * kStashCap + (i + (uint32_t)u - gbase)];
+                    sl[u] = g;
                 }
             }
 #pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const uint32_t i = i0 + (uint32_t)u * kThreads;
-                if (i < total) {
+            for (int u = 0; u < kBatch; ++u)
+                if ((uint32_t)u < n) {
                     uint32_t b = rebase_bits((uint32_t)(e[u] >> 32), t.delta[sl[u]]);
                     if (b < cutrow) b = 0;                             // plan B: below the complete part; 0 matches nothing
-                    t.list[i] = ((uint64_t)b << 32) | (uint32_t)e[u];
+                    t.list[i + (uint32_t)u] = ((uint64_t)b << 32) | (uint32_t)e[u];
                 }
-            }
+            i += n;
         }
     }
     __syncthreads();
