@@ -1280,7 +1280,12 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    for (int i = tid; i < kNB * kRep; i += NT) s.hm[i] = 0;
+    {
+        uint4 *z = reinterpret_cast<uint4 *>(s.hm);                              // two bins per store
+#pragma unroll
+        for (int i = 0; i < kNB * kRep / 2 / NT; ++i) z[tid + i * NT] = make_uint4(0u, 0u, 0u, 0u);
+        static_assert(kNB * kRep % (2 * NT) == 0, "whole stores");
+    }
     if (tid == 0) s.low = 0;
     if (blockIdx.x == 0 && tid == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
     uint32_t k = wave_max_u32(fkey(lmax));
@@ -1310,7 +1315,11 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     {
         // the tokens below 2^-40: counted into bin kBin0
         uint32_t low = 0;
-        for (int i = tid; i < (int)kBin0 * kRep; i += NT) low += pack_count(s.hm[i]);
+        const uint4 *two = reinterpret_cast<const uint4 *>(s.hm);                // two bins per load; counts sit in y and w
+        for (int i = tid; i < (int)kBin0 * kRep / 2; i += NT) {
+            const uint4 q = two[i];
+            low += (q.y >> 11) + (q.w >> 11);
+        }
         low = wave_sum(low);
         if (lane == 0 && low) {
             atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[kBin0 * kRep]), (unsigned long long)low << 43);
