@@ -1331,9 +1331,13 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     // bin t of this frame is octave M - 40 + t/4.  Slices of one row may use different frames; as
     // long as their maxima lie within 87 octaves of each other no two octaves in use coincide.
     auto bin_total = [&](int b) {
+        const uint4 *two = reinterpret_cast<const uint4 *>(&s.hm[((int)kBin0 + b) * kRep]);     // two copies per load
         uint64_t w = 0;
 #pragma unroll
-        for (int c = 0; c < kRep; ++c) w += s.hm[((int)kBin0 + b) * kRep + c];
+        for (int c = 0; c < kRep / 2; ++c) {
+            const uint4 q = two[c];
+            w += (((uint64_t)q.y << 32) | q.x) + (((uint64_t)q.w << 32) | q.z);
+        }
         return w;
     };
     if (tid < kSB) {
