@@ -237,7 +237,7 @@ def main():
             "frac": round(ach / HBM_PEAK_GBS, 4),
             # HBM bytes per call from the FETCH_SIZE / WRITE_SIZE counter runs of this same command
             # (profiles/bench_kernels_hbm_traffic_pmc.md), not measured live
-            "traffic": 574422016,
+            "traffic": 574428160,
             "workload": "(B,T,V)=(128,4,1048576) N(0,1.5), top_k 1024, top_p 0.95: 128 sampled rows of 4 MiB, "
                         "stride T*V, algorithmic bytes 4*V per row = 512 MiB per call",
             "us_per_call": round(t_btv, 2), "rows_per_s": round(Bb / (t_btv * 1e-6), 1),
