@@ -1712,6 +1712,15 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
             }
             g = lo_g; gbase = g ? t.take[g - 1] : 0u; gend = t.take[g];
         }
+        if (per == 1u) {                                               // a short list: one entry, no walking
+            if (i < iend) {
+                const uint64_t e = v.stash[((size_t)row * G + g) * kStashCap + (i - gbase)];
+                uint32_t b = rebase_bits((uint32_t)(e >> 32), t.delta[g]);
+                if (b < cutrow) b = 0;
+                t.list[i] = ((uint64_t)b << 32) | (uint32_t)e;
+            }
+            i = iend;
+        }
         while (i < iend) {
             uint64_t e[kBatch];
             uint32_t sl[kBatch];
