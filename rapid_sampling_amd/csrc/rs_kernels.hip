@@ -1808,8 +1808,12 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     constexpr uint32_t sh_slice = SLICE_LOG2;
     constexpr uint32_t sh_run = sh_slice - 8;                                  // 256 runs of at most 64 tokens
     static_assert(SLICE_LOG2 >= 8 && SLICE_LOG2 <= 14, "runs must fit the final all-pairs step");
-    const uint32_t ga = bucket_step(s, t, total, sh_slice, 0u, 0xFFFFFFFFu, r, weight, lane, wave);
     constexpr uint32_t kPairs = 64;
+    const uint64_t *cands = t.small;                                           // what the all-pairs step works on
+    uint32_t nkept = total;
+    if (total <= kPairs) cands = t.list;                                       // the whole list is few enough as it is
+    else {
+    const uint32_t ga = bucket_step(s, t, total, sh_slice, 0u, 0xFFFFFFFFu, r, weight, lane, wave);
     uint32_t lo_b = ga << sh_slice, len_b = 1u << sh_slice;
     // the kept tokens of that slice: few enough for the all-pairs step as they are, as a rule;
     // otherwise the slice is narrowed to one of its 256 runs first
@@ -1827,12 +1831,13 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         __syncthreads();
         return t.nsmall;
     };
-    uint32_t nkept = collect();
+    nkept = collect();
     if (nkept > kPairs) {
         __syncthreads();                                                       // everyone has read the count
         const uint32_t gb = bucket_step(s, t, total, sh_run, lo_b, lo_b + len_b, r, weight, lane, wave);
         lo_b += gb << sh_run; len_b = 1u << sh_run;
         nkept = collect();
+    }
     }
     // all pairs: every kept token of the range adds up the weights at or before it in index order;
     // the four waves take a quarter of the addends each
@@ -1842,7 +1847,7 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     u128 *partial = reinterpret_cast<u128 *>(s.cand) + kPairs;
     uint64_t me = 0, wme = 0;
     if ((uint32_t)tid < ns) {
-        me = t.small[tid];
+        me = cands[tid];
         wme = weight((uint32_t)(me >> 32));
         rec[tid] = make_uint4((uint32_t)wme, (uint32_t)(wme >> 32), (uint32_t)me, 0u);
     }
