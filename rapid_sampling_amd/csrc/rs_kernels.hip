@@ -1681,7 +1681,13 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         // take the stashes whole.  Together they hold every token of the row at or above
         // cutrow = the largest of the slices' cuts, so a threshold found among those is the row's.
         uint32_t mycut = 0;
-        if ((uint32_t)tid < G) mycut = rebase_bits(ph.cut, dl);
+        if ((uint32_t)tid < G) {
+            mycut = rebase_bits(ph.cut, dl);
+            // A cut above 2^-40 that lands on 2^-40 in the row's frame: the slice's tokens below
+            // its cut land there too and are not in its stash, so the stash is complete only
+            // above that value.  (A cut at 2^-40 in the slice's own frame took the whole slice.)
+            if (ph.cut != kEMinBits && mycut == kEMinBits) mycut = kEMinBits + 1u;
+        }
         cutrow = block_max_u32(s, mycut, lane, wave);
         take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
         total = t.take[kThreads - 1];

@@ -313,6 +313,25 @@ def test_streaming_path_peaked_and_masked_rows(torch_cuda, oracle, B, V):
         os.environ.pop("RS_FORCE_PATH", None)
 
 
+def test_streaming_path_whole_slice_stash_beside_partial_ones(torch_cuda, oracle):
+    """A wide row whose largest token sits in the short last slice: that slice's stash takes all of
+    the slice, tokens at 2^-40 included, while the other slices' stashes stop above 2^-40 of their
+    own, lower frames.  In the row's frame those slices' tokens all weigh 2^-40 and are not in any
+    stash, so the stashes are complete only above 2^-40 and a threshold at 2^-40 (top_k larger than the
+    handful of tokens above it) must not be decided from them."""
+    from tests import capi
+    rng = np.random.default_rng(2024)
+    B, V = 6, 13 * 4096 + 648
+    lg = (rng.standard_normal((B, V)) * 60.0).astype(np.float32)
+    for b in range(3):
+        lg[b, V - 5 - b] = lg[b].max() + np.float32(3.0 * b)        # the row's maximum in the last slice
+    lg[3, 7] = lg[3].max() + np.float32(1.0)                        # and in the first, for comparison
+    lg[4] = (rng.standard_normal(V) * 3.0).astype(np.float32); lg[4, V - 1] = lg[4].max() + np.float32(0.5)
+    u = H.uniforms(B, 23)
+    for (k, p, t) in [(100, 1.0, 0.8), (10, 0.9, 1.0), (1024, 1.0, 0.8), (1000, 0.999, 0.05)]:
+        _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="last-slice maximum k=%s p=%s T=%s" % (k, p, t))
+
+
 @pytest.mark.parametrize("fmt", ["bfloat16", "float16"])
 def test_half_precision_logits(torch_cuda, oracle, fmt):
     """Logits handed over as bfloat16 or float16 (rs_sample_dtype; an extension, the reference takes
