@@ -715,9 +715,20 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         for (int c = 0; c < kRepC; ++c) w += s.hr[(tid + h * kThreads) * kRepC + c];
         s.hm[tid + h * kThreads] = w;
     }
-    uint32_t hx = 0;                                     // cluster histogram last summed
-    uint32_t hx_nb = kNB;                                // and its size
+    // Cluster histograms this row has used and not yet cleared (bit i: rc->h[i]).  A workgroup may
+    // clear its share of one only when every workgroup of the cluster has finished reading it,
+    // and only an exchange in which every workgroup publishes something proves that: a deeper
+    // histogram level does not, since a slice without tokens in the boundary bin adds nothing to it
+    // and the others get past that level without it.
+    uint32_t h_used = G > 1 ? 1u : 0u;
     bool mx_posted = G > 1;                              // my slot is still to be cleared
+    auto clear_used = [&]() {
+        for (uint32_t i = 0; i <= (uint32_t)kLevels; ++i)
+            if (h_used >> i & 1u) zero_slice(rc->h[i], (i == 0u || i == (uint32_t)kLevels) ? (uint32_t)kNB : 128u, part, G);
+        h_used = 0u;
+        if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
+        mx_posted = false;
+    };
     if (G == 1) {
         if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return false;
     } else {
@@ -748,11 +759,10 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                     }
                 }
             if (!hist_combine(s, p.hdr, G, rc->h[kLevels], kNB, (uint32_t)p.V, lane, wave)) return false;
-            // every workgroup has read the first histogram and the slots: it published this one after that
-            zero_slice(rc->h[0], kNB, part, G);
-            if (tid == 0) a_store(&rc->mx[part], 0u);
-            mx_posted = false;
-            hx = kLevels;
+            // every workgroup has read the first histogram and the slots: it published this one
+            // (every slice holds tokens) after that
+            clear_used();
+            h_used = 1u << kLevels;
         }
     }
     if (p.e_bits) {
@@ -800,13 +810,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 }
             }
         if (!hist_combine(s, p.hdr, G, rc->h[levels - 1], 128, expect, lane, wave)) return false;
-        // every workgroup has finished reading the level above: it published this level after that
-        if (G > 1) {
-            zero_slice(rc->h[hx], hx_nb, part, G);
-            if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
-            mx_posted = false;
-        }
-        hx = levels - 1; hx_nb = 128;
+        if (G > 1) h_used |= 1u << (levels - 1);
         f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
         amass += local_mass_above(s, f.bin, exb, lane, wave);
         mycnt = pack_count(s.hm[f.bin]);
@@ -866,9 +870,8 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 if (s.abort) return false;
             }
             if ((uint32_t)tid < G) a_mine = get_mass(w0, w1);
-            // every workgroup wrote its entries after it had read the last histogram level
-            zero_slice(rc->h[hx], hx_nb, part, G);
-            if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
+            // every workgroup wrote its mass after it had read the last histogram level
+            clear_used();
         } else a_mine = tid == 0 ? amass : (u128)0;
         __syncthreads();
 
@@ -957,8 +960,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 if (total == G) break;
                 if (s.abort) return false;
             }
-            zero_slice(rc->h[hx], hx_nb, part, G);
-            if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
+            clear_used();
             before = block_sum_u128(s, (uint32_t)tid < part ? get_mass(w0, w1) : (u128)0, lane, wave);
         }
     }

@@ -332,6 +332,31 @@ def test_streaming_path_whole_slice_stash_beside_partial_ones(torch_cuda, oracle
         _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="last-slice maximum k=%s p=%s T=%s" % (k, p, t))
 
 
+def test_cluster_levels_with_slices_that_hold_no_boundary_tokens(torch_cuda, oracle):
+    """Many rows whose threshold is a tie of thousands of tokens lying in one contiguous range (a
+    masked range with everything kept: the tie at 2^-40; a range of equal largest logits): the
+    cluster kernel goes through every histogram level, and the slices outside the range add nothing
+    to the deeper levels, so their workgroups are not needed for those levels to complete.  A
+    histogram may therefore be cleared only after an exchange every workgroup takes part in; clearing
+    it after the next level left a slower workgroup polling zeros until its wait gave up.  More
+    workgroups than the GPU holds at once, several calls: every result equals the oracle's and no
+    wait gives up."""
+    from tests import capi
+    rng = np.random.default_rng(77)
+    B, V = 100, 78712
+    lg = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    for b in range(B):
+        lo = int(rng.integers(0, V - 1)); n = int(rng.integers(1100, V // 3))
+        if b % 2 == 0:
+            lg[b, lo: lo + n] = -np.inf
+        else:
+            lg[b, lo: lo + n] = lg[b].max() + np.float32(0.25)
+    u = H.uniforms(B, 31)
+    for (k, p, t) in [(-1, 1.0, 0.8), (-1, 0.999, 1.0), (5000, 1.0, 1.3)]:
+        for rep in range(2):
+            _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="contiguous ties k=%s p=%s T=%s #%d" % (k, p, t, rep))
+
+
 @pytest.mark.parametrize("fmt", ["bfloat16", "float16"])
 def test_half_precision_logits(torch_cuda, oracle, fmt):
     """Logits handed over as bfloat16 or float16 (rs_sample_dtype; an extension, the reference takes
