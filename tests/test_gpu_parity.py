@@ -422,6 +422,99 @@ def test_seeded_random_shapes_and_parameters(torch_cuda, oracle):
                   what="random case %d kind %d" % (case, kind))
 
 
+def _random_row(rng, kind, V):
+    """One row of logits of the given kind (see test_seeded_random_batches_of_mixed_rows)."""
+    if kind == 0:
+        return np.full(V, float(rng.choice([0.0, 1.5, -3.0, 1e30, -1e30])), dtype=np.float32)
+    if kind == 1:
+        return rng.random(V, dtype=np.float32)
+    if kind == 2:
+        return rng.standard_normal(V, dtype=np.float32) * np.float32(rng.choice([0.5, 3.0]))
+    if kind == 3:
+        return rng.random(V, dtype=np.float32) * np.float32(4)
+    if kind == 4:                                                       # a masked stretch
+        r = rng.standard_normal(V, dtype=np.float32) * np.float32(2)
+        lo = int(rng.integers(0, V))
+        r[lo: lo + int(rng.integers(1, V))] = -np.inf
+        return r
+    if kind == 5:                                                       # few distinct values
+        return np.round(rng.standard_normal(V, dtype=np.float32) * 3).astype(np.float32)
+    if kind == 6:                                                       # most tokens below 2^-40 of the largest
+        r = rng.standard_normal(V, dtype=np.float32) * np.float32(rng.choice([6.0, 15.0, 60.0, 300.0]))
+        if rng.random() < 0.5:                                          # the largest near the end of the row
+            r[int(rng.integers(max(0, V - 600), V))] = r.max() + np.float32(rng.choice([0.0, 1.0, 50.0]))
+        return r
+    if kind == 7:                                                       # scattered masks
+        r = rng.standard_normal(V, dtype=np.float32)
+        r[rng.random(V) < float(rng.choice([0.5, 0.9, 0.99, 0.9999]))] = -np.inf
+        r[int(rng.integers(0, V))] = 0.5
+        return r
+    if kind == 8:                                                       # a stretch of equal largest logits, NaN, Inf
+        r = rng.standard_normal(V, dtype=np.float32)
+        lo = int(rng.integers(0, V))
+        r[lo: lo + int(rng.integers(1, max(2, V // 2)))] = float(r.max()) + float(rng.choice([0.0, 0.25, 2.0]))
+        if rng.random() < 0.1:
+            r[int(rng.integers(0, V))] = np.nan
+        if rng.random() < 0.1:
+            r[int(rng.integers(0, V))] = np.inf
+        return r
+    if kind == 9:                                                       # stretches at very different levels
+        r = rng.standard_normal(V, dtype=np.float32)
+        step = int(rng.choice([1024, 4096, 16384]))
+        for lo in range(0, V, step):
+            r[lo: lo + step] += np.float32(rng.choice([0.0, -30.0, -60.0, -100.0, -500.0, 20.0]))
+        return r
+    vals = (rng.standard_normal(int(rng.integers(2, 40))) * float(rng.choice([1.0, 5.0, 40.0]))).astype(np.float32)
+    return vals[rng.integers(0, len(vals), V)]                          # ties at every level
+
+
+def test_seeded_random_batches_of_mixed_rows(torch_cuda, oracle):
+    """Seeded random cases in which every row of a batch is of its own kind (eleven kinds: constant,
+    uniform, normal, masked stretches, few distinct values, very wide, scattered masks, stretches of
+    equal largest logits with NaN / Inf, stretches at levels hundreds of octaves apart, a handful of
+    values repeated), over the shapes that take the different routes: short and long slices of the
+    streaming path, one row of up to a million tokens, and batches of 40-140 rows of 32-80 thousand
+    tokens, which give the cluster kernel more workgroups than the GPU holds at once.  Some cases carry
+    penalties, some hand the logits over as bfloat16 / float16.  Each case goes through every path
+    (the cases of this generator found both a wrong tie count on the streaming path and a lost
+    workgroup in the cluster kernel, each at a rate of about one call in a hundred of one shape)."""
+    torch = torch_cuda
+    from tests import capi
+    rng = np.random.default_rng(4242)
+    for case in range(160):
+        mode = case % 8
+        if mode == 0:
+            B, V = int(rng.integers(1, 4)), 4 * int(rng.integers(150000, 262145))
+        elif mode in (1, 5):
+            B, V = int(rng.integers(40, 140)), 4 * int(rng.integers(8000, 20000))
+        elif mode == 2:
+            B, V = int(rng.integers(1, 24)), 4 * int(rng.integers(1, 2000))
+        elif mode == 3:
+            B, V = int(rng.integers(1, 8)), 4 * int(rng.integers(65537, 110000))
+        elif mode == 4:
+            B, V = int(rng.integers(5, 12)), 4 * int(rng.integers(100000, 140000))
+        else:
+            B, V = int(rng.integers(1, 24)), 4 * int(rng.integers(1, 60000))
+        same = rng.random() < 0.3
+        k0 = int(rng.integers(0, 11))
+        lg = np.stack([_random_row(rng, k0 if same else int(rng.integers(0, 11)), V) for _ in range(B)])
+        temp = float(rng.choice([0.05, 0.5, 0.8, 1.0, 1.3, 4.0, 100.0]))
+        top_k = int(rng.choice([-1, 1, 2, 10, 50, 100, 1000, 1024, 1025, 10000]))
+        top_p = float(rng.choice([0.0, 0.01, 0.1, 0.3, 0.5, 0.7, 0.9, 0.99, 1.0]))
+        kw = {}
+        pick = rng.random()
+        if pick < 0.15:
+            kw = dict(pen_np=(rng.random((B, V)) < 0.02).astype(np.float32) * rng.exponential(1.0, (B, V)).astype(np.float32),
+                      presence=float(rng.choice([0.0, 0.1, 1.0])), repetition=float(rng.choice([0.0, 0.1, 0.5])),
+                      decay=float(rng.choice([1.0, 0.95])))
+        elif pick < 0.3:
+            dt = torch.bfloat16 if rng.random() < 0.5 else torch.float16
+            lg = torch.from_numpy(np.nan_to_num(lg, nan=0.0)).to(dt).float().numpy()
+            kw = dict(dtype=dt)
+        _run_case(torch, oracle, capi, lg, temp, top_k, top_p, u_np=H.uniforms(B, 7000 + case),
+                  what="mixed batch %d shape %d" % (case, mode), **kw)
+
+
 def test_one_workspace_many_shapes(torch_cuda, oracle):
     """Calls of different (B, V, top_k) -- and so of different paths and layouts -- on one workspace sized
     for the largest B and the largest V: what one call leaves behind must not disturb the next."""
