@@ -4,6 +4,7 @@ so every compared field must be EQUAL (sampled index, threshold, kept set as
 {e >= thr} from bit-identical e, counts, integer masses); updated penalties are
 compared bit for bit as well (the stated bar is 1e-6 relative)."""
 import os
+from ctypes import c_void_p as C_void_p
 
 import numpy as np
 import pytest
@@ -773,6 +774,50 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     res = plain.sample(lg_ties, c, k, p, uniforms=u)     # no report words: streams whatever happened before
     _check(res, *ref_ties, "bounded, zeroed workspace")
     assert policy(plain) == -1 and plain.status() == 0 and smp.status() == 0
+
+
+def test_two_streams_two_workspaces_concurrently(torch_cuda, oracle):
+    """Calls on two streams, each with its own workspace, state and outputs, issued alternately
+    without any synchronisation in between, so that their kernels share the GPU: a cluster-path
+    workload (64 rows, nucleus sampling, several workgroups per row waiting for each other) beside a
+    streaming-path one and a penalty chain.  Every call's result equals the oracle's and no wait
+    gives up."""
+    torch = torch_cuda
+    from tests import capi
+    L = capi.lib()
+    N = 10
+    jobs = []
+    for (B, V, k_in, p_in, temp, sigma, pen_on, seed) in [(64, 152064, -1, 0.9, 0.8, 2.0, False, 1),
+                                                        (48, 131072, 50, 0.95, 1.0, 1.5, False, 2),
+                                                        (32, 131072, 40, 0.9, 1.0, 2.0, True, 3)]:
+        lg_np = H.logits_normal(B, V, sigma, seed=seed)
+        rc, c, k, p = capi.normalize(temp, k_in, p_in, V, B, 1)
+        us = [H.uniforms(B, 100 * seed + i) for i in range(N)]
+        pen_ref = H.penalties_sparse(B, V, seed=seed) if pen_on else None
+        refs = []
+        for i in range(N):
+            kw = dict(penalties=pen_ref, presence=0.2, repetition=0.1, decay=0.97) if pen_on else {}
+            refs.append(oracle.sample_batch(lg_np, c, k, p, injected_u=us[i], **kw)[0])
+        jobs.append(dict(B=B, V=V, c=c, k=k, p=p, lg=torch.from_numpy(lg_np).cuda(), smp=capi.Sampler(B, V),
+                         u=[torch.from_numpy(u).cuda() for u in us], refs=refs, pen_ref=pen_ref,
+                         pen=torch.from_numpy(H.penalties_sparse(B, V, seed=seed)).cuda() if pen_on else None,
+                         out=[torch.full((B,), -7, dtype=torch.int32, device="cuda") for _ in range(N)]))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()]
+    for i in range(N):
+        for j, st in zip(jobs, streams):
+            rc = L.rs_sample(j["lg"].data_ptr(), j["V"], j["pen"].data_ptr() if j["pen"] is not None else None,
+                             j["out"][i].data_ptr(), None, j["u"][i].data_ptr(), j["B"], j["V"], 0.2, 0.1, 0.97,
+                             j["c"], j["k"], j["p"], j["smp"].ws.data_ptr(), j["smp"].ws.numel(), None, None,
+                             C_void_p(st.cuda_stream))
+            assert rc == 0
+    torch.cuda.synchronize()
+    for n, j in enumerate(jobs):
+        assert j["smp"].status() == 0, n
+        for i in range(N):
+            assert np.array_equal(j["out"][i].cpu().numpy(), j["refs"][i]), (n, i)
+        if j["pen"] is not None:
+            assert np.array_equal(j["pen"].cpu().numpy().view(np.uint32), j["pen_ref"].view(np.uint32))
 
 
 def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
