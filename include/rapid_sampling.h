@@ -11,7 +11,9 @@
  * caller; `stream` is a hipStream_t passed as void* (NULL = the null stream);
  * calls enqueue work on `stream` and return without synchronising; the return
  * value is RS_OK or a negative RS_ERR_* code; nothing throws, and only the
- * calls that say so allocate.
+ * calls that say so allocate.  The library keeps no state of its own between
+ * calls: what a call needs beyond its arguments lives in the workspace and,
+ * optionally, in an rs_policy object, both owned by the caller.
  */
 #ifndef RAPID_SAMPLING_H
 #define RAPID_SAMPLING_H
@@ -93,13 +95,20 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
 int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes);
 
 /*
- * Zero a freshly allocated workspace (device memory, 256-byte aligned).  Call
- * once after allocation, and again after a call reported RS_ERR_DEVICE;
- * rs_sample leaves the workspace ready for the next call on the same stream.
- * The first call for a workspace address also allocates 64 bytes of pinned
- * host memory (see rs_workspace_policy), kept until the process ends.
+ * Zero a freshly allocated workspace (device memory, 256-byte aligned) with a
+ * fill kernel on `stream`.  Call once after allocation, and again after a call
+ * reported RS_ERR_DEVICE; rs_sample leaves the workspace ready for the next
+ * call on the same stream.  Allocates nothing.
  */
 int rs_workspace_init(void *workspace_device, size_t bytes, void *stream);
+
+/*
+ * How long a workgroup waits for its peers before it gives up with
+ * RS_ERR_DEVICE, in milliseconds (0 = the default, 2000).  Stored in the
+ * workspace header by a one-thread kernel on `stream`; rs_workspace_init
+ * resets it to the default.  For tests of the error path.
+ */
+int rs_workspace_set_wait_limit(void *workspace_device, uint32_t milliseconds, void *stream);
 
 /*
  * Read back the sticky device error word of a workspace (synchronises
@@ -108,21 +117,38 @@ int rs_workspace_init(void *workspace_device, size_t bytes, void *stream);
 int rs_workspace_status(const void *workspace_device, int32_t *status, void *stream);
 
 /*
- * Diagnostic: how calls that could take the wait-free streaming path are
- * currently routed on this workspace.  A row that path cannot finish is handed
- * to the general kernel in a further launch, and a call whose rows mostly end
- * that way has wasted a pass: with a bounding top_k (<= 1024) that takes
- * unusual rows (ties of thousands of tokens, slices of a row more than 87
- * octaves apart), without one (top_p < 1 alone) a flat distribution.  Each
- * streaming call reports "most rows handed on: yes/no" to a word of pinned
- * host memory that rs_sample reads, without waiting, before the next call.
- * *state: -1 the workspace was not set up by rs_workspace_init (calls with a
- * bounding top_k always stream, calls without never do); otherwise bit 0 set:
- * calls without a bounding top_k currently go to the general kernel, bit 1
- * set: so do calls with one; in both cases one call in 64 streams again.
- * Results do not depend on the routing.  No counterpart in the reference.
+ * Routing state of the streaming path and an asynchronous error report, owned
+ * by the caller (optional; one per workspace).  No counterpart in the
+ * reference.
+ *
+ * A row the wait-free streaming path cannot finish is handed to the general
+ * kernel in a further launch, and a call whose rows mostly end that way has
+ * wasted a pass: with a bounding top_k (<= 1024) that takes unusual rows (ties
+ * of thousands of tokens), without one (top_p < 1 alone) a flat distribution.
+ * Each streaming call that is given a policy reports "most rows handed on:
+ * yes/no" to a word of pinned host memory inside it, and rs_sample_ex reads
+ * that word, without waiting, before it routes the next call: after a call
+ * that handed most rows on, calls of that kind go straight to the general
+ * kernel and one in 64 streams again.  Without a policy, calls with a bounding
+ * top_k always stream and calls without never do.  Results do not depend on
+ * the routing.
+ *
+ * A kernel that gives up waiting (RS_ERR_DEVICE) also writes the code into a
+ * third pinned word, which rs_policy_error reads without synchronising.
+ *
+ * rs_policy_create allocates (a small host object and 64 bytes of pinned host
+ * memory); rs_policy_destroy frees them -- only after the last call that was
+ * given the policy has completed on the device.
+ * rs_policy_state: bit 0 set: calls without a bounding top_k currently go to
+ * the general kernel, bit 1 set: so do calls with one.
+ * rs_policy_error: *error = RS_OK or RS_ERR_DEVICE as last reported; with
+ * clear != 0 the word is reset.
  */
-int rs_workspace_policy(const void *workspace_device, int32_t *state);
+typedef struct rs_policy rs_policy;
+int  rs_policy_create(rs_policy **policy_out);
+void rs_policy_destroy(rs_policy *policy);
+int  rs_policy_state(const rs_policy *policy, int32_t *state);
+int  rs_policy_error(rs_policy *policy, int32_t *error, int32_t clear);
 
 /*
  * setup_rand (sampling.cu:136-144): initialise B records of RNG state for
@@ -150,18 +176,18 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  *   workspace_device  rs_workspace_bytes(B,V) bytes, initialised once.
  *   diag_device       B rs_row_diag records, or NULL.
  *   e_bits_device     (B,V) uint32: bit patterns of e = 2^(x - floor(max x))
- *                     per token (2^-40 <= e < 2), or NULL.  Together with
- *                     diag.thr_bits this is the kept set {e >= thr}.
+ *                     per token (2^-40 <= e < 2, or 0 for a dead token: e
+ *                     below 2^-40 has probability 0 and is never returned),
+ *                     or NULL.  Together with diag.thr_bits this is the kept
+ *                     set {e >= thr}.
  *
  * Calls that share a workspace must be ordered on one stream.
  *
  * The call is one kernel launch, or three for calls of at least 2^17 tokens
  * without penalties whose kept set is expected to be small (a wait-free pass
  * over the logits, a per-row finish, and the general kernel for rows the
- * finish hands on; see rs_workspace_policy); results are identical either
- * way.  Two environment variables exist for tests: RS_FORCE_R (1..32, float4
- * per thread of the general kernel) and RS_FORCE_PATH (cluster | stream |
- * optimistic).
+ * finish hands on; see rs_policy); results are identical either way.  No
+ * environment variable is read.
  */
 int rs_sample(const float *logits_device, int64_t row_stride,
               float *penalties_device, int32_t *out_device,
@@ -194,6 +220,35 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
                     void *workspace_device, size_t workspace_bytes,
                     rs_row_diag *diag_device, uint32_t *e_bits_device,
                     void *stream);
+
+/*
+ * rs_sample_dtype with explicit options (NULL = all defaults, which makes it
+ * rs_sample_dtype).  `path` forces the way through the library (tests,
+ * benchmarks): RS_PATH_CLUSTER the general one-launch kernel, RS_PATH_STREAM
+ * the streaming path when top_k <= 1024 (else the general kernel),
+ * RS_PATH_ATTEMPT the streaming path whatever top_k is; penalties always take
+ * the general kernel.  `slice_r` forces the float4 groups per thread of the
+ * general kernel (1, 2, 4, 8, 16 or 32; 0 = chosen by the library).
+ * `policy` see rs_policy.  No counterpart in the reference.
+ */
+#define RS_PATH_AUTO    0
+#define RS_PATH_CLUSTER 1
+#define RS_PATH_STREAM  2
+#define RS_PATH_ATTEMPT 3
+typedef struct rs_options {
+    int32_t    path;
+    int32_t    slice_r;
+    rs_policy *policy;
+} rs_options;
+int rs_sample_ex(const void *logits_device, int32_t logits_dtype, int64_t row_stride,
+                 float *penalties_device, int32_t *out_device,
+                 void *rng_state_device, const float *injected_u_device,
+                 int32_t B, int32_t V,
+                 float presence_penalty, float repetition_penalty, float penalty_decay,
+                 float log2e_inv_temp, int32_t top_k, float top_p,
+                 void *workspace_device, size_t workspace_bytes,
+                 rs_row_diag *diag_device, uint32_t *e_bits_device,
+                 const rs_options *options, void *stream);
 
 /*
  * Launch-plus-one-read floor: a kernel with rs_sample's grid for (B,V) that

@@ -140,11 +140,12 @@ def e_bits(x, M):
 
 
 def w_of(bits):
-    """Exact integer weights W = e * 2^63 of bit patterns (array) as uint64."""
+    """Exact integer weights W = e * 2^63 of bit patterns (array) as uint64; 0 for dead tokens (e = 0)."""
     bits = np.ascontiguousarray(bits, dtype=np.uint32)
+    live = bits >= np.uint32(0x2B800000)
     m = (bits & np.uint32(0x7FFFFF)).astype(np.uint64) | np.uint64(0x800000)
-    ex = (bits >> np.uint32(23)).astype(np.uint64)
-    return m << (ex - np.uint64(87))
+    ex = np.where(live, bits >> np.uint32(23), np.uint32(87)).astype(np.uint64)
+    return np.where(live, m << (ex - np.uint64(87)), np.uint64(0))
 
 
 def ceil_mul(f, s):

@@ -18,8 +18,11 @@
  *     e = poly5(f) * 2^(n - M) with M = floor(max x), a fixed degree-5 Horner
  *     polynomial with positive coefficients (monotone, poly(1) < 2).  The
  *     significand of e depends on x alone; the maximum only shifts the
- *     exponent.  e is clamped from below at 2^-40 (tokens further down all
- *     become exactly 2^-40), so 2^-40 <= e < 2 and e_max in [1,2);
+ *     exponent.  Below 2^-40 e is flushed to zero, as the reference's
+ *     exp2f(x - max) underflows to zero 149 octaves down (:235): such a token
+ *     has probability exactly 0, takes no part in the selection and can never
+ *     be returned (a logit masked with -inf must not come back, however large
+ *     top_k and top_p are).  So e = 0 or 2^-40 <= e < 2, and e_max in [1,2);
  *   - the probability of token i is carried as the exact integer
  *         W_i = e_i * 2^63  =  significand24(e_i) << (exponent(e_i) - 87),
  *     the row total D = sum W_i (up to 2^84: 128-bit) replaces the float
@@ -68,7 +71,8 @@ float rs_oracle_scale(float logit, float penalty, int has_penalty, float c)
  * [0,1]; 2^f is a degree-5 minimax polynomial (relative error 8.3e-8)
  * evaluated by Horner with fmaf, all coefficients positive, so it is monotone
  * in f and poly(1) < 2 = 2*poly(0): e is monotone in x.  The exponent n - M
- * is added to the exponent field; below 2^-40 the result is 2^-40 exactly.
+ * is added to the exponent field; below 2^-40 the result is flushed to zero
+ * (bit pattern 0): a dead token.
  */
 static const float RS_C1 = 0x1.62e4bap-1f;
 static const float RS_C2 = 0x1.ebdb56p-3f;
@@ -88,12 +92,14 @@ uint32_t rs_oracle_e_bits(float x, float M)
     p = fmaf(p, f, 1.0f);
     float k = fmaxf(n - M, -41.0f);             /* <= 0; anything below -40 is clamped anyway */
     uint32_t b = f2u(p) + ((uint32_t)(int32_t)k << 23);
-    return b < RS_E_MIN_BITS ? RS_E_MIN_BITS : b;
+    return b < RS_E_MIN_BITS ? 0u : b;
 }
 
-/* exact weight of a token: e * 2^63 = significand24 << (exponent - 87), in [2^23, 2^64) */
+/* exact weight of a token: e * 2^63 = significand24 << (exponent - 87), in [2^23, 2^64);
+ * 0 for a dead token (e flushed to zero) */
 uint64_t rs_oracle_w(uint32_t e_bits)
 {
+    if (e_bits < RS_E_MIN_BITS) return 0;
     uint64_t m = (e_bits & 0x7FFFFFu) | 0x800000u;
     int ex = (int)(e_bits >> 23);
     return m << (ex - 87);
@@ -237,11 +243,16 @@ void rs_oracle_row(const float *logits, float *penalties, int32_t V,
     dg.xmax = xmax;
     const float M = floorf(xmax);
 
-    /* 2. e = 2^(x - M), total D (sampling.cu:228-258 without the division) */
+    /* 2. e = 2^(x - M), total D (sampling.cu:228-258 without the division).
+     *    Dead tokens (e = 0) weigh nothing and are left out of everything that
+     *    follows; the token at the maximum has e >= 1, so a row is never all dead. */
     u128 D = 0;
     uint32_t emin = 0xFFFFFFFFu, emax = 0;
+    uint64_t n_live = 0;
     for (int32_t i = 0; i < V; i++) {
         eb[i] = rs_oracle_e_bits(x[i], M);
+        if (eb[i] == 0) continue;
+        n_live++;
         D += rs_oracle_w(eb[i]);
         if (eb[i] < emin) emin = eb[i];
         if (eb[i] > emax) emax = eb[i];
@@ -252,7 +263,7 @@ void rs_oracle_row(const float *logits, float *penalties, int32_t V,
     /* 3. the reference's quaternary search, literally (sampling.cu:261-329),
      *    with exact counts and integer masses */
     uint32_t left = emin, right = emax + 1;
-    uint64_t cnt_x = (uint64_t)V;
+    uint64_t cnt_x = n_live;
     u128 mass_x = D;
     uint32_t rounds = 0;
     while ((cnt_x > (uint64_t)top_k || mass_x > P) && left < right - 1) {
@@ -263,6 +274,7 @@ void rs_oracle_row(const float *logits, float *penalties, int32_t V,
         u128 my = 0, mz = 0, mw = 0;
         for (int32_t i = 0; i < V; i++) {
             uint32_t b = eb[i];
+            if (b == 0) continue;
             uint64_t w = rs_oracle_w(b);
             if (b >= py) { cy++; my += w; }
             if (b >= pz) { cz++; mz += w; }

@@ -34,14 +34,14 @@
 extern "C" {
 #endif
 
-/* e is clamped from below at 2^-40 (bit pattern 0x2B800000). */
+/* The smallest live e is 2^-40 (bit pattern 0x2B800000); below it e is flushed to zero. */
 #define RS_E_MIN_BITS 0x2B800000u
 
 /* Per-row diagnostics; mirrors rs_row_diag of include/rapid_sampling.h.
  * 128-bit quantities are (low word, high word). */
 typedef struct {
     float    xmax;        /* row maximum of the scaled logits                 */
-    uint32_t emin_bits;   /* bit pattern of the smallest e in the row         */
+    uint32_t emin_bits;   /* bit pattern of the smallest live (non-zero) e     */
     uint64_t D[2];        /* sum of the weights W over the row                */
     uint64_t P[2];        /* ceil(top_p * D)                                  */
     uint32_t left_bits;   /* `left` when the reference's search loop ends     */

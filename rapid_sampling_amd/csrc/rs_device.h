@@ -27,13 +27,23 @@ __device__ __forceinline__ float sf(float x)
 
 typedef unsigned __int128 u128;
 
-constexpr uint32_t kEMinBits = 0x2B800000u;               // bit pattern of 2^-40, the smallest e
+constexpr uint32_t kEMinBits = 0x2B800000u;               // bit pattern of 2^-40, the smallest live e
+constexpr uint32_t kDeadBits = 0x2B000000u;               // 2^-41: where the registers keep what lies below
+
+// A token whose e falls below 2^-40 is DEAD: its probability is exactly 0 (the reference's
+// exp2f(x - max) underflows to 0 likewise, 149 octaves down, sampling.cu:235), it takes no part
+// in the selection and can never be returned -- a logit masked with -inf must not come back
+// however large top_k and top_p are.  In registers and histograms a dead token is any bit
+// pattern below kEMinBits (kept at or above kDeadBits so that it still has a histogram bin,
+// one octave below the live ones, where counts can be checked for completeness); everything
+// that weighs or selects tokens looks at patterns >= kEMinBits only.
 
 // Bit pattern of e = 2^(x - M), M = floor(max x) of the row (reference:
 // exp2f(x - max) at sampling.cu:235; the common factor 2^(max - M) cancels in
 // every probability).  n = floor(x) and f = x - n are exact; 2^f is a degree-5
 // Horner polynomial with positive coefficients (monotone, poly(1) < 2); the
-// result is scaled by 2^(n - M), n - M <= 0, and clamped from below at 2^-40.
+// result is scaled by 2^(n - M), n - M <= 0; what falls below 2^-40 is dead
+// (kept here as something in [2^-41, 2^-40), see above).
 // The significand depends on x alone, so a slice can use its own M and be
 // re-based later by an exponent shift.
 //
@@ -42,7 +52,7 @@ constexpr uint32_t kEMinBits = 0x2B800000u;               // bit pattern of 2^-4
 // count is kept down by hand: the Horner steps with a literal addend are
 // written as v_fmaak_f32 (the compiler otherwise spends a move per step on
 // some of them), and the scaling is v_cvt_i32_f32 (which saturates) +
-// v_ldexp_f32 (exact; anything below 2^-40, zero included, ends at the clamp).
+// v_ldexp_f32 (exact; anything below 2^-41, zero included, ends at the clamp).
 __device__ __forceinline__ uint32_t e_bits_of(float x, float M)
 {
     const float n = __builtin_floorf(x);
@@ -54,10 +64,10 @@ __device__ __forceinline__ uint32_t e_bits_of(float x, float M)
     p = __builtin_fmaf(p, f, 1.0f);
     int k;
     asm("v_cvt_i32_f32 %0, %1" : "=v"(k) : "v"(n - M));
-    return __float_as_uint(fmaxf(__builtin_ldexpf(p, k), 0x1p-40f));
+    return __float_as_uint(fmaxf(__builtin_ldexpf(p, k), 0x1p-41f));
 }
 
-// The same without the clamp: whatever lies below 2^-40 (zero included) stands for 2^-40.  For
+// The same without the clamp: whatever lies below 2^-40 (zero included) is dead.  For
 // code that can tell such tokens by their bin and saves the instruction.
 __device__ __forceinline__ uint32_t e_bits_raw(float x, float M)
 {
@@ -73,7 +83,7 @@ __device__ __forceinline__ uint32_t e_bits_raw(float x, float M)
     return __float_as_uint(__builtin_ldexpf(p, k));
 }
 
-// Exact weight of a token from the bit pattern of e (2^-40 <= e < 2):
+// Exact weight of a live token from the bit pattern of e (2^-40 <= e < 2):
 // W = e * 2^63 = significand24 << (exponent - 87), in [2^23, 2^64).
 __device__ __forceinline__ uint64_t w_of_bits(uint32_t b)
 {

@@ -38,8 +38,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
-#include <mutex>
-#include <unordered_map>
+#include <new>
 
 #include "rapid_sampling.h"
 #include "rs_device.h"
@@ -62,9 +61,7 @@ struct alignas(256) WsHeader {
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows the streaming pass handed to the cluster kernel
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
-    uint32_t pad0[2];
-    int32_t *hint;        // two words of pinned host memory the streaming path reports to, or null
-    uint32_t pad[54];
+    uint32_t pad[59];
 };
 
 // How long a workgroup waits for its peers before it gives up (wall-clock ticks).
@@ -108,6 +105,7 @@ struct Params {
     const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
     int32_t      dtype;        // RS_DTYPE_* of the logits
     uint32_t     report;       // which of the two report words a streaming call writes: 0 top_k bounds the kept set, 1 not
+    int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1] routing reports, [2] error; or null
     int64_t      row_stride;
     int32_t      B, V;
     uint32_t     G;            // workgroups per row
@@ -160,11 +158,12 @@ __device__ __forceinline__ u128 pack_mass(uint64_t w, uint32_t ex)
 }
 
 // Bits of e in a frame `delta` octaves above the one they were computed in
-// (delta <= 64): the exponent drops by delta, clamped at 2^-40.
+// (delta <= 64): the exponent drops by delta; what falls below 2^-40 is dead
+// (kept at or above 2^-41).
 __device__ __forceinline__ uint32_t rebase_bits(uint32_t b, uint32_t delta)
 {
     const uint32_t d = delta << 23;
-    return max(b, d + kEMinBits) - d;
+    return max(b, d + kDeadBits) - d;
 }
 
 // Logits arrive as fp32 or, if the caller opted in, as bf16 or fp16.  Both widen to fp32
@@ -221,6 +220,7 @@ struct Lds {
     uint32_t bc32[8];
     uint32_t ctr;
     int      abort;
+    int32_t *host_words;     // Params::host_words, for the code that gives up a wait
 };
 
 __device__ __forceinline__ uint32_t block_max_u32(Lds &s, uint32_t v, int lane, int wave)
@@ -271,6 +271,11 @@ __device__ __forceinline__ void block_sum2_u128(Lds &s, u128 &a, u128 &b, int la
     for (int w = 0; w < kWaves; ++w) { a += s.q128[w * 2]; b += s.q128[w * 2 + 1]; }
 }
 
+// A wait that ran out of time: the sticky error word of the workspace, the caller's pinned host
+// word if there is one (readable without synchronising), and the flag that makes the workgroup leave.
+struct Lds;
+__device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr);
+
 // Bounded wait bookkeeping: thread 0 looks at the wall clock now and then; the
 // verdict is read by everyone after a workgroup barrier, so it is uniform.
 struct SpinGuard {
@@ -280,12 +285,16 @@ struct SpinGuard {
     // call by every thread once per polling round, before the round's __syncthreads
     __device__ __forceinline__ void tick(Lds &s, WsHeader *hdr)
     {
-        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(hdr)) {
-            a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
-            s.abort = 1;
-        }
+        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(hdr)) give_up(s, hdr);
     }
 };
+
+__device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr)
+{
+    a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
+    if (s.host_words) __hip_atomic_store(s.host_words + 2, (int32_t)RS_ERR_DEVICE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    s.abort = 1;
+}
 
 __device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)
 {
@@ -345,10 +354,12 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
 // takes slot t).  Once all is there the row's frame M = floor(max) is known,
 // and both histograms are stored in that frame: position c holds bin 348 + r,
 // r = c - pos(M) mod 512; r >= 164 lies below 2^-40 of the frame, where
-// tokens are clamped: their count goes to bin 348, without fraction bits.
-// Indices below 348 of s.g and s.hm are left stale.  Returns 0 on success, 1
-// when the slices' maxima are too far apart for shared positions (s.g and
-// s.hm are then undefined), -1 when the wait gave up.
+// tokens are dead: they were counted (the counts must add up) and are dropped.
+// Indices below 348 of s.g and s.hm are left stale.  A slice's dead tokens
+// sit one octave below its 41 live ones, so positions are shared safely while
+// the slices' maxima lie within 86 octaves of each other.  Returns 0 on
+// success, 1 when they do not (s.g and s.hm are then undefined), -1 when the
+// wait gave up.
 __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G, uint64_t *gh, const uint32_t *slots,
                                               uint32_t expected, uint32_t &kmax_out, int lane, int wave)
 {
@@ -387,16 +398,11 @@ __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G,
     kmin = ~kmin;
     kmax_out = kmax;
     const float M = __builtin_floorf(fkey_inv(kmax));
-    if (!(M - __builtin_floorf(fkey_inv(kmin)) < 88.0f)) return 1;
+    if (!(M - __builtin_floorf(fkey_inv(kmin)) < 87.0f)) return 1;
     const uint32_t m4 = (uint32_t)(int)(M - 128.0f * __builtin_floorf(M * 0.0078125f)) * 4u;
     const uint32_t r0 = ((uint32_t)tid + 160u - m4) & 511u, r1 = ((uint32_t)tid + kThreads + 160u - m4) & 511u;
-    uint32_t glow = 0, hlow = 0;
-    if (r0 < 164u) { s.g[kBin0 + r0] = g0; s.hm[kBin0 + r0] = h0; } else { glow += pack_count(g0); hlow += pack_count(h0); }
-    if (r1 < 164u) { s.g[kBin0 + r1] = g1; s.hm[kBin0 + r1] = h1; } else { glow += pack_count(g1); hlow += pack_count(h1); }
-    if (glow) atomicAdd(&s.bc32[3], glow);
-    if (hlow) atomicAdd(&s.bc32[4], hlow);
-    __syncthreads();
-    if (tid == 0) { s.g[kBin0] += (uint64_t)s.bc32[3] << 43; s.hm[kBin0] += (uint64_t)s.bc32[4] << 43; }
+    if (r0 < 164u) { s.g[kBin0 + r0] = g0; s.hm[kBin0 + r0] = h0; }
+    if (r1 < 164u) { s.g[kBin0 + r1] = g1; s.hm[kBin0 + r1] = h1; }
     __syncthreads();
     return 0;
 }
@@ -682,7 +688,6 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         }
         kmax_row = block_max_u32(s, fkey(lmax), lane, wave);            // of this slice, for now
         for (int b = tid; b < kNB * kRepC; b += kThreads) s.hr[b] = 0;
-        if (tid == 0) { s.bc32[3] = 0; s.bc32[4] = 0; }
         // every workgroup posts its key (never 0 for a finite x) in its own slot
         if (G > 1 && tid == 0) a_store(&rc->mx[part], kmax_row);
         __syncthreads();
@@ -690,7 +695,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
     // ---- 2. e in the slice's own frame; level-1 histogram --------------------
     // The significand of e does not depend on the frame, so the row's maximum is not needed
     // yet: bins are kept by absolute octave (mod 128, 4 bins each), where the slices' bins
-    // add up as long as their maxima lie within 87 octaves of each other.  The maxima come
+    // add up as long as their maxima lie within 86 octaves of each other.  The maxima come
     // back with the histogram, in the same polling rounds.
     const float Mloc = __builtin_floorf(fkey_inv(kmax_row));
     const uint32_t pos0 = G > 1 ? (uint32_t)(int)(Mloc - 128.0f * __builtin_floorf(Mloc * 0.0078125f)) * 4u - 508u : 0u;
@@ -769,7 +774,11 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
         uint4 *dst = reinterpret_cast<uint4 *>(p.e_bits + (int64_t)row * p.V);
 #pragma unroll
         for (int j = 0; j < R; ++j)
-            if (j < nv) dst[base4 + j * kThreads] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
+            if (j < nv) {
+                // dead tokens are reported as e = 0
+                auto live = [](uint32_t b) { return b < kEMinBits ? 0u : b; };
+                dst[base4 + j * kThreads] = make_uint4(live(eb[j * 4]), live(eb[j * 4 + 1]), live(eb[j * 4 + 2]), live(eb[j * 4 + 3]));
+            }
     }
     const float xmax = fkey_inv(kmax_row);
     const uint64_t top_k = (uint64_t)p.top_k;
@@ -1017,8 +1026,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
                 uint32_t spins = 0, v;
                 while ((v = a_load(&rc->index_p1)) == 0u) {
                     if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(p.hdr)) {
-                        a_store(&p.hdr->error, (int32_t)RS_ERR_DEVICE);
-                        s.abort = 1;
+                        give_up(s, p.hdr);
                         break;
                     }
                 }
@@ -1075,13 +1083,13 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     __shared__ Lds s;
     if (p.G == 1) {
         // one workgroup per row: nobody waits for anybody, the hardware's ids will do
-        if (threadIdx.x == 0) s.abort = 0;
+        if (threadIdx.x == 0) { s.abort = 0; s.host_words = p.host_words; }
         __syncthreads();
         sample_slice<R, PEN>(p, s, blockIdx.x, 0u);
         return;
     }
     if (threadIdx.x == 0) {
-        s.abort = 0;
+        s.abort = 0; s.host_words = p.host_words;
         const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
         // every workgroup of the launch takes exactly one ticket: after the last one the counter
         // is not touched again, and is put back for the next call
@@ -1097,14 +1105,11 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
 // The launch that follows the streaming pass knows how many rows were handed on.  Its first
 // workgroup tells the host -- a word of pinned memory that rs_sample looks at, without waiting,
 // before its next call -- whether that was most of them: such calls are then better served by
-// the cluster kernel alone for a while.
+// the cluster kernel alone for a while.  The word belongs to the caller's rs_policy.
 __device__ __forceinline__ void report_streaming(const Params &p, uint32_t handed_on)
 {
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-        int32_t *hint = p.hdr->hint;
-        if (hint)
-            __hip_atomic_store(hint + p.report, handed_on * 2u > (uint32_t)p.B ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.host_words)
+        __hip_atomic_store(p.host_words + p.report, handed_on * 2u > (uint32_t)p.B ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // The launch that follows the streaming pass: workgroups work through the
@@ -1120,7 +1125,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
     for (;;) {
         __syncthreads();
         if (threadIdx.x == 0) {
-            s.abort = 0;
+            s.abort = 0; s.host_words = p.host_words;
             s.bc32[0] = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
         }
         __syncthreads();
@@ -1143,7 +1148,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
     report_streaming(p, n);
     if (n == 0u) return;                                         // nothing left over: no ticket was taken
     if (threadIdx.x == 0) {
-        s.abort = 0;
+        s.abort = 0; s.host_words = p.host_words;
         const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
         if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);     // the last ticket of the launch
         s.bc32[0] = t;
@@ -1199,10 +1204,9 @@ struct StreamView {
 
 // Lanes of a wave that add to one LDS address are served one after the other, and rows often put
 // most of their tokens into a few bins.  So each bin is kept in kRep copies (lane l adds to copy
-// l % kRep), and e is not clamped at 2^-40 before it is counted: the histogram spans all 512
-// values of bits >> 21, the tokens below 2^-40 -- often most of a row -- spread over the bins
-// below kBin0 by their own exponents, and those bins hand their counts to bin kBin0 afterwards
-// (such a token weighs 2^-40 exactly: a count and no fraction bits).  The histogram is done with
+// l % kRep), and e is not clamped before it is counted: the histogram spans all 512 values of
+// bits >> 21, the dead tokens (below 2^-40, often most of a row) spread over the bins below
+// kBin0 by their own exponents, where nobody looks at them again.  The histogram is done with
 // before the candidates are staged, and shares their memory.
 // Eight copies for long slices; two for the short slices of small calls, where clearing and
 // folding the copies would cost more than the few tokens of a thread.
@@ -1220,7 +1224,6 @@ struct LdsA {
     uint32_t sub[128];           // level-2 counts inside a boundary bin too large for the stash
     uint32_t u32[16];
     uint32_t cov, n, cut, over;
-    uint32_t low;                // tokens of the slice below 2^-40
 };
 
 template <int R, int NT, int DT>     // NT threads, each with R groups of four tokens of the slice; DT the logits' type
@@ -1288,7 +1291,6 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         for (int i = 0; i < kNB * kRep / 2 / NT; ++i) z[tid + i * NT] = make_uint4(0u, 0u, 0u, 0u);
         static_assert(kNB * kRep % (2 * NT) == 0, "whole stores");
     }
-    if (tid == 0) s.low = 0;
     if (blockIdx.x == 0 && tid == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
     uint32_t k = wave_max_u32(fkey(lmax));
     if (lane == 0) s.u32[wave] = k;
@@ -1314,22 +1316,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         }
     }
     __syncthreads();
-    {
-        // the tokens below 2^-40: counted into bin kBin0
-        uint32_t low = 0;
-        const uint4 *two = reinterpret_cast<const uint4 *>(s.hm);                // two bins per load; counts sit in y and w
-        for (int i = tid; i < (int)kBin0 * kRep / 2; i += NT) {
-            const uint4 q = two[i];
-            low += (q.y >> 11) + (q.w >> 11);
-        }
-        low = wave_sum(low);
-        if (lane == 0 && low) {
-            atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[kBin0 * kRep]), (unsigned long long)low << 43);
-            atomicAdd(&s.low, low);
-        }
-    }
-    __syncthreads();
-    // Add the slice's bins to the row's, which are kept by absolute octave (mod 128, 4 bins each):
+    // Add the slice's live bins to the row's, which are kept by absolute octave (mod 128, 4 bins each):
     // bin t of this frame is octave M - 40 + t/4.  Slices of one row may use different frames; as
     // long as their maxima lie within 87 octaves of each other no two octaves in use coincide.
     auto bin_total = [&](int b) {
@@ -1368,7 +1355,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
         uint32_t run = ci - cs;
         const uint32_t total = lane63(ci);
         if (lane == 0) s.over = 0xFFFFFFFFu;
-        if (lane == 0 && total < Ks) { s.cov = 0u; s.n = total; s.cut = kBin0 << 21; }   // a short slice: all of it
+        if (lane == 0 && total < Ks) { s.cov = 0u; s.n = total; s.cut = kBin0 << 21; }   // a short slice: all its live tokens
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
             const int b = kSB - 1 - 3 * lane - i;
@@ -1407,9 +1394,6 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
                     const uint32_t b = eb[j * 4 + q];
                     if ((b >> 21) == ob) atomicAdd(&s.sub[(b >> 14) & 127u], 1u);
                 }
-            // in the lowest bin, the tokens below 2^-40 (not counted above: their bits say another
-            // bin) all weigh 2^-40 exactly
-            if (ob == kBin0 && tid == 0 && s.low) atomicAdd(&s.sub[0], s.low);
         }
         __syncthreads();
         if (wave == 0) {
@@ -1432,17 +1416,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
     }
     const uint32_t cov = s.cov, n = s.n;
     const uint32_t cut = s.cut;
-    // From here on the bits in the registers are compared with the cut.  Above 2^-40 they are what
-    // they should be; if the cut lies at 2^-40 itself (the stash takes all of a slice, tokens
-    // down there included) they are clamped first.
-    if (cut == kEMinBits) {
-#pragma unroll
-        for (int j = 0; j < R; ++j)
-            if (j < nv) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) eb[j * 4 + q] = max(eb[j * 4 + q], kEMinBits);
-            }
-    }
+    // From here on the bits in the registers are compared with the cut, which is never below
+    // 2^-40: dead tokens are no candidates.
 
     // Candidates (bits >= cut) are at most n <= kStashCap, so at most that many float4 groups
     // hold one.  Each thread copies its groups with a candidate into LDS at an offset from a scan
@@ -1547,7 +1522,7 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     const PartHdr *hdrs = v.hdr + (size_t)row * G;
     uint64_t *rowhist = (p.ctl_end - 1 - row)->rowhist;
 
-    if (tid == 0) { s.abort = 0; t.fail = 0; }
+    if (tid == 0) { s.abort = 0; s.host_words = p.host_words; t.fail = 0; }
     PartHdr ph;
     ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.cut = 0;
     if ((uint32_t)tid < G) ph = hdrs[tid];
@@ -1586,34 +1561,29 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     }
     // the row's level-1 histogram in the row's frame: bin r (octave M - 40 + r/4) sits at absolute
     // position 4 (M mod 128) + r - 160; the other 348 positions hold tokens below 2^-40 of this
-    // frame, which are clamped there: a count and no fraction bits
+    // frame, which are dead there: dropped
     {
         const float mm = M - 128.0f * __builtin_floorf(M * 0.0078125f);
         const uint32_t m4 = (uint32_t)(int)mm * 4u;
         const uint32_t r0 = ((uint32_t)tid + 160u - m4) & 511u, r1 = ((uint32_t)tid + kThreads + 160u - m4) & 511u;
-        uint32_t low = 0;
-        if (r0 < (uint32_t)kSB) s.g[kBin0 + r0] = h0; else low += pack_count(h0);
-        if (r1 < (uint32_t)kSB) s.g[kBin0 + r1] = h1; else low += pack_count(h1);
+        if (r0 < (uint32_t)kSB) s.g[kBin0 + r0] = h0;
+        if (r1 < (uint32_t)kSB) s.g[kBin0 + r1] = h1;
         for (int b = tid; b < (int)kBin0; b += kThreads) s.g[b] = 0;
-        low = block_sum_u32(s, low, lane, wave);
-        if (tid == 0) s.g[kBin0] += (uint64_t)low << 43;
         __syncthreads();
         if (mixed) {
             // Slices whose maxima lie 88 octaves or more apart may have put different octaves into
-            // one position.  Every token of a slice 41 octaves or more below the row's frame weighs
-            // 2^-40 there, whatever its bin: what such a slice added is taken out again, bin by bin
-            // (its own bins are on record), and its tokens are counted into the lowest bin.  The
-            // slices that remain lie within 40 octaves of each other.
+            // one position.  Every token of a slice 41 octaves or more below the row's frame is
+            // dead there, whatever its bin: what such a slice added is taken out again, bin by bin
+            // (its own bins are on record).  The slices that remain lie within 40 octaves of each
+            // other.
             for (uint32_t i = (uint32_t)tid; i < G * (uint32_t)kSB; i += kThreads) {
                 const uint32_t g = i / (uint32_t)kSB, r = i - g * (uint32_t)kSB;
                 if (t.delta[g] >= 41u) {
                     const uint64_t w = v.shist[((size_t)row * G + g) * kSB + r];
                     if (w) {
                         const uint32_t rr = (t.m4[g] + r - m4) & 511u;
-                        if (rr < (uint32_t)kSB) {
+                        if (rr < (uint32_t)kSB)
                             atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[kBin0 + rr]), 0ull - (unsigned long long)w);
-                            atomicAdd(reinterpret_cast<unsigned long long *>(&s.g[kBin0]), (unsigned long long)pack_count(w) << 43);
-                        }
                     }
                 }
             }
@@ -1659,11 +1629,9 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
     bool bad = total > v.list_cap;
     if ((uint32_t)tid < G) {
         const int lb = (int)(f.bin - kBin0) + 4 * (int)dl;            // boundary bin in the slice's frame
-        if (dl >= 64u) mtake = 0;                                      // the whole slice is clamped; the boundary bin
-                                                                       // can then only be bin 348, handled below
+        if (dl >= 64u) mtake = 0;                                      // the whole slice is dead in the row's frame
         else if (lb < kSB) mtake = v.cum[((size_t)row * G + tid) * kSB + lb];
-        if (f.bin == kBin0) bad = true;                                // clamped tokens of other frames are not in a stash
-        else if (mtake && ((int)ph.cov > lb || mtake > ph.n)) bad = true;
+        if (mtake && ((int)ph.cov > lb || mtake > ph.n)) bad = true;
     }
     if (bad) t.fail = 1;
     auto take_prefix = [&](uint32_t mine) {                           // inclusive prefix over the slices, into t.take
@@ -1684,11 +1652,8 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         // cutrow = the largest of the slices' cuts, so a threshold found among those is the row's.
         uint32_t mycut = 0;
         if ((uint32_t)tid < G) {
-            mycut = rebase_bits(ph.cut, dl);
-            // A cut above 2^-40 that lands on 2^-40 in the row's frame: the slice's tokens below
-            // its cut land there too and are not in its stash, so the stash is complete only
-            // above that value.  (A cut at 2^-40 in the slice's own frame took the whole slice.)
-            if (ph.cut != kEMinBits && mycut == kEMinBits) mycut = kEMinBits + 1u;
+            // a cut that lands below 2^-40 in the row's frame: what the stash lacks is dead there
+            mycut = max(rebase_bits(ph.cut, dl), kEMinBits);
         }
         cutrow = block_max_u32(s, mycut, lane, wave);
         take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);

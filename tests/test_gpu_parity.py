@@ -161,6 +161,39 @@ def test_degenerate_rows(torch_cuda, oracle):
     _run_case(torch_cuda, oracle, capi, big, 4.0, 10, 0.9, u_np=H.uniforms(6, 18), what="degenerate T=4")
 
 
+def test_masked_tokens_are_never_returned(torch_cuda, oracle):
+    """Logits at -inf (or merely 41 octaves and more below the maximum) are dead: probability 0,
+    as exp2f underflows in the reference (sampling.cu:235).  With nothing trimming the tail
+    (top_k = -1, top_p = 1) and the uniform at its upper end they must still never come back."""
+    from tests import capi
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    for V in (1 << 16, 1 << 18):
+        B = 6
+        lg = np.full((B, V), -np.inf, dtype=np.float32)
+        live = []
+        for b in range(B):
+            n_live = [4, 4, 100, V // 2, 1, 4][b]
+            ids = np.sort(rng.choice(V, size=n_live, replace=False))
+            lg[b, ids] = rng.standard_normal(n_live).astype(np.float32) * 2
+            if b == 1:
+                lg[b, lg[b] == -np.inf] = -200.0                     # finite, but far below 2^-40 of the maximum
+            if b == 5:
+                lg[b, ids[-1] + 1:] = np.nan                         # cleaned to 0 by sf: live
+                ids = np.concatenate([ids, np.arange(ids[-1] + 1, V)])
+            live.append(set(ids.tolist()))
+        for top_k, top_p in [(-1, 1.0), (1000, 1.0), (-1, 0.999999)]:
+            for u in (1.0, float(np.nextafter(np.float32(1.0), np.float32(0.0))), 0.9999999):
+                u_np = np.full(B, u, dtype=np.float32)
+                res, ref = _run_case(torch, oracle, capi, lg, 1.0, top_k, top_p, u_np=u_np,
+                                     what="masked V=%d k=%d p=%g u=%r" % (V, top_k, top_p, u))
+                for b in range(B):
+                    assert int(res["out"][b]) in live[b], (b, int(res["out"][b]))
+                    assert res["diag"]["thr_bits"][b] >= 0x2B800000
+                    dead = res["e_bits"][b] == 0
+                    assert dead.sum() == V - len(live[b])
+
+
 def test_uniform_extremes(torch_cuda, oracle):
     """u -> 0+ picks the first kept token, u = 1 the last one."""
     from tests import capi

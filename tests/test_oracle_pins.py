@@ -60,13 +60,16 @@ def test_e_bits_accuracy_monotone_and_anchors(oracle):
         live = ref >= 2.0 ** -40
         rel = np.abs(e[live] - ref[live]) / ref[live]
         assert rel.max() < 2.0 * 2.0 ** -23, rel.max()     # within 2 ulp, as the reference's exp2f
-        assert np.all(e[~live] == 2.0 ** -40)              # clamped from below
+        assert np.all(b[~live] == 0)                       # flushed to zero below 2^-40: dead tokens
         assert np.all(np.diff(b.astype(np.int64)) >= 0)    # monotone in x
         assert b.max() < 0x40000000                        # e < 2
+        assert b[live].min() >= 0x2B800000                 # nothing between 0 and 2^-40
     assert oracle.e_bits(F32([5.0]), 5.0)[0] == bits(F32(1.0))[()]
     for k in range(0, 41):
         assert oracle.e_bits(F32([-k]), 0.0)[0] == bits(F32(2.0 ** -k))[()]     # exact powers of two
-    assert oracle.e_bits(F32([-40.5, -1e30, -3.4e38]), 0.0).tolist() == [0x2B800000] * 3
+    assert oracle.e_bits(F32([-40.5, -1e30, -3.4e38]), 0.0).tolist() == [0] * 3
+    just_below = np.nextafter(F32(-40.0), F32(-np.inf))
+    assert oracle.e_bits(np.array([just_below, -40.0], dtype=np.float32), 0.0).tolist() == [0, 0x2B800000]
 
 
 def test_e_significand_does_not_depend_on_the_maximum(oracle):
@@ -77,10 +80,9 @@ def test_e_significand_does_not_depend_on_the_maximum(oracle):
     b0 = oracle.e_bits(x, 20.0)
     for d in (1, 2, 7, 19):
         b1 = oracle.e_bits(x, 20.0 + d)
-        rebased = np.maximum(b0.astype(np.int64) - (d << 23), 0x2B800000)
-        keep = (b0 > 0x2B800000)
-        assert np.array_equal(b1[keep].astype(np.int64), rebased[keep])
-        assert np.all(b1[~keep] == 0x2B800000)
+        rebased = b0.astype(np.int64) - (d << 23)
+        rebased[rebased < 0x2B800000] = 0                  # what falls below 2^-40 of the new frame is dead
+        assert np.array_equal(b1.astype(np.int64), rebased)
 
 
 def test_e_monotone_across_every_octave_boundary(oracle):
@@ -103,7 +105,8 @@ def test_w_is_e_times_2_pow_63(oracle):
     for bi, wi in zip(b, w):
         exact = Fraction(float(np.uint32(bi).view(np.float32))) * 2 ** 63
         assert exact.denominator == 1 and int(wi) == exact.numerator == oracle.lib().rs_oracle_w(int(bi))
-    assert int(w.min()) == 2 ** 23 and int(w.max()) < 2 ** 64
+    assert int(w[b > 0].min()) == 2 ** 23 and int(w.max()) < 2 ** 64
+    assert (b == 0).any() and np.all(w[b == 0] == 0)       # dead tokens weigh nothing
 
 
 @settings(max_examples=300, deadline=None)
@@ -183,7 +186,7 @@ def brute_force_row(logits, c, top_k, top_p, u=None, u64=None, pen=None):
     w = [v.numerator for v in w]
     D = sum(w)
     P = min(max(math.ceil(Fraction(float(F32(top_p))) * D), 1), D)
-    order = sorted(set(int(b) for b in eb), reverse=True)
+    order = sorted(set(int(b) for b in eb if b > 0), reverse=True)     # dead tokens take no part
     cnt = mass = 0
     thr = order[-1]
     for val in order:
@@ -267,8 +270,39 @@ def test_keep_everything(oracle):
     lg = H.logits_normal(1, 8192, 2.0, 9)[0]
     c, kk, pp = oracle.normalize(1.0, -1, 1.0, 8192)
     d = oracle.sample_row(lg, c, kk, pp, u=1.0, want_e=True)
+    assert d["e_bits"].min() > 0                            # every token of this row is live
     assert d["thr_bits"] == d["e_bits"].min() and d["n_gt"] + d["n_eq"] == 8192 and d["rounds"] == 0
     assert d["S"] <= d["D"] and d["index"] == int(np.nonzero(d["e_bits"] >= d["thr_bits"])[0][-1])
+
+
+def test_masked_tokens_are_never_returned(oracle):
+    """A logit at -inf (cleaned to -FLT_MAX, sampling.cu:131-134) has exp2f(x - max) = 0 in the
+    reference (sampling.cu:235,248): threshold * comp cannot give it weight, so it never comes back,
+    whatever top_k and top_p are.  Here e is flushed to zero below 2^-40 of the maximum."""
+    V = 1 << 16
+    rng = np.random.default_rng(21)
+    live_ids = np.sort(rng.choice(V, size=4, replace=False))
+    for low in (-np.inf, -200.0, -41.0 / 1.4426950408889634 - 1.0):
+        lg = np.full(V, low, dtype=np.float32)
+        lg[live_ids] = rng.standard_normal(4).astype(np.float32)
+        for k, p in [(-1, 1.0), (1000, 1.0), (-1, 0.999999), (5, 1.0)]:
+            c, kk, pp = oracle.normalize(1.0, k, p, V)
+            for u in (1.0, float(np.nextafter(F32(1.0), F32(0.0))), 0.9999999, 0.5, 1e-30):
+                d = oracle.sample_row(lg, c, kk, pp, u=u, want_e=True)
+                assert d["index"] in live_ids, (low, k, p, u, d["index"])
+                assert d["thr_bits"] >= 0x2B800000 and d["n_gt"] + d["n_eq"] <= 4
+                assert np.count_nonzero(d["e_bits"]) == 4 and d["S"] <= d["D"]
+            # 64 random bits at their largest reach the last live token, not the tail of the row
+            d = oracle.sample_row(lg, c, kk, pp, u64=2 ** 64 - 1)
+            assert d["index"] in live_ids
+            if k == -1 and p == 1.0:
+                assert d["index"] == live_ids[-1]
+    # fewer live tokens than top_k: the kept set is every live token
+    lg = np.full(V, -np.inf, dtype=np.float32)
+    lg[live_ids] = [0.0, 1.0, 2.0, 3.0]
+    c, kk, pp = oracle.normalize(1.0, 50, 1.0, V)
+    d = oracle.sample_row(lg, c, kk, pp, u=1.0)
+    assert d["n_gt"] + d["n_eq"] == 4 and d["S"] == d["D"] and d["index"] == live_ids[-1]
 
 
 def test_all_equal_logits_are_uniform_over_all_tokens(oracle):
