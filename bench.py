@@ -224,11 +224,11 @@ def main():
         t_btv = block_time_us(torch, call_btv, args.bandwidth_steps, 3)
         t_flat = block_time_us(torch, call_flat, max(2, args.bandwidth_steps // 2), 2)
         t_floor = block_time_us(torch, floor_btv, args.bandwidth_steps, 3)
-        os.environ["RS_FORCE_PATH"] = "cluster"          # the general single-launch kernel on the same input
+        sample._sample.force_path("cluster")             # the general single-launch kernel on the same input
         try:
             t_cluster = block_time_us(torch, call_btv, max(2, args.bandwidth_steps // 2), 2)
         finally:
-            del os.environ["RS_FORCE_PATH"]
+            sample._sample.force_path("auto")
         bytes_btv = Bb * Vb * 4
         bytes_flat = Bb * Tb * Vb * 4
         ach = bytes_btv / (t_btv * 1e-6) / 1e9

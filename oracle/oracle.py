@@ -107,6 +107,8 @@ def lib():
         L.rs_oracle_batch.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_int32, C.c_int32, C.c_float, C.c_int32, C.c_float,
                                       C.c_float, C.c_float, C.c_float, C.c_void_p]
+        L.rs_oracle_batch_e.restype = None
+        L.rs_oracle_batch_e.argtypes = L.rs_oracle_batch.argtypes + [C.c_void_p]
         L.ref_literal_row.restype = None
         L.ref_literal_row.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_float,
                                       C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
@@ -199,11 +201,12 @@ def sample_row(logits, c, top_k, top_p, u=None, u64=0, penalties=None,
 
 
 def sample_batch(logits, c, top_k, top_p, rng=None, injected_u=None, penalties=None,
-                 presence=0.0, repetition=0.0, decay=1.0):
+                 presence=0.0, repetition=0.0, decay=1.0, want_e=False):
     """A batch through the canonical oracle.
 
     logits: (V,), (B, V) or (B, T, V) float32; for (B, T, V) only logits[:, T-1, :] is read
-    (sampling.cu:176,202).  Returns (out int32 (B,), diag structured array (B,)).
+    (sampling.cu:176,202).  Returns (out int32 (B,), diag structured array (B,)), and with want_e
+    also the bit patterns of e of every token, uint32 (B, V).
     """
     logits = np.ascontiguousarray(logits, dtype=np.float32)
     if logits.ndim == 1:
@@ -224,10 +227,11 @@ def sample_batch(logits, c, top_k, top_p, rng=None, injected_u=None, penalties=N
         assert rng is not None and rng.dtype == np.uint32 and rng.shape == (B, 16)
     if penalties is not None:
         assert penalties.dtype == np.float32 and penalties.flags.c_contiguous and penalties.shape == (B, V)
-    lib().rs_oracle_batch(C.c_void_p(base), row_stride, _ptr(penalties), _ptr(out), _ptr(rng),
-                          _ptr(injected_u), B, V, c, top_k, top_p, presence, repetition, decay,
-                          _ptr(diag))
-    return out, diag
+    e = np.empty((B, V), dtype=np.uint32) if want_e else None
+    lib().rs_oracle_batch_e(C.c_void_p(base), row_stride, _ptr(penalties), _ptr(out), _ptr(rng),
+                            _ptr(injected_u), B, V, c, top_k, top_p, presence, repetition, decay,
+                            _ptr(diag), _ptr(e))
+    return (out, diag, e) if want_e else (out, diag)
 
 
 def thr_by_sort(e_bits, top_k, P):

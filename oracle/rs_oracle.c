@@ -344,6 +344,16 @@ void rs_oracle_batch(const float *logits, int64_t row_stride, float *penalties,
                      float presence, float repetition, float decay,
                      rs_oracle_diag *diag)
 {
+    rs_oracle_batch_e(logits, row_stride, penalties, out, rng, injected_u, B, V, c, top_k, top_p,
+                      presence, repetition, decay, diag, NULL);
+}
+
+void rs_oracle_batch_e(const float *logits, int64_t row_stride, float *penalties,
+                       int32_t *out, uint32_t *rng, const float *injected_u,
+                       int32_t B, int32_t V, float c, int32_t top_k, float top_p,
+                       float presence, float repetition, float decay,
+                       rs_oracle_diag *diag, uint32_t *e_bits_out)
+{
     for (int32_t b = 0; b < B; b++) {
         rs_oracle_diag dg;
         uint64_t u64 = 0;
@@ -359,7 +369,7 @@ void rs_oracle_batch(const float *logits, int64_t row_stride, float *penalties,
         rs_oracle_row(logits + (int64_t)b * row_stride,
                       penalties ? penalties + (int64_t)b * V : NULL, V, c, top_k, top_p,
                       injected_u != NULL, injected_u ? injected_u[b] : 0.0f, u64,
-                      presence, repetition, decay, NULL, &dg);
+                      presence, repetition, decay, e_bits_out ? e_bits_out + (size_t)b * V : NULL, &dg);
         out[b] = dg.index;
         if (diag) diag[b] = dg;
     }

@@ -102,6 +102,13 @@ void rs_oracle_batch(const float *logits, int64_t row_stride, float *penalties,
                      float presence, float repetition, float decay,
                      rs_oracle_diag *diag /* B entries or NULL */);
 
+/* the same, also returning the bit patterns of e of every token: e_bits_out (B,V) or NULL */
+void rs_oracle_batch_e(const float *logits, int64_t row_stride, float *penalties,
+                       int32_t *out, uint32_t *rng, const float *injected_u,
+                       int32_t B, int32_t V, float c, int32_t top_k, float top_p,
+                       float presence, float repetition, float decay,
+                       rs_oracle_diag *diag, uint32_t *e_bits_out);
+
 void rs_oracle_rng_init(uint32_t *rng, uint64_t seed, int32_t B);
 
 /* ---- literal fp32 emulation of the reference kernel -------------------- */

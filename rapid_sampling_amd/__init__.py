@@ -11,9 +11,14 @@ Drop-in for the Python API of the reference module (`sample` in
                   logits, penalties, states, presence_penalty, repetition_penalty,
                   penalty_decay, temperature, top_k, top_p)
 
-Beyond the reference: keyword names, `uniforms=` (injected draws, for tests) and
+Beyond the reference: keyword names, `uniforms=` (injected draws, for tests),
 `accept_half=True` (bfloat16 / float16 logits read as they are; by default any
-type but float32 raises the reference's error).
+type but float32 raises the reference's error), `reserve_workspace(B, V)`
+(allocates the current stream's workspace ahead of time: required before the
+calls are captured into a HIP graph), `workspace_status()` (synchronises and
+returns the error word of the current stream's workspace) and `set_wait_limit`.
+A call whose kernel gave up waiting for its peers raises RuntimeError on the
+next call on that stream at the latest.
 
 The functions live in the compiled extension `_sample` (host layer in
 csrc/sampling.cpp, kernels in csrc/rs_kernels.hip behind the C ABI of
@@ -39,6 +44,9 @@ batch_sampling_temperature_topk_topp = _sample.batch_sampling_temperature_topk_t
 batch_sampling_repetition_temperature_topk_topp = _sample.batch_sampling_repetition_temperature_topk_topp
 batch_sampling_debug = _sample.batch_sampling_debug
 floor_read = _sample.floor_read
+reserve_workspace = _sample.reserve_workspace
+workspace_status = _sample.workspace_status
+set_wait_limit = _sample.set_wait_limit
 STATE_BYTES_PER_ROW = _sample.STATE_BYTES_PER_ROW
 DIAG_BYTES = _sample.DIAG_BYTES
 
@@ -50,6 +58,9 @@ __all__ = [
     "batch_sampling_repetition_temperature_topk_topp",
     "batch_sampling_debug",
     "floor_read",
+    "reserve_workspace",
+    "workspace_status",
+    "set_wait_limit",
     "STATE_BYTES_PER_ROW",
     "DIAG_BYTES",
     "KERNEL_LIBRARY",

@@ -1315,6 +1315,13 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : 3)) stream_kernel(const Para
             eb[j * 4] = 0; eb[j * 4 + 1] = 0; eb[j * 4 + 2] = 0; eb[j * 4 + 3] = 0;
         }
     }
+    if (p.e_bits) {
+        // diagnostics: e of every token, still in the slice's frame; the finishing workgroup re-bases it
+        uint4 *dst = reinterpret_cast<uint4 *>(p.e_bits + (int64_t)row * p.V);
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+            if (j < nv) dst[base4 + j * NT] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
+    }
     __syncthreads();
     // Add the slice's live bins to the row's, which are kept by absolute octave (mod 128, 4 bins each):
     // bin t of this frame is octave M - 40 + t/4.  Slices of one row may use different frames; as
@@ -1590,6 +1597,17 @@ __device__ __forceinline__ void finish_row(const Params &p, const StreamView &v,
         }
     }
     __syncthreads();
+    if (p.e_bits) {
+        // diagnostics: the slices' e into the row's frame, dead tokens as 0
+        uint4 *eb4 = reinterpret_cast<uint4 *>(p.e_bits + (int64_t)row * p.V);
+        auto fix = [&](uint32_t b, uint32_t d) { b = rebase_bits(min(b, 0x3FFFFFFFu), d); return b < kEMinBits ? 0u : b; };
+        for (uint32_t i4 = (uint32_t)tid; i4 < ((uint32_t)p.V >> 2); i4 += kThreads) {
+            const uint32_t d = t.delta[i4 >> (SLICE_LOG2 - 2)];
+            uint4 q = eb4[i4];
+            q.x = fix(q.x, d); q.y = fix(q.y, d); q.z = fix(q.z, d); q.w = fix(q.w, d);
+            eb4[i4] = q;
+        }
+    }
     if (drawer) {
         uint32_t o[4];
         philox4x32_10(rs[2], rs[3], rs[4], rs[5], rs[0], rs[1], o);
@@ -1888,6 +1906,16 @@ __global__ void philox_init_kernel(uint32_t *state, uint64_t seed, int32_t B)
     s[4] = (uint32_t)b;
 }
 
+// Clears device memory with plain stores (a recorded memset node misbehaves on graph replays).
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint4 *dst, size_t n16, unsigned char *tail, uint32_t ntail)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = make_uint4(0u, 0u, 0u, 0u);
+    if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+__global__ void set_u32_kernel(uint32_t *dst, uint32_t value) { *dst = value; }
+
 // ------------------------------------------------------------ host side ----
 
 struct Geometry { int R; uint32_t G; };
@@ -1895,14 +1923,13 @@ struct Geometry { int R; uint32_t G; };
 // Tokens per thread (4R) and workgroups per row.  Large batches take long
 // slices (few peers to meet, deep loads); a lone row is cut into a few dozen
 // slices so that many CUs pull it from HBM at once.
-static Geometry choose_geometry(int32_t B, int32_t V, bool pen)
+static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
 {
     const uint32_t V4 = (uint32_t)V / 4;
     const int maxR = pen ? 16 : 32;
-    const char *force = getenv("RS_FORCE_R");
     auto parts = [&](int R) { return (V4 + (uint32_t)(kThreads * R) - 1) / (uint32_t)(kThreads * R); };
-    if (force) {
-        int R = atoi(force);
+    if (force_r) {
+        const int R = force_r;
         if ((R == 1 || R == 2 || R == 4 || R == 8 || R == 16 || R == 32) && R <= maxR && parts(R) <= (uint32_t)kMaxParts)
             return {R, parts(R)};
     }
@@ -1957,58 +1984,48 @@ static size_t stream_bytes(int32_t B, int32_t V)
     return longs > shorts ? longs : shorts;
 }
 
-// The streaming path works when the kept set is small next to the row and the slices of a row
-// share a frame; a row for which it does not is handed to the cluster kernel in a third launch,
-// and a call whose rows mostly end that way has wasted a pass.  With a bounding top_k that takes
-// unusual rows (ties of thousands of tokens, slices more than 87 octaves apart); without one
-// (nucleus sampling alone) it is simply a flat distribution, so such a call is an attempt.  The
-// launch for the rows handed on reports "most of them: yes/no" into a word of pinned host memory
-// that belongs to the workspace, one word for calls with a bounding top_k and one for calls
-// without, and rs_sample looks at the word -- without waiting for anything; a stale value only
-// delays the switch -- before it chooses the path of the next call: after a call that handed
-// most rows on, calls of that kind go straight to the cluster kernel and one in 64 streams again.
-// Workspaces never given to rs_workspace_init have no such words: with a bounding top_k they
-// always stream, without one they never do.
-struct Hint { int32_t *word; uint32_t calls[2]; };
-static std::mutex g_hint_mu;
-static std::unordered_map<const void *, Hint> g_hints;
+}  // namespace rs
 
-static Hint *hint_of(const void *ws, bool create)
-{
-    std::lock_guard<std::mutex> lock(g_hint_mu);
-    auto it = g_hints.find(ws);
-    if (it != g_hints.end()) return &it->second;
-    if (!create) return nullptr;
-    int32_t *word = nullptr;
-    if (hipHostMalloc((void **)&word, 64, hipHostMallocDefault) != hipSuccess || !word) return nullptr;
-    word[0] = 0; word[1] = 0;
-    Hint h;
-    h.word = word; h.calls[0] = 0; h.calls[1] = 0;
-    return &g_hints.emplace(ws, h).first->second;
-}
+// The caller's routing state (see rapid_sampling.h).  word[0], word[1]: "most rows were handed on"
+// as last reported by a streaming call with / without a bounding top_k; word[2]: RS_ERR_DEVICE
+// once a kernel gave up a wait.  calls[]: calls routed away from the streaming path since.
+struct rs_policy {
+    int32_t *word;
+    uint32_t calls[2];
+};
 
+namespace rs {
+
+// The streaming path works when the kept set is small next to the row; a row for which it does
+// not is handed to the cluster kernel in a third launch, and a call whose rows mostly end that way
+// has wasted a pass.  With a bounding top_k that takes unusual rows (ties of thousands of tokens);
+// without one (nucleus sampling alone) it is simply a flat distribution, so such a call is an
+// attempt.  The launch for the rows handed on reports "most of them: yes/no" into a word of the
+// caller's rs_policy, one word for calls with a bounding top_k and one for calls without, and
+// this function looks at the word -- without waiting for anything; a stale value only delays the
+// switch -- before it chooses the path of the next call: after a call that handed most rows on,
+// calls of that kind go straight to the cluster kernel and one in 64 streams again.  Without a
+// policy, calls with a bounding top_k always stream and calls without never do.
+//
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
-// RS_FORCE_PATH=cluster|stream|optimistic overrides (tests).
 enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2 };
-static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pen, bool want_e, const void *ws, hipStream_t st)
+static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pen, const rs_options *opt)
 {
-    if (pen || want_e) return kPathCluster;
+    if (pen) return kPathCluster;
     const bool bounded = top_k <= kStreamK;
-    const char *force = getenv("RS_FORCE_PATH");
-    if (force && force[0] == 'c') return kPathCluster;
-    if (force && force[0] == 's') return bounded ? kPathStream : kPathCluster;
-    if (force && force[0] == 'o') return bounded ? kPathStream : kPathAttempt;
+    const int force = opt ? opt->path : RS_PATH_AUTO;
+    if (force == RS_PATH_CLUSTER) return kPathCluster;
+    if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
+    if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
     if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
     if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // everything is kept: nothing a stash could hold
+    rs_policy *pol = opt ? opt->policy : nullptr;
+    if (!pol) return bounded ? kPathStream : kPathCluster;
     const int yes = bounded ? kPathStream : kPathAttempt, kind = bounded ? 0 : 1;
-    Hint *h = hint_of(ws, false);
-    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (!h || hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone)
-        return bounded ? kPathStream : kPathCluster;            // a captured choice could not follow the reports
-    const bool failing = *(volatile int32_t *)(h->word + kind) != 0;
-    return (!failing || (++h->calls[kind] & 63u) == 0u) ? yes : kPathCluster;
+    const bool failing = *(volatile int32_t *)(pol->word + kind) != 0;
+    return (!failing || (++pol->calls[kind] & 63u) == 0u) ? yes : kPathCluster;
 }
 
 template <bool PEN>
@@ -2051,13 +2068,22 @@ static hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p,
     return hipGetLastError();
 }
 
+static hipError_t fill_zero(void *dst, size_t bytes, hipStream_t st)
+{
+    const size_t n16 = bytes / 16;
+    const uint32_t blocks = (uint32_t)(n16 / 256 < 1 ? 1 : n16 / 256 > 2048 ? 2048 : n16 / 256);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, st, (uint4 *)dst, n16,
+                       (unsigned char *)dst + n16 * 16, (uint32_t)(bytes - n16 * 16));
+    return hipGetLastError();
+}
+
 }  // namespace rs
 
 using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 300; }
+int rs_version(void) { return 400; }
 
 const char *rs_error_string(int code)
 {
@@ -2106,27 +2132,17 @@ int rs_workspace_init(void *ws, size_t bytes, void *stream)
 {
     if (!ws) return RS_ERR_NULL;
     if (bytes < sizeof(WsHeader) || ((uintptr_t)ws & 255)) return RS_ERR_WORKSPACE;
-    if (hipMemsetAsync(ws, 0, bytes, (hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
-    // the word of pinned host memory attempts are reported to (see choose_path)
-    if (Hint *hint = hint_of(ws, true)) {
-        hint->word[0] = 0; hint->word[1] = 0;
-        hint->calls[0] = 0; hint->calls[1] = 0;
-        WsHeader *h = (WsHeader *)ws;
-        if (hipMemcpyAsync(&h->hint, &hint->word, sizeof hint->word, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess)
-            return RS_ERR_LAUNCH;
-    }
-    // test hook: RS_SPIN_LIMIT_MS shortens the bound of the waits (default 2000 ms)
-    if (const char *ms = getenv("RS_SPIN_LIMIT_MS")) {
-        const long v = atol(ms);
-        if (v > 0 && v < 40000) {
-            const uint32_t ticks = (uint32_t)((uint64_t)v * 100000ull >> 10);      // 100 MHz wall clock
-            WsHeader *h = (WsHeader *)ws;
-            if (hipMemcpyAsync(&h->spin_ticks, &ticks, sizeof ticks, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess)
-                return RS_ERR_LAUNCH;
-            if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;   // `ticks` is on the stack
-        }
-    }
-    return RS_OK;
+    return fill_zero(ws, bytes, (hipStream_t)stream) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+int rs_workspace_set_wait_limit(void *ws, uint32_t milliseconds, void *stream)
+{
+    if (!ws) return RS_ERR_NULL;
+    if ((uintptr_t)ws & 255) return RS_ERR_WORKSPACE;
+    if (milliseconds >= 40000u) return RS_ERR_ARG;
+    const uint32_t ticks = (uint32_t)((uint64_t)milliseconds * 100000ull >> 10);      // 100 MHz wall clock
+    hipLaunchKernelGGL(set_u32_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, &((WsHeader *)ws)->spin_ticks, ticks);
+    return hipGetLastError() == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
 }
 
 int rs_workspace_status(const void *ws, int32_t *status, void *stream)
@@ -2140,11 +2156,43 @@ int rs_workspace_status(const void *ws, int32_t *status, void *stream)
     return RS_OK;
 }
 
-int rs_workspace_policy(const void *ws, int32_t *state)
+int rs_policy_create(rs_policy **out)
 {
-    if (!ws || !state) return RS_ERR_NULL;
-    const Hint *h = hint_of(ws, false);
-    *state = h ? (((volatile int32_t *)h->word)[1] != 0 ? 1 : 0) | (((volatile int32_t *)h->word)[0] != 0 ? 2 : 0) : -1;
+    if (!out) return RS_ERR_NULL;
+    *out = nullptr;
+    rs_policy *pol = new (std::nothrow) rs_policy;
+    if (!pol) return RS_ERR_LAUNCH;
+    pol->word = nullptr; pol->calls[0] = 0; pol->calls[1] = 0;
+    if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
+        delete pol;
+        return RS_ERR_LAUNCH;
+    }
+    for (int i = 0; i < 16; ++i) pol->word[i] = 0;
+    *out = pol;
+    return RS_OK;
+}
+
+void rs_policy_destroy(rs_policy *pol)
+{
+    if (!pol) return;
+    if (pol->word) (void)hipHostFree(pol->word);
+    delete pol;
+}
+
+int rs_policy_state(const rs_policy *pol, int32_t *state)
+{
+    if (!pol || !state) return RS_ERR_NULL;
+    const volatile int32_t *w = pol->word;
+    *state = (w[1] != 0 ? 1 : 0) | (w[0] != 0 ? 2 : 0);
+    return RS_OK;
+}
+
+int rs_policy_error(rs_policy *pol, int32_t *error, int32_t clear)
+{
+    if (!pol || !error) return RS_ERR_NULL;
+    volatile int32_t *w = pol->word;
+    *error = w[2];
+    if (clear) w[2] = 0;
     return RS_OK;
 }
 
@@ -2164,9 +2212,9 @@ int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t
               void *workspace, size_t workspace_bytes,
               rs_row_diag *diag, uint32_t *e_bits, void *stream)
 {
-    return rs_sample_dtype(logits, RS_DTYPE_F32, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
-                           repetition, decay, log2e_inv_temp, top_k, top_p, workspace, workspace_bytes, diag, e_bits,
-                           stream);
+    return rs_sample_ex(logits, RS_DTYPE_F32, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                        repetition, decay, log2e_inv_temp, top_k, top_p, workspace, workspace_bytes, diag, e_bits,
+                        nullptr, stream);
 }
 
 int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
@@ -2176,11 +2224,24 @@ int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride
                     void *workspace, size_t workspace_bytes,
                     rs_row_diag *diag, uint32_t *e_bits, void *stream)
 {
+    return rs_sample_ex(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                        repetition, decay, log2e_inv_temp, top_k, top_p, workspace, workspace_bytes, diag, e_bits,
+                        nullptr, stream);
+}
+
+int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                 void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                 float presence, float repetition, float decay,
+                 float log2e_inv_temp, int32_t top_k, float top_p,
+                 void *workspace, size_t workspace_bytes,
+                 rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
+{
     if (!logits || !out || !workspace || (!rng_state && !injected_u)) return RS_ERR_NULL;
     if (logits_dtype != RS_DTYPE_F32 && logits_dtype != RS_DTYPE_BF16 && logits_dtype != RS_DTYPE_F16) return RS_ERR_ARG;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
     if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
+    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_ATTEMPT || opt->slice_r < 0)) return RS_ERR_ARG;
     if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
         return RS_ERR_ALIGN;
     size_t need = 0;
@@ -2188,7 +2249,7 @@ int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride
     if (workspace_bytes < need || ((uintptr_t)workspace & 255)) return RS_ERR_WORKSPACE;
 
     const bool pen = penalties != nullptr;
-    const Geometry g = choose_geometry(B, V, pen);
+    const Geometry g = choose_geometry(B, V, pen, opt ? opt->slice_r : 0);
     Params p;
     p.logits = logits; p.dtype = logits_dtype; p.penalties = penalties; p.out = out;
     p.rng = (uint32_t *)rng_state; p.inj_u = injected_u; p.diag = diag; p.e_bits = e_bits;
@@ -2198,8 +2259,9 @@ int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
     p.need = nullptr; p.stash_k = (uint32_t)top_k; p.report = 0;
+    p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
     dim3 grid((uint32_t)B * g.G);
-    const int path = choose_path(B, V, top_k, top_p, pen, e_bits != nullptr, workspace, (hipStream_t)stream);
+    const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path != kPathCluster) {
         const int sr = stream_r(B, V);
         StreamView v;
@@ -2254,7 +2316,7 @@ int rs_floor_read(const float *logits, int64_t row_stride, int32_t *out, int32_t
     if (!logits || !out) return RS_ERR_NULL;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
-    const Geometry g = choose_geometry(B, V, false);
+    const Geometry g = choose_geometry(B, V, false, 0);
     const dim3 grid((uint32_t)B * g.G);
     hipStream_t st = (hipStream_t)stream;
     switch (g.R) {

@@ -11,6 +11,7 @@
 #include <hip/hip_runtime_api.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPFunctions.h>
 
 #include <map>
 #include <mutex>
@@ -24,6 +25,10 @@
 
 namespace {
 
+// Way through the library that every call of this module asks for (RS_PATH_*): a hook for
+// benchmarks and tests that compare the paths; results do not depend on it.
+int g_forced_path = RS_PATH_AUTO;
+
 void *current_stream(const at::Tensor &t)
 {
     return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
@@ -31,36 +36,85 @@ void *current_stream(const at::Tensor &t)
 
 // One zero-initialised workspace per (device, stream), sized for the largest B
 // and the largest V seen so far (the two maxima separately: that is what lets
-// calls of different shapes share it).  The kernels leave it clean, so it is
-// never cleared again; calls that share it are ordered by the stream.  Takes
-// the place of the reference's per-call `probs` scratch (sampling.cu:488,1014).
-at::Tensor &workspace_for(const at::Tensor &like, void *stream, int64_t B, int64_t V)
+// calls of different shapes share it), with the rs_policy object that routes
+// the streaming path and carries asynchronous error reports.  The kernels
+// leave the workspace clean, so it is never cleared again; calls that share
+// it are ordered by the stream.  Takes the place of the reference's per-call
+// `probs` scratch (sampling.cu:488,1014).
+struct Entry {
+    at::Tensor ws;
+    int64_t B = 0, V = 0;
+    rs_policy *policy = nullptr;
+    bool captured = false;                  // a stream capture has recorded calls that point into ws
+    std::vector<at::Tensor> retired;        // outgrown workspaces a captured graph may still point into
+};
+
+bool is_capturing(void *stream)
 {
-    // `retired` keeps outgrown workspaces alive: a captured HIP graph may still point into one
-    struct Entry { at::Tensor ws; int64_t B = 0, V = 0; std::vector<at::Tensor> retired; };
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
+}
+
+// Entries live until the process ends (never destroyed: tensors must not be released after the
+// runtime has shut down).  The last entry used by a thread is remembered, so that the steady state
+// takes no lock and no map lookup.
+Entry &entry_for(int device, void *stream)
+{
     static std::mutex mu;
-    static std::map<std::pair<int, void *>, Entry> cache;
+    static auto *cache = new std::map<std::pair<int, void *>, Entry *>();
+    thread_local int last_device = -1;
+    thread_local void *last_stream = nullptr;
+    thread_local Entry *last = nullptr;
+    if (last && last_device == device && last_stream == stream) return *last;
     std::lock_guard<std::mutex> lock(mu);
-    Entry &e = cache[{(int)like.device().index(), stream}];
+    Entry *&e = (*cache)[{device, stream}];
+    if (!e) e = new Entry();
+    last_device = device; last_stream = stream; last = e;
+    return *e;
+}
+
+void init_workspace(Entry &e, void *stream)
+{
+    const int rc = rs_workspace_init(e.ws.data_ptr(), (size_t)e.ws.numel(), stream);
+    if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
+}
+
+// Grows the entry's workspace to serve (B, V).  Under stream capture nothing may be allocated
+// (the allocation would belong to the graph's private pool and the fill would be replayed with
+// every launch of the graph): reserve_workspace(B, V) before capturing.
+Entry &workspace_for(const at::Tensor &like, void *stream, int64_t B, int64_t V)
+{
+    Entry &e = entry_for((int)like.device().index(), stream);
     if (!e.ws.defined() || B > e.B || V > e.V) {
+        if (is_capturing(stream))
+            throw std::runtime_error("rapid_sampling: the workspace of this stream must grow for B=" + std::to_string(B) +
+                                     ", V=" + std::to_string(V) + " while the stream is being captured; call "
+                                     "reserve_workspace(B, V) on this stream before the capture begins");
+        if (!e.policy && rs_policy_create(&e.policy) != RS_OK)
+            throw std::runtime_error("rapid_sampling: could not allocate the pinned host words of the workspace");
         e.B = std::max(e.B, B);
         e.V = std::max(e.V, V);
         size_t bytes = 0;
         rs_workspace_bytes((int32_t)e.B, (int32_t)e.V, &bytes);
-        if (e.ws.defined()) e.retired.push_back(e.ws);
-        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        const bool capturing = hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
-        if (capturing) {
-            // a memset must not be recorded into a graph: clear with a fill kernel, and do without
-            // the routing reports rs_workspace_init would set up
-            e.ws = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
-        } else {
-            e.ws = at::empty({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
-            const int rc = rs_workspace_init(e.ws.data_ptr(), bytes, stream);
-            if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
-        }
+        if (e.ws.defined() && e.captured) e.retired.push_back(e.ws);      // otherwise nothing points into it any more
+        e.captured = false;
+        e.ws = at::empty({(int64_t)bytes}, at::TensorOptions().dtype(at::kChar).device(like.device()));
+        init_workspace(e, stream);
     }
-    return e.ws;
+    return e;
+}
+
+// A kernel that gave up waiting for its peers (RS_ERR_DEVICE) leaves garbage in `out` and a dirty
+// workspace.  It says so in a pinned host word, which is looked at -- without synchronising --
+// before every call: the workspace is then set up again and the failure raised, one call late at
+// the latest (workspace_status() synchronises and tells at once).
+void raise_reported_failure(Entry &e, void *stream)
+{
+    int32_t err = RS_OK;
+    if (!e.policy || rs_policy_error(e.policy, &err, 1) != RS_OK || err == RS_OK) return;
+    if (!is_capturing(stream)) init_workspace(e, stream);
+    throw std::runtime_error(std::string("rapid_sampling: an earlier sampling call on this stream failed (") +
+                             rs_error_string(err) + "); its result was not valid. The workspace has been set up again.");
 }
 
 void throw_for(int code, int64_t B, int64_t T, int64_t V, double temperature)
@@ -168,9 +222,12 @@ at::Tensor run(const at::Tensor &logits, const Shape &s, at::Tensor *penalties, 
 
     c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
     void *stream = current_stream(logits);
-    size_t bytes = 0;
-    throw_for(rs_workspace_bytes((int32_t)s.B, (int32_t)s.V, &bytes), s.B, s.T, s.V, temperature);
-    at::Tensor &ws = workspace_for(logits, stream, s.B, s.V);
+    Entry &e = workspace_for(logits, stream, s.B, s.V);
+    raise_reported_failure(e, stream);
+    if (!e.captured && is_capturing(stream)) e.captured = true;
+    at::Tensor &ws = e.ws;
+    rs_options opt;
+    opt.path = g_forced_path; opt.slice_r = 0; opt.policy = e.policy;
     auto out = at::empty({s.B}, at::TensorOptions().dtype(at::kInt).device(logits.device()));
     rs_row_diag *diag = nullptr;
     uint32_t *ebits = nullptr;
@@ -180,10 +237,10 @@ at::Tensor run(const at::Tensor &logits, const Shape &s, at::Tensor *penalties, 
         diag = (rs_row_diag *)dbg->diag.data_ptr();
         ebits = (uint32_t *)dbg->e_bits.data_ptr();
     }
-    const int rc = rs_sample_dtype(s.first_row, s.dtype, s.row_stride, penalties ? penalties->data_ptr<float>() : nullptr,
-                                   out.data_ptr<int32_t>(), inj ? nullptr : states->data_ptr(), inj,
-                                   (int32_t)s.B, (int32_t)s.V, (float)presence, (float)repetition, (float)decay,
-                                   c, k, p, ws.data_ptr(), (size_t)ws.numel(), diag, ebits, stream);
+    const int rc = rs_sample_ex(s.first_row, s.dtype, s.row_stride, penalties ? penalties->data_ptr<float>() : nullptr,
+                                out.data_ptr<int32_t>(), inj ? nullptr : states->data_ptr(), inj,
+                                (int32_t)s.B, (int32_t)s.V, (float)presence, (float)repetition, (float)decay,
+                                c, k, p, ws.data_ptr(), (size_t)ws.numel(), diag, ebits, &opt, stream);
     throw_for(rc, s.B, s.T, s.V, temperature);
     return out;
 }
@@ -240,6 +297,74 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> batch_sampling_debug(
     return {out, dbg.diag, dbg.e_bits};
 }
 
+// Allocates and clears the workspace of the current stream of `device` for calls of up to B rows
+// of up to V tokens.  Needed before a stream capture (nothing may be allocated while capturing);
+// otherwise optional: the first call of a shape does the same.
+void reserve_workspace(int64_t B, int64_t V, std::optional<int64_t> device)
+{
+    size_t bytes = 0;
+    throw_for(rs_workspace_bytes((int32_t)B, (int32_t)V, &bytes), B, 1, V, 1.0);
+    const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+    auto like = at::empty({1}, at::TensorOptions().dtype(at::kChar).device(dev));
+    workspace_for(like, current_stream(like), B, V);
+}
+
+// Synchronises the current stream of `device` and returns the sticky error word of its workspace:
+// 0, or RS_ERR_DEVICE after a kernel gave up waiting (the workspace is then set up again, so the
+// next call starts clean).
+int64_t workspace_status(std::optional<int64_t> device)
+{
+    const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+    auto like = at::empty({1}, at::TensorOptions().dtype(at::kChar).device(dev));
+    void *stream = current_stream(like);
+    Entry &e = entry_for((int)dev.index(), stream);
+    if (!e.ws.defined()) return RS_OK;
+    int32_t st = RS_OK;
+    const int rc = rs_workspace_status(e.ws.data_ptr(), &st, stream);
+    if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
+    if (st != RS_OK) {
+        int32_t dummy;
+        if (e.policy) rs_policy_error(e.policy, &dummy, 1);
+        init_workspace(e, stream);
+    }
+    return st;
+}
+
+// Shortens (milliseconds > 0) or restores (0) the bound of the kernels' waits on the current
+// stream's workspace.  For tests of the error path.
+void set_wait_limit(int64_t milliseconds, std::optional<int64_t> device)
+{
+    const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+    auto like = at::empty({1}, at::TensorOptions().dtype(at::kChar).device(dev));
+    void *stream = current_stream(like);
+    Entry &e = entry_for((int)dev.index(), stream);
+    if (!e.ws.defined()) throw std::runtime_error("rapid_sampling: no workspace on this stream yet");
+    const int rc = rs_workspace_set_wait_limit(e.ws.data_ptr(), (uint32_t)milliseconds, stream);
+    if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
+}
+
+void force_path(const std::string &name)
+{
+    if (name == "auto") g_forced_path = RS_PATH_AUTO;
+    else if (name == "cluster") g_forced_path = RS_PATH_CLUSTER;
+    else if (name == "stream") g_forced_path = RS_PATH_STREAM;
+    else if (name == "attempt") g_forced_path = RS_PATH_ATTEMPT;
+    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt");
+}
+
+// The workspace tensor of the current stream (tests poison it to force the error path).
+at::Tensor debug_workspace(std::optional<int64_t> device)
+{
+    const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
+    auto like = at::empty({1}, at::TensorOptions().dtype(at::kChar).device(dev));
+    Entry &e = entry_for((int)dev.index(), current_stream(like));
+    if (!e.ws.defined()) throw std::runtime_error("rapid_sampling: no workspace on this stream yet");
+    return e.ws;
+}
+
 // Launch-plus-one-read floor kernel on the logits' grid (measurement aid).
 at::Tensor floor_read(at::Tensor &logits)
 {
@@ -269,6 +394,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           py::arg("temperature"), py::arg("top_k"), py::arg("top_p"), py::kw_only(),
           py::arg("uniforms") = py::none(), py::arg("accept_half") = false);
     m.def("floor_read", &floor_read, py::arg("logits"));
+    m.def("reserve_workspace", &reserve_workspace, py::arg("B"), py::arg("V"), py::arg("device") = py::none());
+    m.def("workspace_status", &workspace_status, py::arg("device") = py::none());
+    m.def("force_path", &force_path, py::arg("name"));
+    m.def("debug_workspace", &debug_workspace, py::arg("device") = py::none());
+    m.def("set_wait_limit", &set_wait_limit, py::arg("milliseconds"), py::arg("device") = py::none());
     m.attr("STATE_BYTES_PER_ROW") = RS_STATE_BYTES_PER_ROW;
     m.attr("DIAG_BYTES") = (int)sizeof(rs_row_diag);
 }

@@ -17,6 +17,14 @@ DIAG_DTYPE = np.dtype([
     ("S", "<u8", (2,)), ("r", "<u8", (2,)),
 ])
 
+PATHS = {None: 0, "auto": 0, "cluster": 1, "stream": 2, "optimistic": 3, "attempt": 3}
+
+
+class Options(C.Structure):
+    """rs_options of include/rapid_sampling.h"""
+    _fields_ = [("path", C.c_int32), ("slice_r", C.c_int32), ("policy", C.c_void_p)]
+
+
 _lib = None
 
 
@@ -35,8 +43,19 @@ def lib():
                                         C.POINTER(f32), C.POINTER(i32), C.POINTER(f32)]
         L.rs_workspace_bytes.restype = C.c_int
         L.rs_workspace_bytes.argtypes = [i32, i32, C.POINTER(sz)]
-        L.rs_workspace_policy.restype = C.c_int
-        L.rs_workspace_policy.argtypes = [vp, C.POINTER(C.c_int32)]
+        L.rs_workspace_set_wait_limit.restype = C.c_int
+        L.rs_workspace_set_wait_limit.argtypes = [vp, C.c_uint32, vp]
+        L.rs_policy_create.restype = C.c_int
+        L.rs_policy_create.argtypes = [C.POINTER(vp)]
+        L.rs_policy_destroy.restype = None
+        L.rs_policy_destroy.argtypes = [vp]
+        L.rs_policy_state.restype = C.c_int
+        L.rs_policy_state.argtypes = [vp, C.POINTER(i32)]
+        L.rs_policy_error.restype = C.c_int
+        L.rs_policy_error.argtypes = [vp, C.POINTER(i32), i32]
+        L.rs_sample_ex.restype = C.c_int
+        L.rs_sample_ex.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
+                                   vp, sz, vp, vp, C.POINTER(Options), vp]
         L.rs_workspace_init.restype = C.c_int
         L.rs_workspace_init.argtypes = [vp, sz, vp]
         L.rs_workspace_status.restype = C.c_int
@@ -71,13 +90,47 @@ class Sampler:
     """Holds a workspace on the current torch device and calls rs_sample on the
     current torch stream."""
 
-    def __init__(self, B, V):
+    def __init__(self, B, V, with_policy=False, init=False):
+        """with_policy: own an rs_policy (routing reports, asynchronous error word) and pass it with
+        every call.  init: clear the workspace with rs_workspace_init instead of torch.zeros."""
         import torch
         self.torch = torch
         rc, n = workspace_bytes(B, V)
         assert rc == 0
-        self.ws = torch.zeros(n, dtype=torch.int8, device="cuda")
+        if init:
+            self.ws = torch.empty(n, dtype=torch.int8, device="cuda")
+            assert lib().rs_workspace_init(self.ws.data_ptr(), n, self.stream()) == 0
+        else:
+            self.ws = torch.zeros(n, dtype=torch.int8, device="cuda")
         self.B, self.V = B, V
+        self.policy = None
+        if with_policy:
+            h = C.c_void_p()
+            assert lib().rs_policy_create(C.byref(h)) == 0 and h.value
+            self.policy = h
+
+    def close(self):
+        """Frees the policy; only after the device has finished every call that was given it."""
+        if self.policy is not None:
+            self.torch.cuda.synchronize()
+            lib().rs_policy_destroy(self.policy)
+            self.policy = None
+
+    def policy_state(self):
+        st = C.c_int32(-100)
+        assert lib().rs_policy_state(self.policy, C.byref(st)) == 0
+        return st.value
+
+    def policy_error(self, clear=False):
+        e = C.c_int32(-100)
+        assert lib().rs_policy_error(self.policy, C.byref(e), 1 if clear else 0) == 0
+        return e.value
+
+    def reinit(self):
+        assert lib().rs_workspace_init(self.ws.data_ptr(), self.ws.numel(), self.stream()) == 0
+
+    def set_wait_limit(self, ms):
+        assert lib().rs_workspace_set_wait_limit(self.ws.data_ptr(), ms, self.stream()) == 0
 
     def stream(self):
         return C.c_void_p(self.torch.cuda.current_stream().cuda_stream)
@@ -89,9 +142,11 @@ class Sampler:
         return st.value
 
     def sample(self, logits, c, top_k, top_p, *, rng=None, uniforms=None, penalties=None,
-               presence=0.0, repetition=0.0, decay=1.0, want_diag=True, want_e=False):
+               presence=0.0, repetition=0.0, decay=1.0, want_diag=True, want_e=False, path=None, force_r=None,
+               sync=True):
         """logits: (B,V) or (B,T,V) cuda tensor, float32 (rs_sample) or bfloat16 / float16
-        (rs_sample_dtype).  Returns dict of cpu numpy results."""
+        (rs_sample_dtype); with path / force_r / a policy the call goes through rs_sample_ex.
+        Returns dict of cpu numpy results."""
         torch = self.torch
         dtype = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[logits.dtype]
         if logits.dim() == 3:
@@ -113,12 +168,18 @@ class Sampler:
                 self.ws.data_ptr(), self.ws.numel(),
                 diag.data_ptr() if diag is not None else None,
                 eb.data_ptr() if eb is not None else None, self.stream())
-        if dtype == 0:
+        if path is not None or force_r is not None or self.policy is not None:
+            opt = Options(PATHS[path], force_r or 0, self.policy)
+            rc = lib().rs_sample_ex(ptr, dtype, stride, *tail[:-1], C.byref(opt), tail[-1])
+        elif dtype == 0:
             rc = lib().rs_sample(ptr, stride, *tail)
         else:
             rc = lib().rs_sample_dtype(ptr, dtype, stride, *tail)
         res = {"rc": rc}
         if rc != 0:
+            return res
+        if not sync:
+            res["out_dev"] = out
             return res
         torch.cuda.synchronize()
         res["out"] = out.cpu().numpy()

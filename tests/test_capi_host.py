@@ -201,3 +201,28 @@ def test_product_does_not_import_the_oracle():
                     assert not re.search(pat, text, flags=re.M), (os.path.join(dirpath, fn), pat)
     libs = os.popen("ldd %s 2>/dev/null" % capi.LIB_PATH).read()
     assert "rs_oracle" not in libs
+
+
+def test_library_reads_no_environment_and_takes_no_locks():
+    """The C ABI is stateless: what a call needs lives in its arguments, the workspace and the caller's
+    rs_policy.  The library imports neither getenv nor any mutex / once primitive."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--undefined-only", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    for sym in ("getenv", "pthread_mutex_lock", "pthread_once", "__cxa_guard_acquire"):
+        assert sym not in out, sym
+
+
+def test_options_and_policy_arguments_are_checked():
+    L = capi.lib()
+    assert L.rs_policy_state(None, C.byref(C.c_int32())) == -4
+    assert L.rs_policy_error(None, C.byref(C.c_int32()), 0) == -4
+    assert L.rs_policy_create(None) == -4
+    L.rs_policy_destroy(None)                              # a no-op
+    assert L.rs_workspace_set_wait_limit(None, 5, None) == -4
+    assert L.rs_workspace_set_wait_limit(C.c_void_p(256), 50000, None) == -7
+    # options out of range are refused before anything is launched (pointers are never dereferenced:
+    # the checks come first)
+    bad = capi.Options(9, 0, None)
+    args = [C.c_void_p(4096), 0, 1024, None, C.c_void_p(4096), C.c_void_p(4096), None, 1, 1024,
+            0.0, 0.0, 1.0, 1.0, 10, 0.5, C.c_void_p(4096), 1 << 30, None, None, C.byref(bad), None]
+    assert L.rs_sample_ex(*args) == -7

@@ -4,7 +4,7 @@ so every compared field must be EQUAL (sampled index, threshold, kept set as
 {e >= thr} from bit-identical e, counts, integer masses); updated penalties are
 compared bit for bit as well (the stated bar is 1e-6 relative)."""
 import os
-from ctypes import c_void_p as C_void_p
+from ctypes import byref as C_byref, c_void_p as C_void_p
 
 import numpy as np
 import pytest
@@ -25,12 +25,16 @@ def torch_cuda():
     return torch
 
 
-def _check(res, ref_out, ref_diag, what):
+def _check(res, ref_out, ref_diag, what, ref_e=None):
     assert res["rc"] == 0, what
     for f in FIELDS:
         got, exp = res["diag"][f], ref_diag[f]
         assert np.array_equal(got, exp), "%s: field %s differs, rows %s" % (what, f, np.nonzero(got != exp)[0][:8])
     assert np.array_equal(res["out"], ref_out), what
+    if ref_e is not None:
+        # e of every token bit for bit (0 for dead tokens): with the threshold above, the kept set {e >= thr}
+        bad = np.nonzero((res["e_bits"] != ref_e).any(axis=1))[0]
+        assert bad.size == 0, "%s: e differs in rows %s" % (what, bad[:8])
 
 
 def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_np=None, u_np=None,
@@ -46,45 +50,37 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     oc, ok, op = oracle.normalize(temperature, top_k, top_p, V, B, T)
     assert (c, k, p) == (oc, ok, op)
     pen_ref = None if pen_np is None else pen_np.copy()
-    ref_out, ref_diag = oracle.sample_batch(logits_np, c, k, p, injected_u=u_np, penalties=pen_ref,
-                                            presence=presence, repetition=repetition, decay=decay)
-    if force_r is None:
-        os.environ.pop("RS_FORCE_R", None)
-    else:
-        os.environ["RS_FORCE_R"] = str(force_r)
-    try:
-        smp = capi.Sampler(B, V)
-        lg = torch.from_numpy(logits_np).cuda()
-        if dtype is not None:
-            lg = lg.to(dtype)
-            assert torch.equal(lg.float().cpu(), torch.from_numpy(logits_np)) or np.isnan(logits_np).any()
-        pen = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
-        u = torch.from_numpy(u_np).cuda()
-        print("case", what, "B", B, "T", T, "V", V, "k", k, "p", p, "R", force_r, flush=True)
-        res = smp.sample(lg, c, k, p, uniforms=u, penalties=pen, presence=presence, repetition=repetition,
-                         decay=decay, want_e=True)
-        _check(res, ref_out, ref_diag, what)
-        assert smp.status() == 0
-        if pen is not None:
-            assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32)), what + ": penalties"
-        # second call on the same workspace: it must have been left clean
-        pen2 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
-        res2 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen2, presence=presence, repetition=repetition,
-                          decay=decay)
-        _check(res2, ref_out, ref_diag, what + " (second call)")
-        if pen_np is None:
-            # the wait-free streaming path (taken for top_k <= 1024; rows it cannot finish go on to
-            # the cluster kernel), the same attempted whatever top_k is, then the cluster path again
-            # on the workspace these leave behind
-            for path in ("stream", "optimistic", "cluster"):
-                os.environ["RS_FORCE_PATH"] = path
-                res3 = smp.sample(lg, c, k, p, uniforms=u)
-                _check(res3, ref_out, ref_diag, what + " (path %s)" % path)
-                assert smp.status() == 0
-        return res, ref_diag
-    finally:
-        os.environ.pop("RS_FORCE_R", None)
-        os.environ.pop("RS_FORCE_PATH", None)
+    ref_out, ref_diag, ref_e = oracle.sample_batch(logits_np, c, k, p, injected_u=u_np, penalties=pen_ref,
+                                                   presence=presence, repetition=repetition, decay=decay, want_e=True)
+    smp = capi.Sampler(B, V)
+    lg = torch.from_numpy(logits_np).cuda()
+    if dtype is not None:
+        lg = lg.to(dtype)
+        assert torch.equal(lg.float().cpu(), torch.from_numpy(logits_np)) or np.isnan(logits_np).any()
+    pen = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
+    u = torch.from_numpy(u_np).cuda()
+    print("case", what, "B", B, "T", T, "V", V, "k", k, "p", p, "R", force_r, flush=True)
+    res = smp.sample(lg, c, k, p, uniforms=u, penalties=pen, presence=presence, repetition=repetition,
+                     decay=decay, want_e=True, force_r=force_r)
+    _check(res, ref_out, ref_diag, what, ref_e)
+    assert smp.status() == 0
+    if pen is not None:
+        assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32)), what + ": penalties"
+    # second call on the same workspace: it must have been left clean
+    pen2 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
+    res2 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen2, presence=presence, repetition=repetition,
+                      decay=decay, force_r=force_r)
+    _check(res2, ref_out, ref_diag, what + " (second call)")
+    if pen_np is None:
+        # the general kernel alone, the wait-free streaming path (taken for top_k <= 1024; rows it cannot
+        # finish go on to the general kernel), the same attempted whatever top_k is (both with the e of
+        # every token: the kept set on that path), then the general kernel again on the workspace these
+        # leave behind
+        for path in ("cluster", "stream", "optimistic", "cluster"):
+            res3 = smp.sample(lg, c, k, p, uniforms=u, path=path, force_r=force_r, want_e=path != "cluster")
+            _check(res3, ref_out, ref_diag, what + " (path %s)" % path, ref_e if path != "cluster" else None)
+            assert smp.status() == 0
+    return res, ref_diag
 
 
 def test_c1_uniform_logits_top_p(torch_cuda, oracle):
@@ -226,20 +222,16 @@ def test_streaming_path_mixed_rows(torch_cuda, oracle):
     for (k, p) in [(50, 0.9), (1024, 0.95), (1, 1.0), (1000, 0.2), (7, 1.0), (1024, 1.0)]:
         _run_case(torch_cuda, oracle, capi, lg, 0.9, k, p, u_np=H.uniforms(10, 91), what="stream mixed k=%s p=%s" % (k, p))
     # which rows the streaming path finished itself (diag.rounds == 0) and which it handed on
-    os.environ["RS_FORCE_PATH"] = "stream"
-    try:
-        rc, c, k, p = capi.normalize(0.9, 50, 0.9, V, 10, 1)
-        res = capi.Sampler(10, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p,
-                                         uniforms=torch_cuda.from_numpy(H.uniforms(10, 91)).cuda())
-        rounds = res["diag"]["rounds"]
-        assert rounds[0] == 0 and rounds[1] == 0 and rounds[8] == 0 and rounds[9] == 0, rounds
-        # slices whose maxima are more than 87 octaves apart (rows 2, 3, 5, 6): what the far ones put
-        # into the row's bins is taken out again, and the row is finished all the same
-        assert all(rounds[i] == 0 for i in (2, 3, 5, 6)), rounds
-        # a tie of all 69632 tokens needs no stash: recognised from the row's bins and finished as well
-        assert rounds[4] == 0, rounds
-    finally:
-        os.environ.pop("RS_FORCE_PATH", None)
+    rc, c, k, p = capi.normalize(0.9, 50, 0.9, V, 10, 1)
+    res = capi.Sampler(10, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p, path="stream",
+                                     uniforms=torch_cuda.from_numpy(H.uniforms(10, 91)).cuda())
+    rounds = res["diag"]["rounds"]
+    assert rounds[0] == 0 and rounds[1] == 0 and rounds[8] == 0 and rounds[9] == 0, rounds
+    # slices whose maxima are more than 87 octaves apart (rows 2, 3, 5, 6): what the far ones put
+    # into the row's bins is taken out again, and the row is finished all the same
+    assert all(rounds[i] == 0 for i in (2, 3, 5, 6)), rounds
+    # a tie of all 69632 tokens needs no stash: recognised from the row's bins and finished as well
+    assert rounds[4] == 0, rounds
 
 
 def test_c5_full_size_paths_agree(torch_cuda, oracle):
@@ -258,18 +250,14 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
     u = torch.from_numpy(H.uniforms(B, 123)).cuda()
     smp = capi.Sampler(B, V)
     res = {}
-    try:
-        for path in ("stream", "cluster", "stream"):
-            os.environ["RS_FORCE_PATH"] = path
-            print("full C5", path, flush=True)
-            r = smp.sample(lg, c, k, p, uniforms=u)
-            assert r["rc"] == 0 and smp.status() == 0
-            if path in res:
-                for f in FIELDS:
-                    assert np.array_equal(res[path]["diag"][f], r["diag"][f]), "repeat differs: " + f
-            res[path] = r
-    finally:
-        os.environ.pop("RS_FORCE_PATH", None)
+    for path in ("stream", "cluster", "stream"):
+        print("full C5", path, flush=True)
+        r = smp.sample(lg, c, k, p, uniforms=u, path=path)
+        assert r["rc"] == 0 and smp.status() == 0
+        if path in res:
+            for f in FIELDS:
+                assert np.array_equal(res[path]["diag"][f], r["diag"][f]), "repeat differs: " + f
+        res[path] = r
     for f in FIELDS:
         assert np.array_equal(res["stream"]["diag"][f], res["cluster"]["diag"][f]), f
     assert np.array_equal(res["stream"]["out"], res["cluster"]["out"])
@@ -300,18 +288,14 @@ def test_streaming_path_flat_distributions(torch_cuda, oracle):
     lg[6] = np.round(rng.random(V, dtype=np.float32) * 64) / 64         # 65 distinct values: ties of a thousand tokens
     for (k, p) in [(100, 0.9), (10, 1.0), (1000, 0.3), (1, 1.0), (1024, 1.0)]:
         _run_case(torch_cuda, oracle, capi, lg, 1.0, k, p, u_np=H.uniforms(7, 41), what="flat k=%s p=%s" % (k, p))
-    os.environ["RS_FORCE_PATH"] = "stream"
-    try:
-        rc, c, k, p = capi.normalize(1.0, 100, 0.9, V, 7, 1)
-        res = capi.Sampler(7, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p,
-                                        uniforms=torch_cuda.from_numpy(H.uniforms(7, 41)).cuda())
-        rounds = res["diag"]["rounds"]
-        assert all(rounds[i] == 0 for i in (1, 2, 3, 4, 6)), rounds     # finished from the stashes
-        assert rounds[0] == 0, rounds                                   # all equal: one tie, recognised as such
-        # handed on: a row so flat that even a level-2 sub-bin holds more tokens than a stash
-        assert rounds[5] >= 1, rounds
-    finally:
-        os.environ.pop("RS_FORCE_PATH", None)
+    rc, c, k, p = capi.normalize(1.0, 100, 0.9, V, 7, 1)
+    res = capi.Sampler(7, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p, path="stream",
+                                    uniforms=torch_cuda.from_numpy(H.uniforms(7, 41)).cuda())
+    rounds = res["diag"]["rounds"]
+    assert all(rounds[i] == 0 for i in (1, 2, 3, 4, 6)), rounds     # finished from the stashes
+    assert rounds[0] == 0, rounds                                   # all equal: one tie, recognised as such
+    # handed on: a row so flat that even a level-2 sub-bin holds more tokens than a stash
+    assert rounds[5] >= 1, rounds
 
 
 @pytest.mark.parametrize("B,V", [(6, 65536 + 4096), (20, 262144 + 4096)])
@@ -336,15 +320,11 @@ def test_streaming_path_peaked_and_masked_rows(torch_cuda, oracle, B, V):
     u = H.uniforms(B, 17)
     for (k, p, t) in [(50, 0.9, 1.0), (1024, 1.0, 0.7), (3, 0.5, 0.05), (1000, 0.999, 4.0)]:
         _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="peaked k=%s p=%s T=%s" % (k, p, t))
-    os.environ["RS_FORCE_PATH"] = "stream"
-    try:
-        rc, c, k, p = capi.normalize(1.0, 50, 0.9, V, B, 1)
-        res = capi.Sampler(B, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p,
-                                        uniforms=torch_cuda.from_numpy(u).cuda())
-        rounds = res["diag"]["rounds"]
-        assert all(rounds[i] == 0 for i in range(B)), rounds
-    finally:
-        os.environ.pop("RS_FORCE_PATH", None)
+    rc, c, k, p = capi.normalize(1.0, 50, 0.9, V, B, 1)
+    res = capi.Sampler(B, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p, path="stream",
+                                    uniforms=torch_cuda.from_numpy(u).cuda())
+    rounds = res["diag"]["rounds"]
+    assert all(rounds[i] == 0 for i in range(B)), rounds
 
 
 def test_streaming_path_whole_slice_stash_beside_partial_ones(torch_cuda, oracle):
@@ -652,17 +632,14 @@ def test_hip_graph_decode_loop(torch_cuda, oracle, path, pen_on):
     assert capi.lib().rs_philox_init(st.data_ptr(), 99, B, smp.stream()) == 0
     rng_ref = oracle.rng_init(99, B)
     torch.cuda.synchronize()
-    os.environ["RS_FORCE_PATH"] = path
-    try:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            rc = capi.lib().rs_sample(lg.data_ptr(), V, pen.data_ptr() if pen_on else None, out.data_ptr(),
-                                      st.data_ptr(), None, B, V, 0.1, 0.2, 0.9, c, k, p,
-                                      smp.ws.data_ptr(), smp.ws.numel(), None, None, smp.stream())
-            hist += out                                   # a consumer of the sampled ids inside the graph
-        assert rc == 0
-    finally:
-        os.environ.pop("RS_FORCE_PATH", None)
+    opt = capi.Options(capi.PATHS[path], 0, None)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = capi.lib().rs_sample_ex(lg.data_ptr(), 0, V, pen.data_ptr() if pen_on else None, out.data_ptr(),
+                                     st.data_ptr(), None, B, V, 0.1, 0.2, 0.9, c, k, p,
+                                     smp.ws.data_ptr(), smp.ws.numel(), None, None, C_byref(opt), smp.stream())
+        hist += out                                   # a consumer of the sampled ids inside the graph
+    assert rc == 0
     total = np.zeros(B, dtype=np.int64)
     for i in range(replays):
         ref_out, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref, penalties=pen_ref,
@@ -752,18 +729,14 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     lg_peaked, lg_flat = torch.from_numpy(peaked).cuda(), torch.from_numpy(flat).cuda()
 
     def policy(smp):
-        st = C.c_int32(-5)
-        assert capi.lib().rs_workspace_policy(smp.ws.data_ptr(), C.byref(st)) == 0
-        return st.value
+        return smp.policy_state()
 
-    plain = capi.Sampler(B, V)                           # zeroed by torch: no report word
-    assert policy(plain) == -1
+    plain = capi.Sampler(B, V)                           # no policy: no report words
     res = plain.sample(lg_peaked, c, k, p, uniforms=u)
-    _check(res, *ref_peaked, "zeroed workspace")
+    _check(res, *ref_peaked, "no policy")
     assert (res["diag"]["rounds"] >= 1).all()            # general kernel
 
-    smp = capi.Sampler(B, V)
-    assert capi.lib().rs_workspace_init(smp.ws.data_ptr(), smp.ws.numel(), smp.stream()) == 0
+    smp = capi.Sampler(B, V, with_policy=True, init=True)
     assert policy(smp) == 0
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)
     _check(res, *ref_peaked, "attempt on peaked rows")
@@ -805,8 +778,9 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
     assert policy(smp) == 0
     res = plain.sample(lg_ties, c, k, p, uniforms=u)     # no report words: streams whatever happened before
-    _check(res, *ref_ties, "bounded, zeroed workspace")
-    assert policy(plain) == -1 and plain.status() == 0 and smp.status() == 0
+    _check(res, *ref_ties, "bounded, no policy")
+    assert plain.status() == 0 and smp.status() == 0 and smp.policy_error() == 0
+    smp.close()
 
 
 def test_two_streams_two_workspaces_concurrently(torch_cuda, oracle):
@@ -855,9 +829,10 @@ def test_two_streams_two_workspaces_concurrently(torch_cuda, oracle):
 
 def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
     """A workspace that was never cleaned (here: filled with ones behind its header) holds histograms that
-    never add up.  The workgroups must give up after the bound of their waits (shortened to 20 ms through
-    the test hook of rs_workspace_init), leave a sticky RS_ERR_DEVICE and end normally; after
-    rs_workspace_init the same workspace works again."""
+    never add up.  The workgroups must give up after the bound of their waits (shortened to 20 ms with
+    rs_workspace_set_wait_limit), leave a sticky RS_ERR_DEVICE -- also in the pinned host word of the
+    caller's rs_policy, readable without synchronising -- and end normally; after rs_workspace_init the
+    same workspace works again."""
     torch = torch_cuda
     from tests import capi
     B, V = 2, 65536
@@ -865,24 +840,106 @@ def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
     rc, c, k, p = capi.normalize(1.0, -1, 0.9, V, B, 1)
     u_np = H.uniforms(B, 81)
     ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np)
-    smp = capi.Sampler(B, V)
+    smp = capi.Sampler(B, V, with_policy=True, init=True)
     lg, u = torch.from_numpy(lg_np).cuda(), torch.from_numpy(u_np).cuda()
-    os.environ["RS_SPIN_LIMIT_MS"] = "20"
-    try:
-        assert capi.lib().rs_workspace_init(smp.ws.data_ptr(), smp.ws.numel(), smp.stream()) == 0
-        smp.ws[256:] = 1
+    smp.set_wait_limit(20)
+    smp.ws[256:] = 1
+    torch.cuda.synchronize()
+    assert smp.policy_error() == 0
+    print("poisoned workspace, expecting a bounded wait to give up", flush=True)
+    res = smp.sample(lg, c, k, p, uniforms=u, want_diag=False, path="cluster")
+    assert res["rc"] == 0                       # the launch itself is fine
+    assert smp.policy_error() == -9             # reported to the host without a device read
+    assert smp.status() == -9                   # RS_ERR_DEVICE, sticky
+    smp.reinit()
+    assert smp.policy_error(clear=True) == -9 and smp.policy_error() == 0
+    assert smp.status() == 0
+    res = smp.sample(lg, c, k, p, uniforms=u)
+    _check(res, ref_out, ref_diag, "after re-initialisation")
+    assert smp.status() == 0 and smp.policy_error() == 0
+    smp.close()
+
+
+def test_python_module_raises_after_a_failed_call_and_recovers(torch_cuda, oracle):
+    """The same failure through the drop-in module, whose workspace is private: the call whose kernel gave
+    up returns (its result is garbage), the next call on that stream raises RuntimeError and sets the
+    workspace up again, and the call after that is correct.  workspace_status() tells at once."""
+    torch = torch_cuda
+    import rapid_sampling_amd as sample
+    B, V = 2, 32768                                  # small enough to take the general kernel, several workgroups per row
+    lg_np = H.logits_normal(B, V, 2.0, seed=82)
+    c, k, p = oracle.normalize(1.0, -1, 0.9, V, B, 1)
+    u_np = H.uniforms(B, 83)
+    ref_out, _ = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np)
+    lg, u = torch.from_numpy(lg_np).cuda(), torch.from_numpy(u_np).cuda()
+    st = sample.setup_rand(1, B)
+    side = torch.cuda.Stream()                       # a stream of its own: its workspace is this test's alone
+    with torch.cuda.stream(side):
+        out = sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)
+        assert np.array_equal(out.cpu().numpy(), ref_out) and sample.workspace_status() == 0
+        for check in ("next call", "status"):
+            sample.set_wait_limit(20)
+            ws = sample._sample.debug_workspace()
+            ws[256:] = 1
+            side.synchronize()
+            print("poisoned module workspace:", check, flush=True)
+            sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)      # gives up; no exception yet
+            if check == "next call":
+                side.synchronize()
+                with pytest.raises(RuntimeError, match="earlier sampling call"):
+                    sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)
+            else:
+                assert sample.workspace_status() == -9
+            out = sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)
+            assert np.array_equal(out.cpu().numpy(), ref_out), check
+            assert sample.workspace_status() == 0
+    side.synchronize()
+
+
+def test_python_module_calls_captured_into_a_graph(torch_cuda, oracle):
+    """The drop-in module under torch.cuda.graph: the workspace is reserved before the capture (growing it
+    while capturing raises a clear error), the captured calls replay as a decode loop that continues the
+    Philox stream and the penalties, and an eager call on the capture stream between replays works."""
+    torch = torch_cuda
+    import rapid_sampling_amd as sample
+    B, V, replays = 4, 65536, 4
+    lg_np = H.logits_normal(B, V, 2.0, seed=84)
+    pen_ref = H.penalties_sparse(B, V, seed=85)
+    c, k, p = oracle.normalize(0.9, 40, 0.9, V, B, 1)
+    rng_ref = oracle.rng_init(5, B)
+    lg = torch.from_numpy(lg_np).cuda()
+    pen = torch.from_numpy(pen_ref.copy()).cuda()
+    st = sample.setup_rand(5, B)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        sample.reserve_workspace(B, V)
+        with torch.cuda.graph(graph, stream=side):
+            a = sample.batch_sampling_temperature_topk_topp(lg, st, 0.9, 40, 0.9)
+            b = sample.batch_sampling_repetition_temperature_topk_topp(lg, pen, st, 0.1, 0.2, 0.9, 0.9, 40, 0.9)
+    side.synchronize()
+    for i in range(replays):
+        ref_a, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref)
+        ref_b, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref, penalties=pen_ref, presence=0.1, repetition=0.2, decay=0.9)
+        print("module graph replay", i, flush=True)
+        graph.replay()
         torch.cuda.synchronize()
-        print("poisoned workspace, expecting a bounded wait to give up", flush=True)
-        res = smp.sample(lg, c, k, p, uniforms=u, want_diag=False)
-        assert res["rc"] == 0                       # the launch itself is fine
-        assert smp.status() == -9                   # RS_ERR_DEVICE, sticky
-        assert capi.lib().rs_workspace_init(smp.ws.data_ptr(), smp.ws.numel(), smp.stream()) == 0
-        assert smp.status() == 0
-        res = smp.sample(lg, c, k, p, uniforms=u)
-        _check(res, ref_out, ref_diag, "after re-initialisation")
-        assert smp.status() == 0
-    finally:
-        os.environ.pop("RS_SPIN_LIMIT_MS", None)
+        assert np.array_equal(a.cpu().numpy(), ref_a) and np.array_equal(b.cpu().numpy(), ref_b), i
+        with torch.cuda.stream(side):                    # an eager call on the same stream and workspace
+            ref_c, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref)
+            cc = sample.batch_sampling_temperature_topk_topp(lg, st, 0.9, 40, 0.9)
+            assert np.array_equal(cc.cpu().numpy(), ref_c), i
+    assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32))
+    with torch.cuda.stream(side):
+        assert sample.workspace_status() == 0
+    # a stream without a workspace: the first call would have to allocate while capturing
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(other):
+        with pytest.raises(RuntimeError, match="reserve_workspace"):
+            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=other):
+                sample.batch_sampling_temperature_topk_topp(lg, st, 0.9, 40, 0.9)
+    torch.cuda.synchronize()
 
 
 def test_chi_square_one_million_draws(torch_cuda, oracle):
