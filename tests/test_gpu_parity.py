@@ -190,6 +190,27 @@ def test_masked_tokens_are_never_returned(torch_cuda, oracle):
                     assert dead.sum() == V - len(live[b])
 
 
+@pytest.mark.parametrize("B,V,top_k,top_p,gen", [(512, 256, 10, 0.9, 3), (512, 256, -1, 1.0, 0), (512, 256, 1, 0.1, 4),
+                                                  (512, 262144, 10000, 0.7, 3), (512, 262144, -1, 0.1, 1)])
+def test_corners_of_the_reference_benchmark_grid(torch_cuda, oracle, B, V, top_k, top_p, gen):
+    """The extremes of the reference's benchmark sweep (/root/reference/bench.py:32-35: B up to 512, V from
+    256 to 262144, top_k up to 10000, top_p down to 0.1) with its logit generators (bench.py:66-72:
+    zeros, U[0,1), N(0,1)/2, N(0,1)*3, U[0,1)*4): 512 rows of one workgroup each, and 512 rows of a quarter
+    million tokens with a kept set of thousands."""
+    from tests import capi
+    rng = np.random.default_rng(1000 * gen + V % 1000 + B)
+    if gen == 0:
+        lg = np.zeros((B, V), dtype=np.float32)
+    elif gen == 1:
+        lg = rng.random((B, V), dtype=np.float32)
+    elif gen == 3:
+        lg = rng.standard_normal((B, V), dtype=np.float32) * np.float32(3.0)
+    else:
+        lg = rng.random((B, V), dtype=np.float32) * np.float32(4.0)
+    _run_case(torch_cuda, oracle, capi, lg, 1.0, top_k, top_p, u_np=H.uniforms(B, 55),
+              what="sweep corner B=%d V=%d k=%d p=%g gen=%d" % (B, V, top_k, top_p, gen))
+
+
 def test_uniform_extremes(torch_cuda, oracle):
     """u -> 0+ picks the first kept token, u = 1 the last one."""
     from tests import capi
@@ -238,8 +259,7 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
     """BASELINE config 5 at its full size, (B,T,V) = (128,4,1048576) fp32 = 2 GiB, top_k 1024, top_p 0.95.
     Too large for the oracle in a test; checked through what does not depend on size: the streaming path
     and the cluster path are different decompositions of the same integer arithmetic, so every diagnostic
-    and every index must be equal; the sampled token must lie in the kept set; 8 of the rows are also run
-    through the oracle."""
+    and every index must be equal; and all 128 sampled rows are run through the oracle as well."""
     torch = torch_cuda
     from tests import capi
     B, T, V = 128, 4, 1048576
@@ -264,12 +284,12 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
     assert (res["stream"]["diag"]["rounds"] == 0).all()            # every row finished by the streaming path
     d = res["stream"]["diag"]
     assert (d["n_gt"] < 1024).all() and (d["n_gt"] + d["n_eq"] >= 1).all()
-    rows = [0, 1, 17, 63, 64, 100, 126, 127]
-    sub = lg[rows, T - 1, :].cpu().numpy()
-    ref_out, ref_diag = oracle.sample_batch(sub, c, k, p, injected_u=H.uniforms(B, 123)[rows])
-    for f in FIELDS:
-        assert np.array_equal(d[f][rows], ref_diag[f]), f
-    assert np.array_equal(res["stream"]["out"][rows], ref_out)
+    for lo in range(0, B, 32):                                       # 32 rows (128 MiB) at a time
+        sub = lg[lo:lo + 32, T - 1, :].cpu().numpy()
+        ref_out, ref_diag = oracle.sample_batch(sub, c, k, p, injected_u=H.uniforms(B, 123)[lo:lo + 32])
+        for f in FIELDS:
+            assert np.array_equal(d[f][lo:lo + 32], ref_diag[f]), (f, lo)
+        assert np.array_equal(res["stream"]["out"][lo:lo + 32], ref_out), lo
 
 
 def test_streaming_path_flat_distributions(torch_cuda, oracle):
@@ -561,12 +581,14 @@ def test_penalty_path_single_step(torch_cuda, oracle):
                   presence=0.25, repetition=0.1, decay=0.95, force_r=R, what="penalty step R%d" % R)
 
 
-def test_c4_penalty_chain(torch_cuda, oracle):
+@pytest.mark.parametrize("steps", [24, 256])
+def test_c4_penalty_chain(torch_cuda, oracle, steps):
     """BASELINE config 4 (B=32, V=131072, 2 % Exp(1) penalties, presence=repetition=0.1, decay=0.95,
-    T=0.8, top_k=50, top_p=0.9) for 24 chained steps on fixed logits; penalties evolve in place on both sides."""
+    T=0.8, top_k=50, top_p=0.9): chained decode steps on fixed logits, penalties evolving in place on both
+    sides -- the 256 steps the configuration states, and a quick 24-step case."""
     torch = torch_cuda
     from tests import capi
-    B, V, steps = 32, 131072, 24
+    B, V = 32, 131072
     lg_np = H.logits_normal(B, V, 1.5, seed=40)
     pen_ref = H.penalties_sparse(B, V, seed=41)
     rc, c, k, p = capi.normalize(0.8, 50, 0.9, V, B, 1)
