@@ -35,6 +35,7 @@ extern "C" {
 #define RS_ERR_ARG         -7   /* top_k / top_p not normalised (use rs_normalize_args)       */
 #define RS_ERR_LAUNCH      -8   /* the HIP runtime refused the launch                         */
 #define RS_ERR_DEVICE      -9   /* a kernel gave up waiting for its peer workgroups           */
+#define RS_ERR_SCRATCH     -10  /* rs_sample_static: the call needs more than RS_STATIC_SCRATCH_BYTES */
 
 /* Bytes of RNG state per row.  Same size as the reference's
  * curandStatePhilox4_32_10_t record (sampling.cu:9,141) so that the opaque
@@ -249,6 +250,37 @@ int rs_sample_ex(const void *logits_device, int32_t logits_dtype, int64_t row_st
                  void *workspace_device, size_t workspace_bytes,
                  rs_row_diag *diag_device, uint32_t *e_bits_device,
                  const rs_options *options, void *stream);
+
+/*
+ * rs_sample_ex without a workspace argument, for callers that cannot allocate
+ * device memory or carry a workspace along: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.
+ *
+ * The workspace is a static array in device memory inside the library,
+ * RS_STATIC_SCRATCH_BYTES (32 MiB) on every GPU the library is used on, held
+ * until the process ends.  A call whose rs_workspace_bytes(B, V) exceeds that
+ * size is refused with RS_ERR_SCRATCH before anything is launched (64 rows of
+ * 152064 tokens need 16 MiB, 32 rows of 131072 tokens 14 MiB; 128 rows of
+ * 1048576 tokens, 105 MB, do not fit).  The call allocates nothing and
+ * synchronises nothing: it enqueues one small kernel that clears the launch
+ * header and the B row records the call is about to use (so it also recovers
+ * by itself after an RS_ERR_DEVICE), then exactly what rs_sample_ex enqueues.
+ * The address of the array is looked up once per device, on the first call
+ * made while that device is current.
+ *
+ * Every call on a GPU uses that GPU's one array: calls must be ordered on one
+ * stream (or otherwise serialised); calls that overlap on one GPU race.
+ */
+#define RS_STATIC_SCRATCH_BYTES (32u << 20)
+int rs_sample_static(const void *logits_device, int32_t logits_dtype, int64_t row_stride,
+                     float *penalties_device, int32_t *out_device,
+                     void *rng_state_device, const float *injected_u_device,
+                     int32_t B, int32_t V,
+                     float presence_penalty, float repetition_penalty, float penalty_decay,
+                     float log2e_inv_temp, int32_t top_k, float top_p,
+                     rs_row_diag *diag_device, uint32_t *e_bits_device,
+                     const rs_options *options, void *stream);
 
 /*
  * Launch-plus-one-read floor: a kernel with rs_sample's grid for (B,V) that

@@ -38,10 +38,15 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <new>
 
 #include "rapid_sampling.h"
 #include "rs_device.h"
+
+// Workspace of rs_sample_static: one array per GPU inside the library's code object.  In host code
+// this name is only a handle for hipGetSymbolAddress, never an address.
+static __device__ __align__(256) unsigned char scratch[RS_STATIC_SCRATCH_BYTES];
 
 namespace rs {
 
@@ -1916,6 +1921,14 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint4 *dst, size_t n16, 
 
 __global__ void set_u32_kernel(uint32_t *dst, uint32_t value) { *dst = value; }
 
+// What a call reads before it writes: the launch header and its row records.
+__global__ void __launch_bounds__(256) clear_records_kernel(uint4 *hdr, uint4 *recs, size_t n16)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) recs[i] = make_uint4(0u, 0u, 0u, 0u);
+    if (blockIdx.x == 0 && threadIdx.x < sizeof(WsHeader) / 16) hdr[threadIdx.x] = make_uint4(0u, 0u, 0u, 0u);
+}
+
 // ------------------------------------------------------------ host side ----
 
 struct Geometry { int R; uint32_t G; };
@@ -2098,6 +2111,7 @@ const char *rs_error_string(int code)
     case RS_ERR_ARG:         return "top_k/top_p not normalised: need 1 <= top_k <= V and 0 < top_p <= 1";
     case RS_ERR_LAUNCH:      return "HIP launch failed";
     case RS_ERR_DEVICE:      return "a workgroup gave up waiting for its peers";
+    case RS_ERR_SCRATCH:     return "the call needs a larger workspace than the static scratch of rs_sample_static (RS_STATIC_SCRATCH_BYTES)";
     default:                 return "unknown error";
     }
 }
@@ -2309,6 +2323,40 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
                        : pen ? launch_sample<true>(g.R, grid, (hipStream_t)stream, p)
                              : launch_sample<false>(g.R, grid, (hipStream_t)stream, p);
     return e == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                     void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                     float presence, float repetition, float decay,
+                     float log2e_inv_temp, int32_t top_k, float top_p,
+                     rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
+{
+    size_t need = 0;
+    const int rc = rs_workspace_bytes(B, V, &need);
+    if (rc != RS_OK) return rc;
+    if (need > (size_t)RS_STATIC_SCRATCH_BYTES) return RS_ERR_SCRATCH;
+    // every GPU holds its own copy of the array at its own address: looked up once per device
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void *> base[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return RS_ERR_LAUNCH;
+    void *ws = base[dev].load(std::memory_order_acquire);
+    if (!ws) {
+        if (hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch)) != hipSuccess || !ws) return RS_ERR_LAUNCH;
+        base[dev].store(ws, std::memory_order_release);
+    }
+    // The array keeps what the last call left.  A call leaves it clean unless a wait gave up; the launch
+    // header and this call's row records are cleared all the same, by a kernel (not a memset node: the
+    // call may be under capture), so that every call starts from zero whatever came before.
+    const size_t rec_bytes = (size_t)B * sizeof(RowCtl);
+    char *recs = (char *)ws + (size_t)RS_STATIC_SCRATCH_BYTES - rec_bytes;
+    const size_t n16 = rec_bytes / 16;
+    const uint32_t blocks = (uint32_t)(n16 / 1024 < 1 ? 1 : n16 / 1024 > 1024 ? 1024 : n16 / 1024);
+    hipLaunchKernelGGL(clear_records_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint4 *)ws, (uint4 *)recs, n16);
+    if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
+    return rs_sample_ex(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                        repetition, decay, log2e_inv_temp, top_k, top_p, ws, (size_t)RS_STATIC_SCRATCH_BYTES, diag,
+                        e_bits, opt, stream);
 }
 
 int rs_floor_read(const float *logits, int64_t row_stride, int32_t *out, int32_t B, int32_t V, void *stream)

@@ -68,6 +68,9 @@ def lib():
         L.rs_sample_dtype.restype = C.c_int
         L.rs_sample_dtype.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
                                       vp, sz, vp, vp, vp]
+        L.rs_sample_static.restype = C.c_int
+        L.rs_sample_static.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
+                                       vp, vp, C.POINTER(Options), vp]
         L.rs_floor_read.restype = C.c_int
         L.rs_floor_read.argtypes = [vp, i64, vp, i32, i32, vp]
         _lib = L
