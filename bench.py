@@ -11,8 +11,10 @@ device-side time of one call in microseconds (HIP events around each call on the
 stream the kernel runs on).  Next to it, in the same JSON line:
 
   latency    the launch-plus-one-read floor kernel timed the same way, the
-             ratio to it, and the wall-clock "call + synchronize" time the
-             reference's own bench measures (reference bench.py:84-92)
+             ratio to it, the wall-clock "call + synchronize" time the
+             reference's own bench measures (reference bench.py:84-92), and
+             `readme_point`: the one point the reference publishes
+             (README.md:21-31: same shape, logits U[0,1)*4)
   roofline   the bandwidth-bound configuration (BASELINE.json configs[4]):
              logits (128,4,1048576) fp32 = 2 GiB resident, top_k 1024,
              top_p 0.95; algorithmic bytes = 4*V per sampled row; the time
@@ -35,6 +37,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, vendor figure
+
+# HBM bytes per call of the bandwidth configuration from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+# summarised in the file named here, valid for the library version they were taken with: a library
+# that has moved on reports traffic as null rather than a stale figure.
+TRAFFIC_PROFILE = {"file": "profiles/bench_kernels_hbm_traffic_pmc.md", "rs_version": 300, "bytes": 574428160}
 
 
 def event_times_us(torch, fn, steps, warmup):
@@ -151,6 +158,8 @@ def main():
 
     import rapid_sampling_amd as sample
 
+    import ctypes
+    lib_version = ctypes.CDLL(sample.KERNEL_LIBRARY).rs_version()
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
@@ -175,6 +184,21 @@ def main():
     b2b_us = block_time_us(torch, call, min(args.steps, 2000), 20)
     floor_b2b_us = block_time_us(torch, floor, min(args.steps, 2000), 20)
 
+    # the reference's one published point: same B, V, top_k, top_p, logits U[0,1)*4 (bench.py:72, logit type 4)
+    flat_np = (np.random.default_rng(4).random(V, dtype=np.float32) * np.float32(4.0)).astype(np.float32)
+    flat = torch.from_numpy(flat_np)[None, :].to(dev)
+    side = torch.cuda.Stream()                            # its own stream: its own workspace and routing state
+
+    def call_flat_row():
+        return sample.batch_sampling_temperature_topk_topp(flat, states, temperature, top_k, top_p)
+
+    with torch.cuda.stream(side):
+        readme_us, _ = event_times_us(torch, call_flat_row, min(args.steps, 2000), min(args.warmup, 100))
+        readme_sync = sync_call_us(torch, call_flat_row, 200)
+        readme_state = sample._sample.policy_state()
+    side.synchronize()
+    readme_p50 = statistics.median(readme_us)
+
     result = {
         "metric": "p50 us/call (B=1,V=256K); HBM GB/s vs peak at B=128x4,V=1M",
         "value": round(p50, 3),
@@ -198,6 +222,14 @@ def main():
             "call_plus_sync_p50_us": round(statistics.median(sync_us), 2),
             "reference_call_plus_sync_us": 220.3,
             "reference_note": "reference README.md:21-31: same B, V, top_p, top_k, logits U[0,1)*4, unnamed NVIDIA GPU",
+            "readme_point": {
+                "workload": "B=1, V=262144, logits U[0,1)*4 seed 4, temperature 1.0, top_k -1, top_p 0.3 (README.md:21-31)",
+                "p50_us": round(readme_p50, 3), "ratio_to_floor": round(readme_p50 / floor_p50, 3),
+                "call_plus_sync_p50_us": round(statistics.median(readme_sync), 2),
+                "path": "general kernel (the flat row's nucleus is too large for the streaming path; routed by its reports)"
+                        if readme_state & 1 else "streaming path",
+                "reference_call_plus_sync_us": 220.3,
+            },
         },
     }
 
@@ -218,12 +250,17 @@ def main():
         def call_flat():
             return sample.batch_sampling_temperature_topk_topp(flat, st_b, 1.0, 1024, 0.95)
 
-        def floor_btv():
-            return sample.floor_read(big)
+        def floor_variant(n):
+            return lambda: sample.floor_read(big, n)
 
         t_btv = block_time_us(torch, call_btv, args.bandwidth_steps, 3)
         t_flat = block_time_us(torch, call_flat, max(2, args.bandwidth_steps // 2), 2)
-        t_floor = block_time_us(torch, floor_btv, args.bandwidth_steps, 3)
+        # read-only kernels on the same rows: plain / non-temporal loads on the general kernel's grid
+        # and on the streaming pass's grid
+        floor_names = ["plain loads, 128 KiB per workgroup", "non-temporal loads, 128 KiB per workgroup",
+                       "plain loads, 64 KiB per workgroup", "non-temporal loads, 64 KiB per workgroup"]
+        t_floors = [block_time_us(torch, floor_variant(n), args.bandwidth_steps, 3) for n in range(4)]
+        t_floor = min(t_floors)
         sample._sample.force_path("cluster")             # the general single-launch kernel on the same input
         try:
             t_cluster = block_time_us(torch, call_btv, max(2, args.bandwidth_steps // 2), 2)
@@ -235,16 +272,17 @@ def main():
         result["roofline"] = {
             "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(ach / HBM_PEAK_GBS, 4),
-            # HBM bytes per call from the FETCH_SIZE / WRITE_SIZE counter runs of this same command
-            # (profiles/bench_kernels_hbm_traffic_pmc.md), not measured live
-            "traffic": 574428160,
+            "traffic": TRAFFIC_PROFILE["bytes"] if lib_version == TRAFFIC_PROFILE["rs_version"] else None,
+            "traffic_source": "%s (library version %d; running %d)" % (TRAFFIC_PROFILE["file"], TRAFFIC_PROFILE["rs_version"], lib_version),
             "workload": "(B,T,V)=(128,4,1048576) N(0,1.5), top_k 1024, top_p 0.95: 128 sampled rows of 4 MiB, "
                         "stride T*V, algorithmic bytes 4*V per row = 512 MiB per call",
             "us_per_call": round(t_btv, 2), "rows_per_s": round(Bb / (t_btv * 1e-6), 1),
             "kernels": "streaming path, three launches per call: rs::stream_kernel (reads the logits; dominant), "
                        "rs::finish_kernel, rs::sample_list_kernel; achieved = bytes / time of the whole call",
             "cluster_path_us_per_call": round(t_cluster, 2),
-            "read_once_floor_GBs": round(bytes_btv / (t_floor * 1e-6) / 1e9, 1),
+            "read_peak_GBs": round(bytes_btv / (t_floor * 1e-6) / 1e9, 1),
+            "frac_of_read_peak": round(t_floor / t_btv, 4),
+            "read_only_kernels_GBs": {n: round(bytes_btv / (t * 1e-6) / 1e9, 1) for n, t in zip(floor_names, t_floors)},
             "flattened_512_rows": {"us_per_call": round(t_flat, 2),
                                    "achieved": round(bytes_flat / (t_flat * 1e-6) / 1e9, 1),
                                    "rows_per_s": round(Bb * Tb / (t_flat * 1e-6), 1)},

@@ -227,8 +227,10 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
  * rs_sample_dtype).  `path` forces the way through the library (tests,
  * benchmarks): RS_PATH_CLUSTER the general one-launch kernel, RS_PATH_STREAM
  * the streaming path when top_k <= 1024 (else the general kernel),
- * RS_PATH_ATTEMPT the streaming path whatever top_k is; penalties always take
- * the general kernel.  `slice_r` forces the float4 groups per thread of the
+ * RS_PATH_ATTEMPT the streaming path whatever top_k is (penalties take the
+ * general kernel on these three), RS_PATH_FUSED the streaming pass and the
+ * finish in one launch (any call whose rows span at least two slices, with or
+ * without penalties; else the general kernel).  `slice_r` forces the float4 groups per thread of the
  * general kernel (1, 2, 4, 8, 16 or 32; 0 = chosen by the library).
  * `policy` see rs_policy.  No counterpart in the reference.
  */
@@ -236,6 +238,7 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
 #define RS_PATH_CLUSTER 1
 #define RS_PATH_STREAM  2
 #define RS_PATH_ATTEMPT 3
+#define RS_PATH_FUSED   4
 typedef struct rs_options {
     int32_t    path;
     int32_t    slice_r;
@@ -283,13 +286,16 @@ int rs_sample_static(const void *logits_device, int32_t logits_dtype, int64_t ro
                      const rs_options *options, void *stream);
 
 /*
- * Launch-plus-one-read floor: a kernel with rs_sample's grid for (B,V) that
- * reads every logit once and max-combines one int per row into out_device
- * (which it does not clear).  Measurement aid for the B=1 latency bound; no
- * counterpart in the reference.
+ * Launch-plus-one-read floor: a kernel that reads every logit of the B rows once
+ * and max-combines one int per row into out_device (which it does not clear),
+ * every thread issuing all its loads before it uses the first.  variant 0: the
+ * general kernel's grid for (B,V), plain loads; 1: the same with loads marked
+ * non-temporal (as the sampling kernels read the logits); 2, 3: the same two
+ * on the streaming pass's grid.  Measurement aid for the B=1 latency bound and
+ * for the read bandwidth the hardware delivers; no counterpart in the reference.
  */
 int rs_floor_read(const float *logits_device, int64_t row_stride, int32_t *out_device,
-                  int32_t B, int32_t V, void *stream);
+                  int32_t B, int32_t V, int32_t variant, void *stream);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,7 @@ A call whose kernel gave up waiting for its peers raises RuntimeError on the
 next call on that stream at the latest.
 
 The functions live in the compiled extension `_sample` (host layer in
-csrc/sampling.cpp, kernels in csrc/rs_kernels.hip behind the C ABI of
+csrc/sampling.cpp, kernels in csrc/rs_*.hip and csrc/rs_*.h behind the C ABI of
 include/rapid_sampling.h).  There is no Python or CPU fallback: without the
 built extension the import fails.
 """

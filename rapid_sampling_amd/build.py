@@ -36,9 +36,28 @@ def _run(cmd, verbose):
     subprocess.check_call(cmd)
 
 
+KERNEL_SOURCES = ["rs_api.hip", "rs_cluster.hip", "rs_stream.hip"]
+
+
 def build_kernels(verbose=False):
-    _run([HIPCC] + HIP_FLAGS + ["-I" + INCLUDE, "-I" + CSRC, "-o", KERNEL_LIB,
-                                os.path.join(CSRC, "rs_kernels.hip")], verbose)
+    """One object per translation unit, compiled side by side (each instantiates its own kernels;
+    no device code is linked across objects), then one shared library."""
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    flags = [f for f in HIP_FLAGS if f != "-shared"]
+    procs = []
+    for src in KERNEL_SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        cmd = [HIPCC] + flags + ["-c", "-I" + INCLUDE, "-I" + CSRC, "-o", obj, os.path.join(CSRC, src)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((cmd, obj, subprocess.Popen(cmd)))
+    objs = []
+    for cmd, obj, proc in procs:
+        if proc.wait() != 0:
+            raise subprocess.CalledProcessError(proc.returncode, cmd)
+        objs.append(obj)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", KERNEL_LIB] + objs, verbose)
     return KERNEL_LIB
 
 

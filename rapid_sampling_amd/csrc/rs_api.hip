@@ -1,0 +1,544 @@
+// MI355X (gfx950) token sampler: kernels and the C ABI of include/rapid_sampling.h.
+//
+// Steps per row (reference lines in /root/reference/sampling.cu):
+//   1  x = sf((sf(l) - pen) * c), row max                         :208-227, :547-559
+//   2  e = 2^(x - floor(max)) kept as bit patterns                :228-258
+//   3  threshold = largest t with count{e>=t} >= top_k or mass{e>=t} >= top_p*D.
+//      The reference finds it by a 4-way search on bit patterns with one pass
+//      over the row per step (:261-329); here it is a radix selection on the
+//      same bit patterns: a (count, mass) histogram over the top 10 bits, then
+//      the few tokens of the boundary bin are gathered and resolved in LDS
+//      (or, for huge bins, the next 7 bits are histogrammed, up to 4 levels).
+//   4  counts and mass above / at the threshold                   :332-355
+//   5  tie weight                                                 :365-371
+//   6  inverse-CDF pick in index order                            :374-426
+//   7  penalty decay + one-hot add, in place, from registers      :427-437
+// Everything summed across tokens is an integer, so the result does not depend
+// on how a row is cut up or in which order the pieces arrive.
+//
+// Two ways through these steps:
+//
+//   cluster path (sample_kernel, one launch): a row is worked by a CLUSTER of
+//     G workgroups of 256 threads; each thread keeps R float4 (4R tokens) in
+//     registers for the whole call, so the row is read from HBM exactly once.
+//     The workgroups of a cluster exchange histograms, the slice maxima, the
+//     boundary tokens and their kept masses through the row's record in the
+//     workspace; what is exchanged carries its own completeness (counts that
+//     add up, words that are non-zero once written), every wait is bounded.
+//     Any top_k / top_p, penalties, any batch.
+//
+//   streaming path (stream_kernel, finish_kernel, sample_list_kernel): for
+//     calls of 2^17 tokens and more without penalties whose kept set is small
+//     next to the row (top_k <= 1024, or a small nucleus).  No workgroup waits
+//     for another: one pass over the logits leaves per-row histograms and
+//     per-slice stashes of the largest tokens, a small kernel finishes each
+//     row from them, and rows it cannot finish that way go through the
+//     cluster kernel afterwards.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#include <atomic>
+#include <new>
+
+#include "rs_common.h"
+
+// Workspace of rs_sample_static: one array per GPU inside the library's code object.  In host code
+// this name is only a handle for hipGetSymbolAddress, never an address.
+static __device__ __align__(256) unsigned char scratch[RS_STATIC_SCRATCH_BYTES];
+
+namespace rs {
+
+// Launch-plus-one-read floor: same grid, each row read once (every load of a thread issued before
+// the first use, non-temporal or plain), one int out.
+template <int R, bool ONCE>
+__global__ void __launch_bounds__(kThreads) floor_kernel(const float *logits, int64_t row_stride, int32_t *out,
+                                                         int32_t V, uint32_t G)
+{
+    const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
+    const uint32_t V4 = (uint32_t)V >> 2;
+    const uint32_t base4 = part * (uint32_t)(kThreads * R) + threadIdx.x;
+    const uint4 *lg = reinterpret_cast<const uint4 *>(logits + (int64_t)row * row_stride);
+    uint4 v[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const uint4 *q = lg + min(base4 + (uint32_t)(j * kThreads), V4 - 1);
+        v[j] = ONCE ? load_once(q) : *q;
+    }
+    float m = -3.402823466e+38f;
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+        m = fmaxf(m, fmaxf(fmaxf(__uint_as_float(v[j].x), __uint_as_float(v[j].y)), fmaxf(__uint_as_float(v[j].z), __uint_as_float(v[j].w))));
+    uint32_t k = wave_max_u32(fkey(m));
+    if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<uint32_t *>(out + row), k);
+}
+
+__global__ void philox_init_kernel(uint32_t *state, uint64_t seed, int32_t B)
+{
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    uint32_t *s = state + (size_t)b * 16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0;
+    s[0] = (uint32_t)seed; s[1] = (uint32_t)(seed >> 32);
+    s[4] = (uint32_t)b;
+}
+
+// Clears device memory with plain stores (a recorded memset node misbehaves on graph replays).
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint4 *dst, size_t n16, unsigned char *tail, uint32_t ntail)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = make_uint4(0u, 0u, 0u, 0u);
+    if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+__global__ void set_u32_kernel(uint32_t *dst, uint32_t value) { *dst = value; }
+
+// What a call reads before it writes: the launch header and its row records.
+__global__ void __launch_bounds__(256) clear_records_kernel(uint4 *hdr, uint4 *recs, size_t n16)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) recs[i] = make_uint4(0u, 0u, 0u, 0u);
+    if (blockIdx.x == 0 && threadIdx.x < sizeof(WsHeader) / 16) hdr[threadIdx.x] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// ------------------------------------------------------------ host side ----
+
+struct Geometry { int R; uint32_t G; };
+
+// Tokens per thread (4R) and workgroups per row.  Large batches take long
+// slices (few peers to meet, deep loads); a lone row is cut into a few dozen
+// slices so that many CUs pull it from HBM at once.
+static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
+{
+    const uint32_t V4 = (uint32_t)V / 4;
+    const int maxR = pen ? 16 : 32;
+    auto parts = [&](int R) { return (V4 + (uint32_t)(kThreads * R) - 1) / (uint32_t)(kThreads * R); };
+    if (force_r) {
+        const int R = force_r;
+        if ((R == 1 || R == 2 || R == 4 || R == 8 || R == 16 || R == 32) && R <= maxR && parts(R) <= (uint32_t)kMaxParts)
+            return {R, parts(R)};
+    }
+    // Measured on MI355X: a cluster works best with at most ~64 workgroups (each exchange costs
+    // more the more peers poll), slices of 32 float4 per thread only pay for rows of a quarter
+    // million tokens and more (the variant spills), and a call wants a few hundred workgroups in
+    // flight -- 256 for small batches, where latency counts, 512 beyond.
+    int minR = maxR;
+    for (int R = 1; R <= maxR; R *= 2)
+        if (parts(R) <= 64u) { minR = R; break; }
+    const int topR = (V4 >= 65536u || minR > 16) ? maxR : (maxR < 16 ? maxR : 16);
+    const uint64_t want = B <= 16 ? 256 : 512;
+    for (int R = topR; R >= minR; R /= 2)
+        if ((uint64_t)B * parts(R) >= want) return {R, parts(R)};
+    return {minR, parts(minR)};
+}
+
+
+// Streaming geometry: workgroups of 256 threads; slices of 16384 tokens (16 float4 per thread), or
+// of 4096 tokens (4 float4) for calls of up to kStreamSmall tokens in rows of up to 262144, where a
+// shorter slice shortens the one wave of workgroups the whole pass consists of (longer rows would
+// be cut into more slices than a finishing workgroup handles quickly).
+constexpr int kStreamNT = 256;
+constexpr uint64_t kStreamSmall = 1ull << 22;
+constexpr uint32_t kListGrid = 256;            // workgroups of the launch for the rows handed on (they loop)
+static int stream_r(int32_t B, int32_t V) { return (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144 ? 4 : kStreamLongR; }
+static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+struct StreamLayout { size_t hdr, cum, shist, stash, need, end; };
+static StreamLayout stream_layout(int32_t B, size_t parts, size_t base)
+{
+    StreamLayout l;
+    l.hdr = align256(base);
+    l.cum = align256(l.hdr + parts * sizeof(PartHdr));
+    l.shist = align256(l.cum + parts * kSB * sizeof(uint32_t));
+    l.stash = align256(l.shist + parts * kSB * sizeof(uint64_t));
+    l.need = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
+    l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
+    return l;
+}
+// Bytes of per-slice data a workspace for (B, V) sets aside: enough for the long slices of (B, V)
+// itself and for the short slices of any call of at most B rows that takes them (at most
+// kStreamSmall tokens: fewer than kStreamSmall / 4096 + B slices), so that the size grows with
+// B and with V and a workspace for the largest B and V serves every smaller call.
+static size_t stream_bytes(int32_t B, int32_t V)
+{
+    const size_t longs = stream_layout(B, (size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader)).end;
+    size_t small_parts = (size_t)B * stream_parts(V, 4);
+    const size_t cap = (size_t)(kStreamSmall / 4096) + (size_t)B;
+    if (small_parts > cap) small_parts = cap;
+    const size_t shorts = stream_layout(B, small_parts, sizeof(WsHeader)).end;
+    return longs > shorts ? longs : shorts;
+}
+
+}  // namespace rs
+
+// The caller's routing state (see rapid_sampling.h).  word[0], word[1]: "most rows were handed on"
+// as last reported by a streaming call with / without a bounding top_k; word[2]: RS_ERR_DEVICE
+// once a kernel gave up a wait.  calls[]: calls routed away from the streaming path since.
+struct rs_policy {
+    int32_t *word;
+    uint32_t calls[2];
+};
+
+namespace rs {
+
+// The streaming path works when the kept set is small next to the row; a row for which it does
+// not is handed to the cluster kernel in a third launch, and a call whose rows mostly end that way
+// has wasted a pass.  With a bounding top_k that takes unusual rows (ties of thousands of tokens);
+// without one (nucleus sampling alone) it is simply a flat distribution, so such a call is an
+// attempt.  The launch for the rows handed on reports "most of them: yes/no" into a word of the
+// caller's rs_policy, one word for calls with a bounding top_k and one for calls without, and
+// this function looks at the word -- without waiting for anything; a stale value only delays the
+// switch -- before it chooses the path of the next call: after a call that handed most rows on,
+// calls of that kind go straight to the cluster kernel and one in 64 streams again.  Without a
+// policy, calls with a bounding top_k always stream and calls without never do.
+//
+// Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
+// kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
+// times faster for large ones); below that the single launch wins by up to a microsecond.
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3 };
+
+// Slice length of the one-launch path (float4 groups per thread), 0 when the call does not suit it.
+// Its workgroups hold their compute units until their row is finished, so a call pays twice once it
+// has more workgroups than the GPU holds at a time (256 CUs x 3, x 2 for the longest slices with
+// penalties: registers): the shortest slice that keeps the call within that is taken.  Calls of up
+// to kStreamSmall tokens may use any of the three lengths (the workspace has room for their short
+// slices), larger ones the long slices only.  `any_size` (forced by the caller): longest slices
+// whatever the number of workgroups.
+static int fused_r(int32_t B, int32_t V, bool pen, bool any_size)
+{
+    const bool small_call = (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144;
+    const int choices[3] = {4, 8, 16};
+    for (int i = small_call ? 0 : 2; i < 3; ++i) {
+        const int R = choices[i];
+        const uint32_t parts = stream_parts(V, R);
+        if (parts < 2u || parts > (uint32_t)kMaxParts) continue;
+        const uint64_t resident = 256u * (R == 16 && pen ? 2u : 3u);
+        if ((uint64_t)B * parts <= resident || (any_size && i == 2)) return R;
+    }
+    if (any_size && small_call && stream_parts(V, 4) >= 2u) return 4;
+    return 0;
+}
+
+static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pen, const rs_options *opt)
+{
+    const bool bounded = top_k <= kStreamK;
+    const int force = opt ? opt->path : RS_PATH_AUTO;
+    if (force == RS_PATH_FUSED) return fused_r(B, V, pen, true) ? kPathFused : kPathCluster;
+    // The one-launch path by default: calls with penalties whose kept set is bounded by top_k (the
+    // general kernel, the only other way with penalties, spends most of its time in exchanges).
+    if (force == RS_PATH_AUTO && pen && bounded && fused_r(B, V, pen, false)) return kPathFused;
+    if (pen) return kPathCluster;
+    if (force == RS_PATH_CLUSTER) return kPathCluster;
+    if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
+    if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
+    if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
+    if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // everything is kept: nothing a stash could hold
+    rs_policy *pol = opt ? opt->policy : nullptr;
+    if (!pol) return bounded ? kPathStream : kPathCluster;
+    const int yes = bounded ? kPathStream : kPathAttempt, kind = bounded ? 0 : 1;
+    const bool failing = *(volatile int32_t *)(pol->word + kind) != 0;
+    return (!failing || (++pol->calls[kind] & 63u) == 0u) ? yes : kPathCluster;
+}
+
+static hipError_t fill_zero(void *dst, size_t bytes, hipStream_t st)
+{
+    const size_t n16 = bytes / 16;
+    const uint32_t blocks = (uint32_t)(n16 / 256 < 1 ? 1 : n16 / 256 > 2048 ? 2048 : n16 / 256);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, st, (uint4 *)dst, n16,
+                       (unsigned char *)dst + n16 * 16, (uint32_t)(bytes - n16 * 16));
+    return hipGetLastError();
+}
+
+}  // namespace rs
+
+using namespace rs;
+
+extern "C" {
+
+int rs_version(void) { return 400; }
+
+const char *rs_error_string(int code)
+{
+    switch (code) {
+    case RS_OK:              return "ok";
+    case RS_ERR_VOCAB:       return "Vocabulary size must be multiple of 4, and no larger than 1048576";
+    case RS_ERR_BATCH:       return "B and T must be positive";
+    case RS_ERR_TEMPERATURE: return "Temperature outside range, expect [0.001, 1000]";
+    case RS_ERR_NULL:        return "a required pointer is NULL";
+    case RS_ERR_WORKSPACE:   return "workspace too small or not 256-byte aligned";
+    case RS_ERR_ALIGN:       return "rows of logits/penalties must be 16-byte aligned";
+    case RS_ERR_ARG:         return "top_k/top_p not normalised: need 1 <= top_k <= V and 0 < top_p <= 1";
+    case RS_ERR_LAUNCH:      return "HIP launch failed";
+    case RS_ERR_DEVICE:      return "a workgroup gave up waiting for its peers";
+    case RS_ERR_SCRATCH:     return "the call needs a larger workspace than the static scratch of rs_sample_static (RS_STATIC_SCRATCH_BYTES)";
+    default:                 return "unknown error";
+    }
+}
+
+int rs_normalize_args(double temperature, int64_t top_k, double top_p,
+                      int64_t B, int64_t T, int64_t V,
+                      float *log2e_inv_temp, int32_t *top_k_out, float *top_p_out)
+{
+    if (!log2e_inv_temp || !top_k_out || !top_p_out) return RS_ERR_NULL;
+    if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
+    if (!(B > 0 && T > 0)) return RS_ERR_BATCH;
+    if (!(temperature >= 0.001 && temperature <= 1000)) return RS_ERR_TEMPERATURE;
+    if (top_k <= 0 || top_k > V) top_k = V;
+    if (top_p < 0 || top_p > 1) top_p = 1;
+    if (top_p == 0) { top_k = 1; top_p = 1; }
+    *log2e_inv_temp = (float)(1.4426950408889634074 / temperature);
+    *top_k_out = (int32_t)top_k;
+    *top_p_out = (float)top_p;
+    return RS_OK;
+}
+
+int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes)
+{
+    if (!bytes) return RS_ERR_NULL;
+    if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
+    if (B <= 0) return RS_ERR_BATCH;
+    *bytes = stream_bytes(B, V) + (size_t)B * sizeof(RowCtl);
+    return RS_OK;
+}
+
+int rs_workspace_init(void *ws, size_t bytes, void *stream)
+{
+    if (!ws) return RS_ERR_NULL;
+    if (bytes < sizeof(WsHeader) || ((uintptr_t)ws & 255)) return RS_ERR_WORKSPACE;
+    return fill_zero(ws, bytes, (hipStream_t)stream) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+int rs_workspace_set_wait_limit(void *ws, uint32_t milliseconds, void *stream)
+{
+    if (!ws) return RS_ERR_NULL;
+    if ((uintptr_t)ws & 255) return RS_ERR_WORKSPACE;
+    if (milliseconds >= 40000u) return RS_ERR_ARG;
+    const uint32_t ticks = (uint32_t)((uint64_t)milliseconds * 100000ull >> 10);      // 100 MHz wall clock
+    hipLaunchKernelGGL(set_u32_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, &((WsHeader *)ws)->spin_ticks, ticks);
+    return hipGetLastError() == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+int rs_workspace_status(const void *ws, int32_t *status, void *stream)
+{
+    if (!ws || !status) return RS_ERR_NULL;
+    int32_t e = 0;
+    const WsHeader *h = (const WsHeader *)ws;
+    if (hipMemcpyAsync(&e, &h->error, sizeof e, hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
+    *status = e;
+    return RS_OK;
+}
+
+int rs_policy_create(rs_policy **out)
+{
+    if (!out) return RS_ERR_NULL;
+    *out = nullptr;
+    rs_policy *pol = new (std::nothrow) rs_policy;
+    if (!pol) return RS_ERR_LAUNCH;
+    pol->word = nullptr; pol->calls[0] = 0; pol->calls[1] = 0;
+    if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
+        delete pol;
+        return RS_ERR_LAUNCH;
+    }
+    for (int i = 0; i < 16; ++i) pol->word[i] = 0;
+    *out = pol;
+    return RS_OK;
+}
+
+void rs_policy_destroy(rs_policy *pol)
+{
+    if (!pol) return;
+    if (pol->word) (void)hipHostFree(pol->word);
+    delete pol;
+}
+
+int rs_policy_state(const rs_policy *pol, int32_t *state)
+{
+    if (!pol || !state) return RS_ERR_NULL;
+    const volatile int32_t *w = pol->word;
+    *state = (w[1] != 0 ? 1 : 0) | (w[0] != 0 ? 2 : 0);
+    return RS_OK;
+}
+
+int rs_policy_error(rs_policy *pol, int32_t *error, int32_t clear)
+{
+    if (!pol || !error) return RS_ERR_NULL;
+    volatile int32_t *w = pol->word;
+    *error = w[2];
+    if (clear) w[2] = 0;
+    return RS_OK;
+}
+
+int rs_philox_init(void *state, uint64_t seed, int32_t B, void *stream)
+{
+    if (!state) return RS_ERR_NULL;
+    if (B <= 0) return RS_ERR_BATCH;
+    hipLaunchKernelGGL(philox_init_kernel, dim3((B + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       (uint32_t *)state, seed, B);
+    return hipGetLastError() == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+int rs_sample(const float *logits, int64_t row_stride, float *penalties, int32_t *out,
+              void *rng_state, const float *injected_u, int32_t B, int32_t V,
+              float presence, float repetition, float decay,
+              float log2e_inv_temp, int32_t top_k, float top_p,
+              void *workspace, size_t workspace_bytes,
+              rs_row_diag *diag, uint32_t *e_bits, void *stream)
+{
+    return rs_sample_ex(logits, RS_DTYPE_F32, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                        repetition, decay, log2e_inv_temp, top_k, top_p, workspace, workspace_bytes, diag, e_bits,
+                        nullptr, stream);
+}
+
+int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                    void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                    float presence, float repetition, float decay,
+                    float log2e_inv_temp, int32_t top_k, float top_p,
+                    void *workspace, size_t workspace_bytes,
+                    rs_row_diag *diag, uint32_t *e_bits, void *stream)
+{
+    return rs_sample_ex(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                        repetition, decay, log2e_inv_temp, top_k, top_p, workspace, workspace_bytes, diag, e_bits,
+                        nullptr, stream);
+}
+
+int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                 void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                 float presence, float repetition, float decay,
+                 float log2e_inv_temp, int32_t top_k, float top_p,
+                 void *workspace, size_t workspace_bytes,
+                 rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
+{
+    if (!logits || !out || !workspace || (!rng_state && !injected_u)) return RS_ERR_NULL;
+    if (logits_dtype != RS_DTYPE_F32 && logits_dtype != RS_DTYPE_BF16 && logits_dtype != RS_DTYPE_F16) return RS_ERR_ARG;
+    if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
+    if (B <= 0) return RS_ERR_BATCH;
+    if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
+    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_FUSED || opt->slice_r < 0)) return RS_ERR_ARG;
+    if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
+        return RS_ERR_ALIGN;
+    size_t need = 0;
+    rs_workspace_bytes(B, V, &need);
+    if (workspace_bytes < need || ((uintptr_t)workspace & 255)) return RS_ERR_WORKSPACE;
+
+    const bool pen = penalties != nullptr;
+    const Geometry g = choose_geometry(B, V, pen, opt ? opt->slice_r : 0);
+    Params p;
+    p.logits = logits; p.dtype = logits_dtype; p.penalties = penalties; p.out = out;
+    p.rng = (uint32_t *)rng_state; p.inj_u = injected_u; p.diag = diag; p.e_bits = e_bits;
+    p.hdr = (WsHeader *)workspace;
+    p.ctl_end = (RowCtl *)((char *)workspace + (workspace_bytes & ~(size_t)255));
+    p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
+    p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
+    p.top_k = top_k; p.top_p = top_p;
+    p.need = nullptr; p.stash_k = (uint32_t)top_k; p.report = 0;
+    p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
+    dim3 grid((uint32_t)B * g.G);
+    const int path = choose_path(B, V, top_k, top_p, pen, opt);
+    if (path != kPathCluster) {
+        const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V);
+        StreamView v;
+        v.G = stream_parts(V, sr);
+        const StreamLayout l = stream_layout(B, (size_t)B * v.G, sizeof(WsHeader));
+        char *w = (char *)workspace;
+        v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
+        v.shist = (uint64_t *)(w + l.shist);
+        v.need = (uint32_t *)(w + l.need);
+        // without a bounding top_k the stashes are sized as for top_k = kStreamK: enough for a nucleus
+        // of up to about a thousand tokens
+        const uint32_t kk = min((uint32_t)top_k, (uint32_t)kStreamK);
+        p.stash_k = min(kk, max(32u, 8u * kk / v.G));            // eight times a slice's share of the row's top_k
+        hipStream_t st = (hipStream_t)stream;
+        // The finishing workgroup's list: twice what a well-behaved row needs (its top_k tokens and
+        // a boundary bin, or every stash whole), as a power of two; a row that needs more is handed
+        // on.  Kept small where it can be: the list is LDS, and LDS decides how many rows finish at once.
+        const uint32_t whole = v.G * (p.stash_k + 64u);            // every stash whole; of no use beyond kFinCap
+        const uint32_t est = 2u * max(kk + 512u, whole <= (uint32_t)kFinCap ? whole : 0u);
+        v.list_cap = 2048u;
+        while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
+        // the one-launch path keeps a list of 2048 tokens in LDS it holds anyway; a longer one costs every
+        // workgroup of the call dynamic LDS (fewer workgroups per CU), so it is only taken when even a
+        // well-behaved row would not fit 2048 (a row that then needs more falls back inside the kernel)
+        if (path == kPathFused && est / 2u <= 2048u) v.list_cap = 2048u;
+        p.report = path == kPathAttempt ? 1u : 0u;
+        const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
+        if (path == kPathFused)
+            return launch_fused(sr, pen, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+        if (launch_stream(sr, logits_dtype, (uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
+        p.need = v.need;               // the cluster kernel follows for the rows the finish left over
+        // Workgroups for the rows handed on.  Few rows are expected when top_k bounds the kept set: a
+        // small grid whose workgroups take tickets until the list is exhausted.  After an attempt it
+        // may be all of them: one workgroup per slice of every row, as in the cluster kernel; those
+        // beyond the list leave at once.
+        if (path == kPathStream && grid.x > kListGrid) grid.x = kListGrid / g.G * g.G > 0 ? kListGrid / g.G * g.G : g.G;
+    }
+    const hipError_t e = p.need ? launch_list(g.R, grid, (hipStream_t)stream, p, path == kPathAttempt)
+                              : launch_sample(pen, g.R, grid, (hipStream_t)stream, p);
+    return e == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                     void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                     float presence, float repetition, float decay,
+                     float log2e_inv_temp, int32_t top_k, float top_p,
+                     rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
+{
+    size_t need = 0;
+    const int rc = rs_workspace_bytes(B, V, &need);
+    if (rc != RS_OK) return rc;
+    if (need > (size_t)RS_STATIC_SCRATCH_BYTES) return RS_ERR_SCRATCH;
+    // every GPU holds its own copy of the array at its own address: looked up once per device
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void *> base[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return RS_ERR_LAUNCH;
+    void *ws = base[dev].load(std::memory_order_acquire);
+    if (!ws) {
+        if (hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch)) != hipSuccess || !ws) return RS_ERR_LAUNCH;
+        base[dev].store(ws, std::memory_order_release);
+    }
+    // The array keeps what the last call left.  A call leaves it clean unless a wait gave up; the launch
+    // header and this call's row records are cleared all the same, by a kernel (not a memset node: the
+    // call may be under capture), so that every call starts from zero whatever came before.
+    const size_t rec_bytes = (size_t)B * sizeof(RowCtl);
+    char *recs = (char *)ws + (size_t)RS_STATIC_SCRATCH_BYTES - rec_bytes;
+    const size_t n16 = rec_bytes / 16;
+    const uint32_t blocks = (uint32_t)(n16 / 1024 < 1 ? 1 : n16 / 1024 > 1024 ? 1024 : n16 / 1024);
+    hipLaunchKernelGGL(clear_records_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint4 *)ws, (uint4 *)recs, n16);
+    if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
+    return rs_sample_ex(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
+                        repetition, decay, log2e_inv_temp, top_k, top_p, ws, (size_t)RS_STATIC_SCRATCH_BYTES, diag,
+                        e_bits, opt, stream);
+}
+
+int rs_floor_read(const float *logits, int64_t row_stride, int32_t *out, int32_t B, int32_t V, int32_t variant, void *stream)
+{
+    if (!logits || !out) return RS_ERR_NULL;
+    if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
+    if (B <= 0) return RS_ERR_BATCH;
+    if (variant < 0 || variant > 3) return RS_ERR_ARG;
+    const uint32_t V4 = (uint32_t)V / 4;
+    const bool once = (variant & 1) != 0;
+    hipStream_t st = (hipStream_t)stream;
+#define RS_FLOOR(Rv) do { const uint32_t G = (V4 + kThreads * Rv - 1) / (kThreads * Rv); const dim3 grid((uint32_t)B * G);                          \
+        if (once) hipLaunchKernelGGL((floor_kernel<Rv, true>), grid, dim3(kThreads), 0, st, logits, row_stride, out, V, G);                     \
+        else hipLaunchKernelGGL((floor_kernel<Rv, false>), grid, dim3(kThreads), 0, st, logits, row_stride, out, V, G); } while (0)
+    if (variant >= 2) {
+        // the streaming pass's own geometry
+        if (stream_r(B, V) == 4) RS_FLOOR(4); else RS_FLOOR(kStreamLongR);
+    } else {
+        switch (choose_geometry(B, V, false, 0).R) {
+        case 1:  RS_FLOOR(1); break;
+        case 2:  RS_FLOOR(2); break;
+        case 4:  RS_FLOOR(4); break;
+        case 8:  RS_FLOOR(8); break;
+        case 16: RS_FLOOR(16); break;
+        default: RS_FLOOR(32); break;
+        }
+    }
+#undef RS_FLOOR
+    return hipGetLastError() == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -1,0 +1,42 @@
+// Instantiations and launchers of the streaming kernels.
+#include "rs_stream.h"
+
+namespace rs {
+
+constexpr int kStreamNT = 256;
+
+hipError_t launch_stream(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
+                         const StreamView &v)
+{
+    const dim3 sgrid(B * v.G), sblock(kStreamNT);
+    if (slice_r == 4) {
+        if (dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_F32>), sgrid, sblock, 0, st, p, v);
+        else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);
+        else hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_F16>), sgrid, sblock, 0, st, p, v);
+        hipLaunchKernelGGL((finish_kernel<12>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v);
+    } else {
+        if (dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<kStreamLongR, kStreamNT, RS_DTYPE_F32>), sgrid, sblock, 0, st, p, v);
+        else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<kStreamLongR, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);
+        else hipLaunchKernelGGL((stream_kernel<kStreamLongR, kStreamNT, RS_DTYPE_F16>), sgrid, sblock, 0, st, p, v);
+        hipLaunchKernelGGL((finish_kernel<kStreamLongLog2>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_fused(int slice_r, bool pen, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
+                        const StreamView &v)
+{
+    const dim3 grid(B * v.G), block(kThreads);
+    const size_t dyn = v.list_cap <= 2048u ? 0 : finish_lds_bytes;      // a short list lives in static LDS
+#define RS_FUSED(Rv) do { if (pen) hipLaunchKernelGGL((fused_kernel<Rv, true>), grid, block, dyn, st, p, v);          \
+                          else hipLaunchKernelGGL((fused_kernel<Rv, false>), grid, block, dyn, st, p, v); } while (0)
+    switch (slice_r) {
+    case 4:  RS_FUSED(4); break;
+    case 8:  RS_FUSED(8); break;
+    default: RS_FUSED(16); break;
+    }
+#undef RS_FUSED
+    return hipGetLastError();
+}
+
+}  // namespace rs

@@ -332,6 +332,18 @@ int64_t workspace_status(std::optional<int64_t> device)
     return st;
 }
 
+// Routing state of the current stream's workspace (rs_policy_state): bit 0 set: calls without a
+// bounding top_k currently take the general kernel, bit 1 set: so do calls with one.  -1: no workspace yet.
+int64_t policy_state(std::optional<int64_t> device)
+{
+    const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
+    auto like = at::empty({1}, at::TensorOptions().dtype(at::kChar).device(dev));
+    Entry &e = entry_for((int)dev.index(), current_stream(like));
+    int32_t st = -1;
+    if (e.policy) rs_policy_state(e.policy, &st);
+    return st;
+}
+
 // Shortens (milliseconds > 0) or restores (0) the bound of the kernels' waits on the current
 // stream's workspace.  For tests of the error path.
 void set_wait_limit(int64_t milliseconds, std::optional<int64_t> device)
@@ -352,7 +364,8 @@ void force_path(const std::string &name)
     else if (name == "cluster") g_forced_path = RS_PATH_CLUSTER;
     else if (name == "stream") g_forced_path = RS_PATH_STREAM;
     else if (name == "attempt") g_forced_path = RS_PATH_ATTEMPT;
-    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt");
+    else if (name == "fused") g_forced_path = RS_PATH_FUSED;
+    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused");
 }
 
 // The workspace tensor of the current stream (tests poison it to force the error path).
@@ -366,14 +379,14 @@ at::Tensor debug_workspace(std::optional<int64_t> device)
 }
 
 // Launch-plus-one-read floor kernel on the logits' grid (measurement aid).
-at::Tensor floor_read(at::Tensor &logits)
+at::Tensor floor_read(at::Tensor &logits, int64_t variant)
 {
     const Shape s = read_logits(logits, std::nullopt, false);
     c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
     // not cleared: the kernel max-combines into it, and a second launch to zero it would be timed along
     auto out = at::empty({s.B}, at::TensorOptions().dtype(at::kInt).device(logits.device()));
     const int rc = rs_floor_read(static_cast<const float *>(s.first_row), s.row_stride, out.data_ptr<int32_t>(), (int32_t)s.B, (int32_t)s.V,
-                                 current_stream(logits));
+                                 (int32_t)variant, current_stream(logits));
     if (rc != RS_OK) throw std::runtime_error(std::string("rapid_sampling: ") + rs_error_string(rc));
     return out;
 }
@@ -393,9 +406,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           py::arg("presence_penalty"), py::arg("repetition_penalty"), py::arg("penalty_decay"),
           py::arg("temperature"), py::arg("top_k"), py::arg("top_p"), py::kw_only(),
           py::arg("uniforms") = py::none(), py::arg("accept_half") = false);
-    m.def("floor_read", &floor_read, py::arg("logits"));
+    m.def("floor_read", &floor_read, py::arg("logits"), py::arg("variant") = 1);
     m.def("reserve_workspace", &reserve_workspace, py::arg("B"), py::arg("V"), py::arg("device") = py::none());
     m.def("workspace_status", &workspace_status, py::arg("device") = py::none());
+    m.def("policy_state", &policy_state, py::arg("device") = py::none());
     m.def("force_path", &force_path, py::arg("name"));
     m.def("debug_workspace", &debug_workspace, py::arg("device") = py::none());
     m.def("set_wait_limit", &set_wait_limit, py::arg("milliseconds"), py::arg("device") = py::none());

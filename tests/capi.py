@@ -17,7 +17,7 @@ DIAG_DTYPE = np.dtype([
     ("S", "<u8", (2,)), ("r", "<u8", (2,)),
 ])
 
-PATHS = {None: 0, "auto": 0, "cluster": 1, "stream": 2, "optimistic": 3, "attempt": 3}
+PATHS = {None: 0, "auto": 0, "cluster": 1, "stream": 2, "optimistic": 3, "attempt": 3, "fused": 4}
 
 
 class Options(C.Structure):
@@ -72,7 +72,7 @@ def lib():
         L.rs_sample_static.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
                                        vp, vp, C.POINTER(Options), vp]
         L.rs_floor_read.restype = C.c_int
-        L.rs_floor_read.argtypes = [vp, i64, vp, i32, i32, vp]
+        L.rs_floor_read.argtypes = [vp, i64, vp, i32, i32, i32, vp]
         _lib = L
     return _lib
 

@@ -71,15 +71,21 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     res2 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen2, presence=presence, repetition=repetition,
                       decay=decay, force_r=force_r)
     _check(res2, ref_out, ref_diag, what + " (second call)")
-    if pen_np is None:
-        # the general kernel alone, the wait-free streaming path (taken for top_k <= 1024; rows it cannot
-        # finish go on to the general kernel), the same attempted whatever top_k is (both with the e of
-        # every token: the kept set on that path), then the general kernel again on the workspace these
-        # leave behind
-        for path in ("cluster", "stream", "optimistic", "cluster"):
-            res3 = smp.sample(lg, c, k, p, uniforms=u, path=path, force_r=force_r, want_e=path != "cluster")
-            _check(res3, ref_out, ref_diag, what + " (path %s)" % path, ref_e if path != "cluster" else None)
-            assert smp.status() == 0
+    # Every way through the library on this one workspace: the general kernel alone, the wait-free
+    # streaming path (taken for top_k <= 1024; rows it cannot finish go on to the general kernel), the
+    # same attempted whatever top_k is, the one-launch path (streaming pass and finish in one kernel,
+    # falling back inside the kernel), then the general kernel again on the workspace these leave
+    # behind.  All but the general kernel also return the e of every token: the kept set on that path.
+    # With penalties: the one-launch path and the general kernel.
+    paths = ("cluster", "stream", "optimistic", "fused", "cluster") if pen_np is None else ("fused", "cluster", "fused")
+    for path in paths:
+        pen3 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
+        res3 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen3, presence=presence, repetition=repetition, decay=decay,
+                          path=path, force_r=force_r, want_e=path != "cluster")
+        _check(res3, ref_out, ref_diag, what + " (path %s)" % path, ref_e if path != "cluster" else None)
+        assert smp.status() == 0
+        if pen3 is not None:
+            assert np.array_equal(pen3.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32)), what + ": penalties, path " + path
     return res, ref_diag
 
 
@@ -739,7 +745,7 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     torch = torch_cuda
     import ctypes as C
     from tests import capi
-    B, V = 16, 65536
+    B, V = 600, 65536                                    # too many slices for the one-launch path: three launches, routed
     peaked = H.logits_normal(B, V, 3.0, seed=90)
     flat = H.logits_uniform(B, V, seed=91)
     rc, c, k, p = capi.normalize(1.0, -1, 0.3, V, B, 1)
@@ -896,7 +902,9 @@ def test_python_module_raises_after_a_failed_call_and_recovers(torch_cuda, oracl
     lg, u = torch.from_numpy(lg_np).cuda(), torch.from_numpy(u_np).cuda()
     st = sample.setup_rand(1, B)
     side = torch.cuda.Stream()                       # a stream of its own: its workspace is this test's alone
-    with torch.cuda.stream(side):
+    sample._sample.force_path("cluster")             # the kernel whose workgroups wait for counts that add up
+    try:
+      with torch.cuda.stream(side):
         out = sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)
         assert np.array_equal(out.cpu().numpy(), ref_out) and sample.workspace_status() == 0
         for check in ("next call", "status"):
@@ -915,6 +923,8 @@ def test_python_module_raises_after_a_failed_call_and_recovers(torch_cuda, oracl
             out = sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)
             assert np.array_equal(out.cpu().numpy(), ref_out), check
             assert sample.workspace_status() == 0
+    finally:
+        sample._sample.force_path("auto")
     side.synchronize()
 
 
