@@ -69,8 +69,12 @@ __global__ void __launch_bounds__(kThreads) floor_kernel(const float *logits, in
 #pragma unroll
     for (int j = 0; j < R; ++j)
         m = fmaxf(m, fmaxf(fmaxf(__uint_as_float(v[j].x), __uint_as_float(v[j].y)), fmaxf(__uint_as_float(v[j].z), __uint_as_float(v[j].w))));
-    uint32_t k = wave_max_u32(fkey(m));
-    if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<uint32_t *>(out + row), k);
+    // one combine per workgroup: contended atomics on a few addresses would be timed instead of the read
+    __shared__ uint32_t wmax[kWaves];
+    const uint32_t k = wave_max_u32(fkey(m));
+    if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = k;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(reinterpret_cast<uint32_t *>(out + row), max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
 }
 
 __global__ void philox_init_kernel(uint32_t *state, uint64_t seed, int32_t B)
@@ -197,6 +201,7 @@ namespace rs {
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
 enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3 };
+constexpr uint64_t kPenStreamMin = 1ull << 23;
 
 // Slice length of the one-launch path (float4 groups per thread), 0 when the call does not suit it.
 // Its workgroups hold their compute units until their row is finished, so a call pays twice once it
@@ -228,17 +233,26 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     // The one-launch path by default: calls with penalties whose kept set is bounded by top_k (the
     // general kernel, the only other way with penalties, spends most of its time in exchanges).
     if (force == RS_PATH_AUTO && pen && bounded && fused_r(B, V, pen, false)) return kPathFused;
+    // Larger calls with penalties: the streaming pass with a pass over the penalties behind it, from
+    // kPenStreamMin tokens on (measured crossover with the general kernel), long slices only.
+    rs_policy *pol = opt ? opt->policy : nullptr;
+    // after a call of this kind that handed most rows on: straight to the general kernel, one in 64 tries again
+    auto routed_away = [&](int kind) {
+        if (!pol || *(volatile int32_t *)(pol->word + kind) == 0) return false;
+        return (++pol->calls[kind] & 63u) != 0u;
+    };
+    if (pen && bounded && stream_r(B, V) == kStreamLongR && stream_parts(V, kStreamLongR) >= 2u) {
+        if (force == RS_PATH_STREAM || force == RS_PATH_ATTEMPT) return kPathStream;
+        if (force == RS_PATH_AUTO && (uint64_t)B * (uint64_t)V >= kPenStreamMin && !routed_away(0)) return kPathStream;
+    }
     if (pen) return kPathCluster;
     if (force == RS_PATH_CLUSTER) return kPathCluster;
     if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
     if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
     if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
     if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // everything is kept: nothing a stash could hold
-    rs_policy *pol = opt ? opt->policy : nullptr;
     if (!pol) return bounded ? kPathStream : kPathCluster;
-    const int yes = bounded ? kPathStream : kPathAttempt, kind = bounded ? 0 : 1;
-    const bool failing = *(volatile int32_t *)(pol->word + kind) != 0;
-    return (!failing || (++pol->calls[kind] & 63u) == 0u) ? yes : kPathCluster;
+    return routed_away(bounded ? 0 : 1) ? kPathCluster : bounded ? kPathStream : kPathAttempt;
 }
 
 static hipError_t fill_zero(void *dst, size_t bytes, hipStream_t st)
@@ -434,6 +448,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.top_k = top_k; p.top_p = top_p;
     p.need = nullptr; p.stash_k = (uint32_t)top_k; p.report = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
+    p.defer_pen = 0;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path != kPathCluster) {
@@ -465,6 +480,17 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (path == kPathFused)
             return launch_fused(sr, pen, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+        if (pen) {
+            // penalties: read by the streaming pass and by the kernel for the rows handed on, rewritten
+            // by one pass over them at the end
+            p.defer_pen = 1;
+            if (launch_stream_pen((uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
+            p.need = v.need;
+            p.G = stream_parts(V, 16);
+            const uint32_t lgrid = kListGrid / p.G * p.G > 0 ? kListGrid / p.G * p.G : p.G;
+            if (launch_list_pen16(dim3(lgrid), st, p) != hipSuccess) return RS_ERR_LAUNCH;
+            return launch_penalty_pass(st, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+        }
         if (launch_stream(sr, logits_dtype, (uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
         p.need = v.need;               // the cluster kernel follows for the rows the finish left over
         // Workgroups for the rows handed on.  Few rows are expected when top_k bounds the kept set: a

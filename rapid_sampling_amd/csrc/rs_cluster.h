@@ -517,13 +517,13 @@ __device__ __forceinline__ bool slice_finish(const Params &p, Lds &s, Slice<R, P
             const int32_t idx = (int32_t)((base4 + (uint32_t)jstar * kThreads) * 4 + (uint32_t)kk);
             p.out[row] = idx;
             if (p.diag) p.diag[row].index = idx;
-            if (PEN && G > 1) a_store(&rc->index_p1, (uint32_t)idx + 1u);
+            if (PEN && !p.defer_pen && G > 1) a_store(&rc->index_p1, (uint32_t)idx + 1u);
             if (PEN) s.bc32[7] = (uint32_t)idx;
         }
     }
 
     // ---- 7. penalties: decay and one-hot add, from registers ---------------
-    if (PEN) {
+    if (PEN && !p.defer_pen) {
         __syncthreads();
         if (G > 1) {
             if (tid == 0) {
@@ -635,8 +635,8 @@ __device__ __forceinline__ void report_streaming(const Params &p, uint32_t hande
 
 // The launch that follows the streaming pass: workgroups work through the
 // rows on its list, taking tickets until the list is exhausted.
-template <int R>
-__global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list_kernel(const Params p)
+template <int R, bool PEN = false>
+__global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_list_kernel(const Params p)
 {
     __shared__ Lds s;
     const uint32_t G = p.G;
@@ -653,7 +653,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list
         const uint32_t ticket = s.bc32[0];
         const uint32_t slot = ticket / G;
         if (slot >= a_load(&p.hdr->n_need)) break;
-        if (!sample_slice<R, false>(p, s, p.need[slot], ticket - slot * G)) return;
+        if (!sample_slice<R, PEN>(p, s, p.need[slot], ticket - slot * G)) return;
     }
     leave_launch(p.hdr);
 }

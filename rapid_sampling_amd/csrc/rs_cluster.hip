@@ -44,6 +44,13 @@ hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p, bool o
 }
 
 
+// rows the streaming pass with penalties handed on: penalties enter x, their update is left to the pass that follows
+hipError_t launch_list_pen16(dim3 grid, hipStream_t st, const Params &p)
+{
+    hipLaunchKernelGGL((sample_list_kernel<16, true>), grid, dim3(kThreads), 0, st, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_sample(bool pen, int R, dim3 grid, hipStream_t st, const Params &p)
 {
     return pen ? launch_sample_t<true>(R, grid, st, p) : launch_sample_t<false>(R, grid, st, p);

@@ -767,6 +767,56 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
 
 
 
+// The streaming pass for calls with penalties too large for the one-launch path: logits and penalties
+// are read once, x = sf((sf(l) - pen) * c) as in the cluster kernel, everything after that is the
+// streaming pass.  The penalties are not rewritten here (the sampled token is not known yet):
+// penalty_pass_kernel does that once every row has its token -- 16 bytes per token in all instead
+// of the 12 a single pass would move, at several times the cluster kernel's rate.
+template <int R>
+__global__ void __launch_bounds__(kThreads, 2) stream_pen_kernel(const Params p, const StreamView v)
+{
+    constexpr int kRep = stream_copies<R>();
+    __shared__ LdsA<kRep> s;
+    const uint32_t G = v.G;
+    const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
+    Slice<R, true> sl;
+    slice_setup(p, sl, row, part, G);
+    const float lmax = slice_load(p, sl);
+    if (blockIdx.x == 0 && threadIdx.x == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
+    slice_count_and_stash<R, kThreads, kRep, false>(p, v, s, sl.eb, lmax, row, part, sl.base4, sl.nv);
+}
+
+// pen <- fma(pen, decay, onehot * (pen == 0 ? presence : repetition)), the switch on the value before
+// the decay (reference: sampling.cu:427-437), for every row from its sampled token in p.out.
+__global__ void __launch_bounds__(kThreads) penalty_pass_kernel(const Params p, uint32_t groups_per_row)
+{
+    constexpr int kPer = 8;                              // float4 groups per thread
+    const uint32_t row = blockIdx.x / groups_per_row, part = blockIdx.x - row * groups_per_row;
+    const uint32_t V4 = (uint32_t)p.V >> 2;
+    const uint32_t idx = (uint32_t)p.out[row];
+    float4 *pn4 = reinterpret_cast<float4 *>(p.penalties + (int64_t)row * p.V);
+    const uint32_t base4 = part * (uint32_t)(kThreads * kPer) + threadIdx.x;
+    float4 q[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const uint32_t i4 = base4 + (uint32_t)j * kThreads;
+        if (i4 < V4) q[j] = pn4[i4];
+    }
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const uint32_t i4 = base4 + (uint32_t)j * kThreads;
+        if (i4 < V4) {
+            float4 w = q[j];
+            const uint32_t e0 = i4 * 4;
+            w.x = __builtin_fmaf(w.x, p.decay, (e0 + 0 != idx) ? 0.0f : (w.x == 0.0f ? p.presence : p.repetition));
+            w.y = __builtin_fmaf(w.y, p.decay, (e0 + 1 != idx) ? 0.0f : (w.y == 0.0f ? p.presence : p.repetition));
+            w.z = __builtin_fmaf(w.z, p.decay, (e0 + 2 != idx) ? 0.0f : (w.z == 0.0f ? p.presence : p.repetition));
+            w.w = __builtin_fmaf(w.w, p.decay, (e0 + 3 != idx) ? 0.0f : (w.w == 0.0f ? p.presence : p.repetition));
+            pn4[i4] = w;
+        }
+    }
+}
+
 // ------------------------------------------------------------ one-launch path --
 // The streaming pass and the finish in ONE launch, for calls small enough that a second and a third
 // launch (and the cold start of the finishing workgroup) cost as much as the work itself, and for

@@ -23,6 +23,20 @@ hipError_t launch_stream(int slice_r, int32_t dtype, uint32_t B, size_t finish_l
     return hipGetLastError();
 }
 
+hipError_t launch_stream_pen(uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v)
+{
+    hipLaunchKernelGGL((stream_pen_kernel<kStreamLongR>), dim3(B * v.G), dim3(kThreads), 0, st, p, v);
+    hipLaunchKernelGGL((finish_kernel<kStreamLongLog2>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v);
+    return hipGetLastError();
+}
+
+hipError_t launch_penalty_pass(hipStream_t st, const Params &p)
+{
+    const uint32_t V4 = (uint32_t)p.V / 4, groups = (V4 + kThreads * 8 - 1) / (kThreads * 8);
+    hipLaunchKernelGGL(penalty_pass_kernel, dim3((uint32_t)p.B * groups), dim3(kThreads), 0, st, p, groups);
+    return hipGetLastError();
+}
+
 hipError_t launch_fused(int slice_r, bool pen, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
                         const StreamView &v)
 {

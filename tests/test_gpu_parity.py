@@ -77,7 +77,7 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     # falling back inside the kernel), then the general kernel again on the workspace these leave
     # behind.  All but the general kernel also return the e of every token: the kept set on that path.
     # With penalties: the one-launch path and the general kernel.
-    paths = ("cluster", "stream", "optimistic", "fused", "cluster") if pen_np is None else ("fused", "cluster", "fused")
+    paths = ("cluster", "stream", "optimistic", "fused", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
     for path in paths:
         pen3 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
         res3 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen3, presence=presence, repetition=repetition, decay=decay,
@@ -614,6 +614,37 @@ def test_c4_penalty_chain(torch_cuda, oracle, steps):
     rel = np.abs(got - pen_ref) / np.maximum(np.abs(pen_ref), 1e-30)
     assert rel.max() <= 1e-6
     assert smp.status() == 0
+
+
+@pytest.mark.parametrize("B,V,steps", [(96, 152064, 3), (128, 1048576, 2)])
+def test_penalties_at_scale_streaming_pass(torch_cuda, oracle, B, V, steps):
+    """Calls with penalties too large for the one-launch path (more workgroups than the GPU holds at once)
+    take the streaming pass over logits and penalties, the finish, and one pass over the penalties that
+    applies decay and the one-hot add: chained steps, tokens, diagnostics and penalties bit for bit
+    against the oracle; the general kernel on the same inputs beside it."""
+    torch = torch_cuda
+    from tests import capi
+    lg_np = H.logits_normal(B, V, 1.5, seed=140)
+    pen_ref = H.penalties_sparse(B, V, seed=141)
+    rc, c, k, p = capi.normalize(0.8, 50, 0.9, V, B, 1)
+    smp = capi.Sampler(B, V)
+    lg = torch.from_numpy(lg_np).cuda()
+    pen = torch.from_numpy(pen_ref.copy()).cuda()
+    for step in range(steps):
+        u_np = H.uniforms(B, 500 + step)
+        u = torch.from_numpy(u_np).cuda()
+        pen_c = pen.clone()
+        ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np, penalties=pen_ref,
+                                                presence=0.1, repetition=0.2, decay=0.95)
+        print("penalties at scale: step", step, B, V, flush=True)
+        res = smp.sample(lg, c, k, p, uniforms=u, penalties=pen, presence=0.1, repetition=0.2, decay=0.95)
+        _check(res, ref_out, ref_diag, "streaming with penalties, step %d" % step)
+        assert (res["diag"]["rounds"] == 0).all()                      # finished by the streaming path
+        assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32)), step
+        res_c = smp.sample(lg, c, k, p, uniforms=u, penalties=pen_c, presence=0.1, repetition=0.2, decay=0.95, path="cluster")
+        _check(res_c, ref_out, ref_diag, "general kernel, step %d" % step)
+        assert torch.equal(pen_c.view(torch.int32), pen.view(torch.int32))
+        assert smp.status() == 0
 
 
 def test_philox_stream_matches_oracle(torch_cuda, oracle):
