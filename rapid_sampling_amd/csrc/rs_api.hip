@@ -144,20 +144,18 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
 // be cut into more slices than a finishing workgroup handles quickly).
 constexpr int kStreamNT = 256;
 constexpr uint64_t kStreamSmall = 1ull << 22;
-constexpr uint32_t kListGrid = 256;            // workgroups of the launch for the rows handed on (they loop)
 static int stream_r(int32_t B, int32_t V) { return (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144 ? 4 : kStreamLongR; }
 static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-struct StreamLayout { size_t hdr, cum, shist, stash, need, end; };
-static StreamLayout stream_layout(int32_t B, size_t parts, size_t base)
+struct StreamLayout { size_t hdr, cum, shist, stash, end; };
+static StreamLayout stream_layout(size_t parts, size_t base)
 {
     StreamLayout l;
     l.hdr = align256(base);
     l.cum = align256(l.hdr + parts * sizeof(PartHdr));
     l.shist = align256(l.cum + parts * kSB * sizeof(uint32_t));
     l.stash = align256(l.shist + parts * kSB * sizeof(uint64_t));
-    l.need = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
-    l.end = align256(l.need + (size_t)B * sizeof(uint32_t));
+    l.end = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
     return l;
 }
 // Bytes of per-slice data a workspace for (B, V) sets aside: enough for the long slices of (B, V)
@@ -166,11 +164,11 @@ static StreamLayout stream_layout(int32_t B, size_t parts, size_t base)
 // B and with V and a workspace for the largest B and V serves every smaller call.
 static size_t stream_bytes(int32_t B, int32_t V)
 {
-    const size_t longs = stream_layout(B, (size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader)).end;
+    const size_t longs = stream_layout((size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader)).end;
     size_t small_parts = (size_t)B * stream_parts(V, 4);
     const size_t cap = (size_t)(kStreamSmall / 4096) + (size_t)B;
     if (small_parts > cap) small_parts = cap;
-    const size_t shorts = stream_layout(B, small_parts, sizeof(WsHeader)).end;
+    const size_t shorts = stream_layout(small_parts, sizeof(WsHeader)).end;
     return longs > shorts ? longs : shorts;
 }
 
@@ -446,7 +444,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
-    p.need = nullptr; p.stash_k = (uint32_t)top_k; p.report = 0;
+    p.stash_k = (uint32_t)top_k; p.report = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
     p.defer_pen = 0;
     dim3 grid((uint32_t)B * g.G);
@@ -455,11 +453,10 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V);
         StreamView v;
         v.G = stream_parts(V, sr);
-        const StreamLayout l = stream_layout(B, (size_t)B * v.G, sizeof(WsHeader));
+        const StreamLayout l = stream_layout((size_t)B * v.G, sizeof(WsHeader));
         char *w = (char *)workspace;
         v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.shist = (uint64_t *)(w + l.shist);
-        v.need = (uint32_t *)(w + l.need);
         // without a bounding top_k the stashes are sized as for top_k = kStreamK: enough for a nucleus
         // of up to about a thousand tokens
         const uint32_t kk = min((uint32_t)top_k, (uint32_t)kStreamK);
@@ -481,27 +478,15 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         if (path == kPathFused)
             return launch_fused(sr, pen, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         if (pen) {
-            // penalties: read by the streaming pass and by the kernel for the rows handed on, rewritten
-            // by one pass over them at the end
+            // penalties: read by the streaming pass (and by the finishing workgroup of a row it has to
+            // do the slow way), rewritten by one pass over them at the end
             p.defer_pen = 1;
             if (launch_stream_pen((uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
-            p.need = v.need;
-            p.G = stream_parts(V, 16);
-            const uint32_t lgrid = kListGrid / p.G * p.G > 0 ? kListGrid / p.G * p.G : p.G;
-            if (launch_list_pen16(dim3(lgrid), st, p) != hipSuccess) return RS_ERR_LAUNCH;
             return launch_penalty_pass(st, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         }
-        if (launch_stream(sr, logits_dtype, (uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
-        p.need = v.need;               // the cluster kernel follows for the rows the finish left over
-        // Workgroups for the rows handed on.  Few rows are expected when top_k bounds the kept set: a
-        // small grid whose workgroups take tickets until the list is exhausted.  After an attempt it
-        // may be all of them: one workgroup per slice of every row, as in the cluster kernel; those
-        // beyond the list leave at once.
-        if (path == kPathStream && grid.x > kListGrid) grid.x = kListGrid / g.G * g.G > 0 ? kListGrid / g.G * g.G : g.G;
+        return launch_stream(sr, logits_dtype, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
     }
-    const hipError_t e = p.need ? launch_list(g.R, grid, (hipStream_t)stream, p, path == kPathAttempt)
-                              : launch_sample(pen, g.R, grid, (hipStream_t)stream, p);
-    return e == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+    return launch_sample(pen, g.R, grid, (hipStream_t)stream, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
 }
 
 int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,

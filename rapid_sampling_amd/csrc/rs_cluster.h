@@ -623,63 +623,4 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     sample_slice<R, PEN>(p, s, row, ticket - row * p.G);
 }
 
-// The launch that follows the streaming pass knows how many rows were handed on.  Its first
-// workgroup tells the host -- a word of pinned memory that rs_sample looks at, without waiting,
-// before its next call -- whether that was most of them: such calls are then better served by
-// the cluster kernel alone for a while.  The word belongs to the caller's rs_policy.
-__device__ __forceinline__ void report_streaming(const Params &p, uint32_t handed_on)
-{
-    if (blockIdx.x == 0 && threadIdx.x == 0 && p.host_words)
-        __hip_atomic_store(p.host_words + p.report, handed_on * 2u > (uint32_t)p.B ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-}
-
-// The launch that follows the streaming pass: workgroups work through the
-// rows on its list, taking tickets until the list is exhausted.
-template <int R, bool PEN = false>
-__global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_list_kernel(const Params p)
-{
-    __shared__ Lds s;
-    const uint32_t G = p.G;
-    const uint32_t n = a_load(&p.hdr->n_need);
-    report_streaming(p, n);
-    if (n == 0u) return;                                         // nothing left over: no ticket was taken
-    for (;;) {
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            s.abort = 0; s.host_words = p.host_words;
-            s.bc32[0] = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        }
-        __syncthreads();
-        const uint32_t ticket = s.bc32[0];
-        const uint32_t slot = ticket / G;
-        if (slot >= a_load(&p.hdr->n_need)) break;
-        if (!sample_slice<R, PEN>(p, s, p.need[slot], ticket - slot * G)) return;
-    }
-    leave_launch(p.hdr);
-}
-
-// The same for a launch of one workgroup per slice of every row of the batch:
-// each takes one ticket, those beyond the list leave at once.  Used behind an
-// attempt, after which the list may hold every row.
-template <int R>
-__global__ void __launch_bounds__(kThreads, (min_waves<R, false>())) sample_list_once_kernel(const Params p)
-{
-    __shared__ Lds s;
-    const uint32_t n = a_load(&p.hdr->n_need);
-    report_streaming(p, n);
-    if (n == 0u) return;                                         // nothing left over: no ticket was taken
-    if (threadIdx.x == 0) {
-        s.abort = 0; s.host_words = p.host_words;
-        const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);     // the last ticket of the launch
-        s.bc32[0] = t;
-    }
-    __syncthreads();
-    const uint32_t ticket = s.bc32[0];
-    const uint32_t slot = ticket / p.G;
-    if (slot >= n) return;
-    sample_slice<R, false>(p, s, p.need[slot], ticket - slot * p.G);
-}
-
-
 }  // namespace rs

@@ -19,38 +19,6 @@ static hipError_t launch_sample_t(int R, dim3 grid, hipStream_t st, const Params
     return hipGetLastError();
 }
 
-hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p, bool once)
-{
-    if (once) {
-        switch (R) {
-        case 1:  hipLaunchKernelGGL((sample_list_once_kernel<1>),  grid, dim3(kThreads), 0, st, p); break;
-        case 2:  hipLaunchKernelGGL((sample_list_once_kernel<2>),  grid, dim3(kThreads), 0, st, p); break;
-        case 4:  hipLaunchKernelGGL((sample_list_once_kernel<4>),  grid, dim3(kThreads), 0, st, p); break;
-        case 8:  hipLaunchKernelGGL((sample_list_once_kernel<8>),  grid, dim3(kThreads), 0, st, p); break;
-        case 16: hipLaunchKernelGGL((sample_list_once_kernel<16>), grid, dim3(kThreads), 0, st, p); break;
-        default: hipLaunchKernelGGL((sample_list_once_kernel<32>), grid, dim3(kThreads), 0, st, p); break;
-        }
-        return hipGetLastError();
-    }
-    switch (R) {
-    case 1:  hipLaunchKernelGGL((sample_list_kernel<1>),  grid, dim3(kThreads), 0, st, p); break;
-    case 2:  hipLaunchKernelGGL((sample_list_kernel<2>),  grid, dim3(kThreads), 0, st, p); break;
-    case 4:  hipLaunchKernelGGL((sample_list_kernel<4>),  grid, dim3(kThreads), 0, st, p); break;
-    case 8:  hipLaunchKernelGGL((sample_list_kernel<8>),  grid, dim3(kThreads), 0, st, p); break;
-    case 16: hipLaunchKernelGGL((sample_list_kernel<16>), grid, dim3(kThreads), 0, st, p); break;
-    default: hipLaunchKernelGGL((sample_list_kernel<32>), grid, dim3(kThreads), 0, st, p); break;
-    }
-    return hipGetLastError();
-}
-
-
-// rows the streaming pass with penalties handed on: penalties enter x, their update is left to the pass that follows
-hipError_t launch_list_pen16(dim3 grid, hipStream_t st, const Params &p)
-{
-    hipLaunchKernelGGL((sample_list_kernel<16, true>), grid, dim3(kThreads), 0, st, p);
-    return hipGetLastError();
-}
-
 hipError_t launch_sample(bool pen, int R, dim3 grid, hipStream_t st, const Params &p)
 {
     return pen ? launch_sample_t<true>(R, grid, st, p) : launch_sample_t<false>(R, grid, st, p);

@@ -29,9 +29,10 @@ struct alignas(256) WsHeader {
     uint32_t ticket;      // next logical workgroup id of the running launch
     uint32_t finished;    // workgroups that have left the running launch
     int32_t  error;       // sticky RS_ERR_DEVICE
-    uint32_t n_need;      // rows the streaming pass handed to the cluster kernel
+    uint32_t n_need;      // rows of the running (or last) streaming call that the finishing workgroups did the slow way
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
-    uint32_t pad[59];
+    uint32_t last_call;   // batch size | kind << 31 of the last streaming call (kind: 0 top_k bounds the kept set, 1 not)
+    uint32_t pad[58];
 };
 
 // How long a workgroup waits for its peers before it gives up (wall-clock ticks).
@@ -74,7 +75,6 @@ struct Params {
     WsHeader    *hdr;
     RowCtl      *ctl_end;      // one past the record of row 0; row r is ctl_end[-1 - r]
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
-    const uint32_t *need;      // null, or the list of rows this launch is for (hdr->n_need entries)
     int32_t      dtype;        // RS_DTYPE_* of the logits
     uint32_t     report;       // which of the two report words a streaming call writes: 0 top_k bounds the kept set, 1 not
     int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1] routing reports, [2] error; or null
@@ -529,17 +529,6 @@ __device__ __forceinline__ u128 get_mass(uint64_t w0, uint64_t w1)
     return ((u128)(w1 & ~kValid) << 62) | (w0 & ~kValid);
 }
 
-// Last act of a workgroup of the cluster kernel: the workgroup that leaves last
-// resets the launch-wide counters for the next call.
-__device__ __forceinline__ void leave_launch(WsHeader *hdr)
-{
-    if (threadIdx.x == 0) {
-        wait_vmem();
-        const uint32_t fin = __hip_atomic_fetch_add(&hdr->finished, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        if (fin == gridDim.x - 1) { a_store(&hdr->finished, 0u); a_store(&hdr->ticket, 0u); a_store(&hdr->n_need, 0u); }
-    }
-}
-
 // Tie weight, kept total S and inverse-CDF target r from the threshold and
 // the masses around it (reference: sampling.cu:365-371 and :374-381).  One
 // thread; also fills the diagnostics record when there is one.
@@ -605,7 +594,6 @@ struct StreamView {
     uint64_t *stash;      // [B][G][kStashCap]   bits(e, slice frame) << 32 | index, by descending bin
     uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
     uint64_t *shist;      // [B][G][kSB]   the slice's own bins (slice frame), as it added them to the row's
-    uint32_t *need;       // [B]  rows left to the cluster kernel
     uint32_t  G;          // slices per row
     uint32_t  list_cap;   // entries of the finishing workgroup's token list (a power of two up to kFinCap)
 };
@@ -613,8 +601,6 @@ struct StreamView {
 
 // Launchers, one per translation unit that instantiates the kernels.
 hipError_t launch_sample(bool pen, int R, dim3 grid, hipStream_t st, const Params &p);
-hipError_t launch_list(int R, dim3 grid, hipStream_t st, const Params &p, bool once);
-hipError_t launch_list_pen16(dim3 grid, hipStream_t st, const Params &p);
 hipError_t launch_stream_pen(uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
 hipError_t launch_penalty_pass(hipStream_t st, const Params &p);
 hipError_t launch_stream(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,

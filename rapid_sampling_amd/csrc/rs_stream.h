@@ -49,6 +49,28 @@ struct LdsA {
     uint32_t cov, n, cut, over;
 };
 
+// Routing report of the streaming path.  Rows that the finishing workgroups had to do the slow way
+// are counted in the workspace header; the first thread of the next streaming call collects the
+// count (its memory round trip overlaps with the thread's loads of the logits) and tells the
+// caller's policy whether that was most of the rows of that call -- a call that goes badly says so
+// itself, at once (finish_row), a call that goes well is vouched for by the next one.
+struct PrevCall { uint32_t slow_rows, meta; };
+__device__ __forceinline__ PrevCall report_begin(const Params &p)
+{
+    PrevCall pc;
+    pc.slow_rows = __hip_atomic_exchange(&p.hdr->n_need, 0u, __ATOMIC_RELAXED, RS_AGENT);
+    pc.meta = a_load(&p.hdr->last_call);                 // batch size | kind << 31 of that call, 0 = none yet
+    return pc;
+}
+__device__ __forceinline__ void report_end(const Params &p, const PrevCall &pc)
+{
+    a_store(&p.hdr->last_call, (uint32_t)p.B | (p.report << 31));
+    if (p.host_words && pc.meta) {
+        const uint32_t rows = pc.meta & 0x7FFFFFFFu;
+        __hip_atomic_store(p.host_words + (pc.meta >> 31), pc.slow_rows * 2u > rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
 #ifndef RS_STREAM_WAVES
 #define RS_STREAM_WAVES 3
 #endif
@@ -289,6 +311,10 @@ __global__ void __launch_bounds__(NT, (R <= 4 ? 5 : RS_STREAM_WAVES)) stream_ker
     const int nv = base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - base4 + NT - 1) / NT);
     const char *lrow = logits_row(p, row);
 
+    const bool reporter = blockIdx.x == 0 && tid == 0;
+    PrevCall prev;
+    prev.slow_rows = 0; prev.meta = 0;
+    if (reporter) prev = report_begin(p);
     uint32_t eb[R * 4];                                 // l, then x, then bits(e)
     // x = l * c is the definition unless a NaN or Inf shows up (see sample_kernel).  Slots past the
     // end of the row read its last group again: harmless for the maximum and the probe, and they
@@ -334,7 +360,7 @@ __global__ void __launch_bounds__(NT, (R <= 4 ? 5 : RS_STREAM_WAVES)) stream_ker
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    if (blockIdx.x == 0 && tid == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
+    if (reporter) report_end(p, prev);
     slice_count_and_stash<R, NT, kRep, false>(p, v, s, eb, lmax, row, part, base4, nv);
 }
 
@@ -385,6 +411,199 @@ __device__ __forceinline__ uint32_t bucket_step(Lds &s, LdsB &t, uint32_t nlist,
     __syncthreads();
     r = s.bc128[1];
     return t.bucket;
+}
+
+// A row the stashes cannot finish (a nucleus or a tie of thousands of tokens, more kept tokens than
+// the list holds): the finishing workgroup does it alone, from the logits, in a few passes over the
+// row -- the level-1 histogram in the row's frame (M = floor of the row's maximum is known), the
+// next digits of the threshold inside the boundary bin until the bin's tokens fit a gathered list,
+// the rest in LDS, then the inverse CDF by buckets of the token index, by sub-buckets, and token
+// by token.  A few passes of one workgroup over one row take tens of microseconds (a row of a
+// million tokens: more than a hundred): fine for the odd row, and calls whose rows mostly end here
+// are routed to the cluster kernel by the caller's policy.  Same integers as every other path.
+__device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float xmax, const uint64_t rand64)
+{
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const uint32_t V4 = (uint32_t)p.V >> 2;
+    const float M = __builtin_floorf(xmax);
+    const char *lrow = logits_row(p, row);
+    const float4 *pn4 = p.penalties ? reinterpret_cast<const float4 *>(p.penalties + (int64_t)row * p.V) : nullptr;
+    // bits of e of the four tokens of group i4, by the definition (reference: sampling.cu:220, :553)
+    auto bits4 = [&](uint32_t i4, uint32_t *b) {
+        const float4 l = load_logits4(lrow, i4, p.dtype);
+        float x0, x1, x2, x3;
+        if (pn4) {
+            const float4 q = pn4[i4];
+            x0 = sf((sf(l.x) - q.x) * p.c); x1 = sf((sf(l.y) - q.y) * p.c); x2 = sf((sf(l.z) - q.z) * p.c); x3 = sf((sf(l.w) - q.w) * p.c);
+        } else {
+            x0 = sf(l.x * p.c); x1 = sf(l.y * p.c); x2 = sf(l.z * p.c); x3 = sf(l.w * p.c);
+        }
+        b[0] = e_bits_of(x0, M); b[1] = e_bits_of(x1, M); b[2] = e_bits_of(x2, M); b[3] = e_bits_of(x3, M);
+    };
+    const uint64_t top_k = (uint64_t)p.top_k;
+
+    // level 1 (dead tokens, below 2^-40, are left out)
+    __syncthreads();
+    for (int b = tid; b < kNB * kRepC; b += kThreads) s.hr[b] = 0;
+    __syncthreads();
+    for (uint32_t i4 = (uint32_t)tid; i4 < V4; i4 += kThreads) {
+        uint32_t b[4];
+        bits4(i4, b);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (b[k] >= kEMinBits)
+                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hr[(b[k] >> 21) * kRepC + (lane & (kRepC - 1))]),
+                          (unsigned long long)(kPackOne | (b[k] & 0x7FFFFFu)));
+    }
+    __syncthreads();
+    for (int b = tid; b < kNB; b += kThreads) {
+        uint64_t w = 0;
+#pragma unroll
+        for (int c = 0; c < kRepC; ++c) w += s.hr[b * kRepC + c];
+        s.g[b] = w;
+    }
+    __syncthreads();
+    Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
+    const u128 D = s.D, P = s.P;
+    const uint32_t exb = f.bin >> 2;
+    uint32_t lo = f.bin << 21, span = (1u << 21) - 1u, levels = 1;
+    bool one_tie = false;
+    if (f.cnt_bin > (uint32_t)kCap && f.cnt_above == 0u) {
+        const uint32_t emax = e_bits_of(xmax, M);
+        one_tie = bin_is_one_tie(s.g[f.bin], f.bin, emax);
+        if (one_tie) { lo = emax; span = 0u; }
+    }
+    // further digits over the whole row while the boundary bin holds more tokens than can be gathered
+    while (!one_tie && f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
+        ++levels;
+        const uint32_t dsh = level_shift(levels);
+        __syncthreads();
+        lds_hist_zero(s, 128);
+        __syncthreads();
+        for (uint32_t i4 = (uint32_t)tid; i4 < V4; i4 += kThreads) {
+            uint32_t b[4];
+            bits4(i4, b);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (b[k] - lo <= span) lds_hist_add(s, (b[k] >> dsh) & 127u, b[k]);
+        }
+        __syncthreads();
+        f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
+        lo |= f.bin << dsh;
+        span = (1u << dsh) - 1u;
+    }
+    if (f.cnt_bin <= (uint32_t)kCap) {
+        // gather the bin's tokens and resolve the remaining digits on them
+        __syncthreads();
+        if (tid == 0) s.ctr = 0;
+        __syncthreads();
+        for (uint32_t i4 = (uint32_t)tid; i4 < V4; i4 += kThreads) {
+            uint32_t b[4];
+            bits4(i4, b);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (b[k] - lo <= span) {
+                    const uint32_t o = atomicAdd(&s.ctr, 1u);
+                    if (o < (uint32_t)kCap) s.cand[o] = ((uint64_t)b[k] << 32) | (i4 * 4u + (uint32_t)k);
+                }
+        }
+        __syncthreads();
+        const uint32_t ncand = min(s.ctr, (uint32_t)kCap);
+        for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels && f.cnt_bin > 1u && span != 0u; ++lv) {
+            const uint32_t dsh = level_shift(lv);
+            lds_hist_zero(s, 128);
+            __syncthreads();
+            for (uint32_t i = tid; i < ncand; i += kThreads) {
+                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
+                if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, b);
+            }
+            __syncthreads();
+            f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
+            lo |= f.bin << dsh;
+            span = (1u << dsh) - 1u;
+        }
+        if (span != 0u) {
+            for (uint32_t i = tid; i < ncand; i += kThreads) {
+                const uint32_t b = (uint32_t)(s.cand[i] >> 32);
+                if (b - lo <= span) s.bc32[6] = b;
+            }
+            __syncthreads();
+            lo = s.bc32[6];
+        }
+    }
+    const uint32_t thr = lo;
+    if (tid == 0) {
+        const Target tg = tie_and_target(p, row, rand64, xmax, D, P, thr, f.cnt_above, f.cnt_bin, f.mass_above, 8u, true);
+        s.bc64[1] = tg.w_tie; s.bc128[0] = tg.r;
+    }
+    __syncthreads();
+    const uint64_t w_tie = s.bc64[1];
+    u128 r = s.bc128[0];
+    auto weight = [&](uint32_t b) -> uint64_t { return (b > thr) ? w_of_bits(b) : (b == thr ? w_tie : 0); };
+
+    // inverse CDF in index order: 256 buckets of 2^sh1 tokens, 256 sub-buckets of 2^sh2, then one by one
+    uint32_t sh1 = 0;
+    while (((uint32_t)p.V - 1u) >> sh1 >= 256u) ++sh1;
+    const uint32_t sh2 = sh1 > 8u ? sh1 - 8u : 0u;
+    auto bucket_pass = [&](uint32_t lo_idx, uint32_t hi_idx, uint32_t shift) -> uint32_t {
+        t.blo[tid] = 0; t.bhi[tid] = 0;
+        __syncthreads();
+        const uint32_t a4 = lo_idx >> 2, e4 = min(V4, (hi_idx + 3u) >> 2);
+        for (uint32_t i4 = a4 + (uint32_t)tid; i4 < e4; i4 += kThreads) {
+            uint32_t b[4];
+            bits4(i4, b);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t idx = i4 * 4u + (uint32_t)k;
+                const uint64_t w = weight(b[k]);
+                if (w && idx >= lo_idx && idx < hi_idx) {
+                    const uint32_t bk = (idx - lo_idx) >> shift;           // < 256: the range spans at most 256 buckets
+                    atomicAdd(reinterpret_cast<unsigned long long *>(&t.blo[bk]), (unsigned long long)(w & 0xFFFFFFFFull));
+                    atomicAdd(reinterpret_cast<unsigned long long *>(&t.bhi[bk]), (unsigned long long)(w >> 32));
+                }
+            }
+        }
+        __syncthreads();
+        const u128 mine = (u128)t.blo[tid] + ((u128)t.bhi[tid] << 32);
+        u128 inc = wave_inclusive_scan(mine);
+        if (lane == kWave - 1) s.q128[wave] = inc;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) inc += s.q128[w];
+        const u128 exc = inc - mine;
+        if (exc < r && r <= inc) { t.bucket = (uint32_t)tid; s.bc128[1] = r - exc; }
+        __syncthreads();
+        r = s.bc128[1];
+        const uint32_t bk = t.bucket;
+        __syncthreads();
+        return bk;
+    };
+    const uint32_t b1 = bucket_pass(0u, (uint32_t)p.V, sh1);
+    uint32_t lo_idx = b1 << sh1;
+    if (sh1 > sh2) {
+        const uint32_t b2 = bucket_pass(lo_idx, min((uint32_t)p.V, lo_idx + (1u << sh1)), sh2);
+        lo_idx += b2 << sh2;
+    }
+    if (tid == 0) {
+        // the last few tokens one after the other
+        const uint32_t hi_idx = min((uint32_t)p.V, lo_idx + (1u << sh2));
+        uint32_t pick = lo_idx;
+        u128 acc = 0;
+        for (uint32_t i4 = lo_idx >> 2; i4 * 4u < hi_idx; ++i4) {
+            uint32_t b[4];
+            bits4(i4, b);
+            bool found = false;
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t idx = i4 * 4u + (uint32_t)k;
+                if (idx < lo_idx || idx >= hi_idx) continue;
+                acc += weight(b[k]);
+                if (acc >= r) { pick = idx; found = true; break; }
+            }
+            if (found) break;
+        }
+        p.out[row] = (int32_t)pick;
+        if (p.diag) p.diag[row].index = (int32_t)pick;
+        t.result = pick + 1u;
+    }
 }
 
 // Finishes a row from what its slices published.  Returns true when the row is done (token written),
@@ -502,6 +721,22 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     const uint64_t top_k = (uint64_t)p.top_k;
     Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
+    // What the stashes cannot finish, this workgroup does alone from the logits (three-launch path).
+    // Such rows are counted, and once they are most of the call's the caller's policy is told at once
+    // (that calls went well is reported by the next streaming call, see finish_kernel).
+    auto slow = [&]() -> bool {
+        if (drawer) {                                    // the row is finished here: this draw is used up
+            rng_st[2] = rs[2] + 1u;
+            if (rs[2] + 1u == 0u) rng_st[3] = rs[3] + 1u;
+        }
+        finish_row_slow(p, s, t, row, xmax, p.inj_u ? 0ull : t.rand64);
+        if (tid == 0) {
+            const uint32_t c = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
+            if ((c + 1u) * 2u > (uint32_t)p.B && c * 2u <= (uint32_t)p.B && p.host_words)
+                __hip_atomic_store(p.host_words + p.report, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        return true;
+    };
 
     // A row that is one tie of all its tokens (rows of equal logits) needs no stash at all: the
     // threshold is the largest token's value, every token weighs the tie weight, and the token at
@@ -564,12 +799,9 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
         total = t.take[kThreads - 1];
         if (total > v.list_cap || total == 0u) {
-            // not resolvable from the stashes: leave the row to the cluster kernel
-            if (!FUSED && tid == 0) {
-                const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
-                v.need[slot] = row;
-            }
-            return false;
+            // not resolvable from the stashes
+            if (FUSED) return false;
+            return slow();
         }
         subset = true;
     }
@@ -636,11 +868,8 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         f = hist_find_level1<false, true>(s, top_k, p.top_p, lane, wave);
         if (f.bin == 0u) {
             // even all of them are neither top_k tokens nor top_p of the mass
-            if (!FUSED && tid == 0) {
-                const uint32_t slot = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
-                v.need[slot] = row;
-            }
-            return false;
+            if (FUSED) return false;
+            return slow();
         }
         exb = f.bin >> 2;
     }
@@ -779,10 +1008,14 @@ __global__ void __launch_bounds__(kThreads, 2) stream_pen_kernel(const Params p,
     __shared__ LdsA<kRep> s;
     const uint32_t G = v.G;
     const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
+    const bool reporter = blockIdx.x == 0 && threadIdx.x == 0;
+    PrevCall prev;
+    prev.slow_rows = 0; prev.meta = 0;
+    if (reporter) prev = report_begin(p);
     Slice<R, true> sl;
     slice_setup(p, sl, row, part, G);
     const float lmax = slice_load(p, sl);
-    if (blockIdx.x == 0 && threadIdx.x == 0) a_store(&p.hdr->n_need, 0u);   // the list of the previous call is history
+    if (reporter) report_end(p, prev);
     slice_count_and_stash<R, kThreads, kRep, false>(p, v, s, sl.eb, lmax, row, part, sl.base4, sl.nv);
 }
 
