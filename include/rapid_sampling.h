@@ -130,7 +130,7 @@ int rs_workspace_status(const void *workspace_device, int32_t *status, void *str
  * yes/no" to a word of pinned host memory inside it, and rs_sample_ex reads
  * that word, without waiting, before it routes the next call: after a call
  * that handed most rows on, calls of that kind go straight to the general
- * kernel and one in 64 streams again.  Without a policy, calls with a bounding
+ * kernel and one in 256 streams again.  Without a policy, calls with a bounding
  * top_k always stream and calls without never do.  Results do not depend on
  * the routing.
  *

@@ -192,7 +192,7 @@ namespace rs {
 // caller's rs_policy, one word for calls with a bounding top_k and one for calls without, and
 // this function looks at the word -- without waiting for anything; a stale value only delays the
 // switch -- before it chooses the path of the next call: after a call that handed most rows on,
-// calls of that kind go straight to the cluster kernel and one in 64 streams again.  Without a
+// calls of that kind go straight to the cluster kernel and one in 256 streams again.  Without a
 // policy, calls with a bounding top_k always stream and calls without never do.
 //
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
@@ -234,10 +234,10 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     // Larger calls with penalties: the streaming pass with a pass over the penalties behind it, from
     // kPenStreamMin tokens on (measured crossover with the general kernel), long slices only.
     rs_policy *pol = opt ? opt->policy : nullptr;
-    // after a call of this kind that handed most rows on: straight to the general kernel, one in 64 tries again
+    // after a call of this kind that handed most rows on: straight to the general kernel, one in 256 tries again
     auto routed_away = [&](int kind) {
         if (!pol || *(volatile int32_t *)(pol->word + kind) == 0) return false;
-        return (++pol->calls[kind] & 63u) != 0u;
+        return (++pol->calls[kind] & 255u) != 0u;
     };
     if (pen && bounded && stream_r(B, V) == kStreamLongR && stream_parts(V, kStreamLongR) >= 2u) {
         if (force == RS_PATH_STREAM || force == RS_PATH_ATTEMPT) return kPathStream;

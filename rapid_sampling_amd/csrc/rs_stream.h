@@ -421,24 +421,43 @@ __device__ __forceinline__ uint32_t bucket_step(Lds &s, LdsB &t, uint32_t nlist,
 // by token.  A few passes of one workgroup over one row take tens of microseconds (a row of a
 // million tokens: more than a hundred): fine for the odd row, and calls whose rows mostly end here
 // are routed to the cluster kernel by the caller's policy.  Same integers as every other path.
-__device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float xmax, const uint64_t rand64)
+__device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float xmax, const uint64_t rand64)
 {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const float M = __builtin_floorf(xmax);
     const char *lrow = logits_row(p, row);
     const float4 *pn4 = p.penalties ? reinterpret_cast<const float4 *>(p.penalties + (int64_t)row * p.V) : nullptr;
-    // bits of e of the four tokens of group i4, by the definition (reference: sampling.cu:220, :553)
-    auto bits4 = [&](uint32_t i4, uint32_t *b) {
-        const float4 l = load_logits4(lrow, i4, p.dtype);
+    // bits of e of four tokens, by the definition (reference: sampling.cu:220, :553)
+    auto bits_of4 = [&](const float4 l, const float4 q) -> uint4 {
         float x0, x1, x2, x3;
         if (pn4) {
-            const float4 q = pn4[i4];
             x0 = sf((sf(l.x) - q.x) * p.c); x1 = sf((sf(l.y) - q.y) * p.c); x2 = sf((sf(l.z) - q.z) * p.c); x3 = sf((sf(l.w) - q.w) * p.c);
         } else {
             x0 = sf(l.x * p.c); x1 = sf(l.y * p.c); x2 = sf(l.z * p.c); x3 = sf(l.w * p.c);
         }
-        b[0] = e_bits_of(x0, M); b[1] = e_bits_of(x1, M); b[2] = e_bits_of(x2, M); b[3] = e_bits_of(x3, M);
+        return make_uint4(e_bits_of(x0, M), e_bits_of(x1, M), e_bits_of(x2, M), e_bits_of(x3, M));
+    };
+    // fn(token index, bits of its e) for the tokens of groups [lo4, hi4) of the row, four loads in flight per thread
+    auto row_pass = [&](uint32_t lo4, uint32_t hi4, auto fn) {
+        constexpr int kAhead = 4;
+        for (uint32_t base = lo4 + (uint32_t)tid; base < hi4; base += kAhead * kThreads) {
+            float4 l[kAhead], q[kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const uint32_t i4 = min(base + (uint32_t)u * kThreads, hi4 - 1u);
+                l[u] = load_logits4(lrow, i4, p.dtype);
+                q[u] = pn4 ? pn4[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const uint32_t i4 = base + (uint32_t)u * kThreads;
+                if (i4 < hi4) {
+                    const uint4 b = bits_of4(l[u], q[u]);
+                    fn(i4 * 4u, b.x); fn(i4 * 4u + 1u, b.y); fn(i4 * 4u + 2u, b.z); fn(i4 * 4u + 3u, b.w);
+                }
+            }
+        }
     };
     const uint64_t top_k = (uint64_t)p.top_k;
 
@@ -446,15 +465,11 @@ __device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, c
     __syncthreads();
     for (int b = tid; b < kNB * kRepC; b += kThreads) s.hr[b] = 0;
     __syncthreads();
-    for (uint32_t i4 = (uint32_t)tid; i4 < V4; i4 += kThreads) {
-        uint32_t b[4];
-        bits4(i4, b);
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            if (b[k] >= kEMinBits)
-                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hr[(b[k] >> 21) * kRepC + (lane & (kRepC - 1))]),
-                          (unsigned long long)(kPackOne | (b[k] & 0x7FFFFFu)));
-    }
+    row_pass(0u, V4, [&](uint32_t, uint32_t b) {
+        if (b >= kEMinBits)
+            atomicAdd(reinterpret_cast<unsigned long long *>(&s.hr[(b >> 21) * kRepC + (lane & (kRepC - 1))]),
+                      (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
+    });
     __syncthreads();
     for (int b = tid; b < kNB; b += kThreads) {
         uint64_t w = 0;
@@ -480,13 +495,9 @@ __device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, c
         __syncthreads();
         lds_hist_zero(s, 128);
         __syncthreads();
-        for (uint32_t i4 = (uint32_t)tid; i4 < V4; i4 += kThreads) {
-            uint32_t b[4];
-            bits4(i4, b);
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (b[k] - lo <= span) lds_hist_add(s, (b[k] >> dsh) & 127u, b[k]);
-        }
+        row_pass(0u, V4, [&](uint32_t, uint32_t b) {
+            if (b - lo <= span) lds_hist_add(s, (b >> dsh) & 127u, b);
+        });
         __syncthreads();
         f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
         lo |= f.bin << dsh;
@@ -497,16 +508,12 @@ __device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, c
         __syncthreads();
         if (tid == 0) s.ctr = 0;
         __syncthreads();
-        for (uint32_t i4 = (uint32_t)tid; i4 < V4; i4 += kThreads) {
-            uint32_t b[4];
-            bits4(i4, b);
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (b[k] - lo <= span) {
-                    const uint32_t o = atomicAdd(&s.ctr, 1u);
-                    if (o < (uint32_t)kCap) s.cand[o] = ((uint64_t)b[k] << 32) | (i4 * 4u + (uint32_t)k);
-                }
-        }
+        row_pass(0u, V4, [&](uint32_t idx, uint32_t b) {
+            if (b - lo <= span) {
+                const uint32_t o = atomicAdd(&s.ctr, 1u);
+                if (o < (uint32_t)kCap) s.cand[o] = ((uint64_t)b << 32) | idx;
+            }
+        });
         __syncthreads();
         const uint32_t ncand = min(s.ctr, (uint32_t)kCap);
         for (uint32_t lv = levels + 1; lv <= (uint32_t)kLevels && f.cnt_bin > 1u && span != 0u; ++lv) {
@@ -549,20 +556,14 @@ __device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, c
         t.blo[tid] = 0; t.bhi[tid] = 0;
         __syncthreads();
         const uint32_t a4 = lo_idx >> 2, e4 = min(V4, (hi_idx + 3u) >> 2);
-        for (uint32_t i4 = a4 + (uint32_t)tid; i4 < e4; i4 += kThreads) {
-            uint32_t b[4];
-            bits4(i4, b);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t idx = i4 * 4u + (uint32_t)k;
-                const uint64_t w = weight(b[k]);
-                if (w && idx >= lo_idx && idx < hi_idx) {
-                    const uint32_t bk = (idx - lo_idx) >> shift;           // < 256: the range spans at most 256 buckets
-                    atomicAdd(reinterpret_cast<unsigned long long *>(&t.blo[bk]), (unsigned long long)(w & 0xFFFFFFFFull));
-                    atomicAdd(reinterpret_cast<unsigned long long *>(&t.bhi[bk]), (unsigned long long)(w >> 32));
-                }
+        row_pass(a4, e4, [&](uint32_t idx, uint32_t b) {
+            const uint64_t w = weight(b);
+            if (w && idx >= lo_idx && idx < hi_idx) {
+                const uint32_t bk = (idx - lo_idx) >> shift;               // < 256: the range spans at most 256 buckets
+                atomicAdd(reinterpret_cast<unsigned long long *>(&t.blo[bk]), (unsigned long long)(w & 0xFFFFFFFFull));
+                atomicAdd(reinterpret_cast<unsigned long long *>(&t.bhi[bk]), (unsigned long long)(w >> 32));
             }
-        }
+        });
         __syncthreads();
         const u128 mine = (u128)t.blo[tid] + ((u128)t.bhi[tid] << 32);
         u128 inc = wave_inclusive_scan(mine);
@@ -588,17 +589,15 @@ __device__ __noinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, c
         const uint32_t hi_idx = min((uint32_t)p.V, lo_idx + (1u << sh2));
         uint32_t pick = lo_idx;
         u128 acc = 0;
-        for (uint32_t i4 = lo_idx >> 2; i4 * 4u < hi_idx; ++i4) {
-            uint32_t b[4];
-            bits4(i4, b);
-            bool found = false;
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t idx = i4 * 4u + (uint32_t)k;
-                if (idx < lo_idx || idx >= hi_idx) continue;
-                acc += weight(b[k]);
-                if (acc >= r) { pick = idx; found = true; break; }
-            }
-            if (found) break;
+        bool found = false;
+        for (uint32_t i4 = lo_idx >> 2; i4 * 4u < hi_idx && !found; ++i4) {
+            const uint4 b = bits_of4(load_logits4(lrow, i4, p.dtype), pn4 ? pn4[i4] : make_float4(0.f, 0.f, 0.f, 0.f));
+            auto step = [&](uint32_t idx, uint32_t bits) {
+                if (found || idx < lo_idx || idx >= hi_idx) return;
+                acc += weight(bits);
+                if (acc >= r) { pick = idx; found = true; }
+            };
+            step(i4 * 4u, b.x); step(i4 * 4u + 1u, b.y); step(i4 * 4u + 2u, b.z); step(i4 * 4u + 3u, b.w);
         }
         p.out[row] = (int32_t)pick;
         if (p.diag) p.diag[row].index = (int32_t)pick;

@@ -808,7 +808,7 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
         res = smp.sample(lg_peaked, c, k, p, uniforms=u)
         _check(res, *ref_peaked, "after a failed attempt %d" % i)
         assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 1
-    for i in range(140):                                 # one call in 64 tries again; the second such call vouches for the first
+    for i in range(520):                                 # one call in 256 tries again; the second such call vouches for the first
         res = smp.sample(lg_peaked, c, k, p, uniforms=u, want_diag=False)
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
     assert policy(smp) == 0
@@ -833,7 +833,7 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)     # not streamed
     _check(res, *ref_peaked, "bounded, after rows of ties")
     assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 2
-    for i in range(140):
+    for i in range(520):
         res = smp.sample(lg_peaked, c, k, p, uniforms=u, want_diag=False)
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
     assert policy(smp) == 0
