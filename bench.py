@@ -18,8 +18,9 @@ stream the kernel runs on).  Next to it, in the same JSON line:
   roofline   the bandwidth-bound configuration (BASELINE.json configs[4]):
              logits (128,4,1048576) fp32 = 2 GiB resident, top_k 1024,
              top_p 0.95; algorithmic bytes = 4*V per sampled row; the time
-             is that of the whole call (its three launches), averaged over
-             back-to-back calls between two HIP events
+             is that of the whole call (its two launches), averaged over
+             back-to-back calls between two HIP events; beside it the same
+             rows with penalties (12*V algorithmic bytes per row)
   configs    time per call and rows/s of the other BASELINE configurations
   cpu_baseline  the CPU oracle (single thread) on a bounded sample of the
              headline workload; cpu_torch is torch-CPU softmax/sort/cumsum/
@@ -277,8 +278,8 @@ def main():
             "workload": "(B,T,V)=(128,4,1048576) N(0,1.5), top_k 1024, top_p 0.95: 128 sampled rows of 4 MiB, "
                         "stride T*V, algorithmic bytes 4*V per row = 512 MiB per call",
             "us_per_call": round(t_btv, 2), "rows_per_s": round(Bb / (t_btv * 1e-6), 1),
-            "kernels": "streaming path, three launches per call: rs::stream_kernel (reads the logits; dominant), "
-                       "rs::finish_kernel, rs::sample_list_kernel; achieved = bytes / time of the whole call",
+            "kernels": "streaming path, two launches per call: rs::stream_kernel (reads the logits; dominant) and "
+                       "rs::finish_kernel; achieved = bytes / time of the whole call",
             "cluster_path_us_per_call": round(t_cluster, 2),
             "read_peak_GBs": round(bytes_btv / (t_floor * 1e-6) / 1e9, 1),
             "frac_of_read_peak": round(t_floor / t_btv, 4),
@@ -299,6 +300,23 @@ def main():
             "us_per_call": round(t_half, 2), "achieved": round(Bb * Vb * 2 / (t_half * 1e-6) / 1e9, 1),
             "note": "(128,1048576) bfloat16 rows of the same values rounded, 2*V bytes per row, accept_half=True"}
         del half
+        # the same rows with penalties: logits and penalties read once, penalties rewritten once the
+        # tokens are known -- 12*V algorithmic bytes per row (4*V logits, 4*V + 4*V penalties)
+        pen_b = torch.where(torch.rand((Bb, Vb), generator=g, device=dev) < 0.02,
+                            torch.empty((Bb, Vb), device=dev).exponential_(1.0, generator=g),
+                            torch.zeros((), device=dev))
+        last = big[:, Tb - 1, :]
+
+        def call_pen():
+            return sample.batch_sampling_repetition_temperature_topk_topp(last, pen_b, st_h, 0.1, 0.1, 0.95, 1.0, 1024, 0.95)
+
+        t_pen = block_time_us(torch, call_pen, max(2, args.bandwidth_steps // 2), 2)
+        result["roofline"]["with_penalties"] = {
+            "us_per_call": round(t_pen, 2), "achieved": round(Bb * Vb * 12 / (t_pen * 1e-6) / 1e9, 1),
+            "frac": round(Bb * Vb * 12 / (t_pen * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "(128,1048576) fp32 rows (stride T*V) with a (128,1048576) penalties tensor, 2 % non-zero: "
+                    "rs::stream_pen_kernel, rs::finish_kernel, rs::penalty_pass_kernel; algorithmic bytes 12*V per row"}
+        del pen_b, last
         if args.traffic_probe:
             src = big.view(-1)[: Bb * Vb]
             dst = torch.empty_like(src)

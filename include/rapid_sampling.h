@@ -122,17 +122,20 @@ int rs_workspace_status(const void *workspace_device, int32_t *status, void *str
  * by the caller (optional; one per workspace).  No counterpart in the
  * reference.
  *
- * A row the wait-free streaming path cannot finish is handed to the general
- * kernel in a further launch, and a call whose rows mostly end that way has
- * wasted a pass: with a bounding top_k (<= 1024) that takes unusual rows (ties
- * of thousands of tokens), without one (top_p < 1 alone) a flat distribution.
- * Each streaming call that is given a policy reports "most rows handed on:
- * yes/no" to a word of pinned host memory inside it, and rs_sample_ex reads
- * that word, without waiting, before it routes the next call: after a call
- * that handed most rows on, calls of that kind go straight to the general
- * kernel and one in 256 streams again.  Without a policy, calls with a bounding
- * top_k always stream and calls without never do.  Results do not depend on
- * the routing.
+ * A row the wait-free streaming path cannot finish from what its pass over
+ * the logits set aside is done by one workgroup alone, from the logits again,
+ * which takes several times as long as the general kernel needs for a whole
+ * call of moderate size: with a bounding top_k (<= 1024) that takes unusual
+ * rows (ties of thousands of tokens), without one (top_p < 1 alone) a flat
+ * distribution.  Calls that are given a policy report "a row went the slow
+ * way: yes/no" to a word of pinned host memory inside it (yes at once, no by
+ * the next call on the workspace), and rs_sample_ex reads that word, without
+ * waiting, before it routes the next call: while it is set, calls of that
+ * kind go to the general kernel; after 64 of them the streaming path is tried
+ * again, each try that fails doubles that number (up to 1024), and a run of
+ * good streaming calls as long as the last stay away puts it back to 64.
+ * Without a policy, calls with a bounding top_k always stream and calls
+ * without never do.  Results do not depend on the routing.
  *
  * A kernel that gives up waiting (RS_ERR_DEVICE) also writes the code into a
  * third pinned word, which rs_policy_error reads without synchronising.
@@ -184,11 +187,14 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  *
  * Calls that share a workspace must be ordered on one stream.
  *
- * The call is one kernel launch, or three for calls of at least 2^17 tokens
- * without penalties whose kept set is expected to be small (a wait-free pass
- * over the logits, a per-row finish, and the general kernel for rows the
- * finish hands on; see rs_policy); results are identical either way.  No
- * environment variable is read.
+ * The call is one kernel launch (the general kernel; with penalties and
+ * top_k <= 1024 the one-launch streaming kernel while the call fits the GPU at
+ * once), two for calls of at least 2^17 tokens without penalties whose kept
+ * set is expected to be small (a wait-free pass over the logits and a per-row
+ * finish; see rs_policy), or three for calls of at least 2^23 tokens with
+ * penalties and top_k <= 1024 (the same two and a pass that rewrites the
+ * penalties); results are identical either way.  No environment variable is
+ * read.
  */
 int rs_sample(const float *logits_device, int64_t row_stride,
               float *penalties_device, int32_t *out_device,

@@ -16,7 +16,9 @@ Beyond the reference: keyword names, `uniforms=` (injected draws, for tests),
 type but float32 raises the reference's error), `reserve_workspace(B, V)`
 (allocates the current stream's workspace ahead of time: required before the
 calls are captured into a HIP graph), `workspace_status()` (synchronises and
-returns the error word of the current stream's workspace) and `set_wait_limit`.
+returns the error word of the current stream's workspace), `set_wait_limit` and
+`reset_routing()` (forgets what the stream's calls have learnt about which
+kernel suits the workload; for measurements that change workload on one stream).
 A call whose kernel gave up waiting for its peers raises RuntimeError on the
 next call on that stream at the latest.
 
@@ -47,6 +49,7 @@ floor_read = _sample.floor_read
 reserve_workspace = _sample.reserve_workspace
 workspace_status = _sample.workspace_status
 set_wait_limit = _sample.set_wait_limit
+reset_routing = _sample.reset_routing
 STATE_BYTES_PER_ROW = _sample.STATE_BYTES_PER_ROW
 DIAG_BYTES = _sample.DIAG_BYTES
 
@@ -61,6 +64,7 @@ __all__ = [
     "reserve_workspace",
     "workspace_status",
     "set_wait_limit",
+    "reset_routing",
     "STATE_BYTES_PER_ROW",
     "DIAG_BYTES",
     "KERNEL_LIBRARY",

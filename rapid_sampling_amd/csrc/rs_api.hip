@@ -174,26 +174,32 @@ static size_t stream_bytes(int32_t B, int32_t V)
 
 }  // namespace rs
 
-// The caller's routing state (see rapid_sampling.h).  word[0], word[1]: "most rows were handed on"
-// as last reported by a streaming call with / without a bounding top_k; word[2]: RS_ERR_DEVICE
-// once a kernel gave up a wait.  calls[]: calls routed away from the streaming path since.
+// The caller's routing state (see rapid_sampling.h).  word[0], word[1]: "a row had to be done the
+// slow way" as last reported by a streaming call with / without a bounding top_k; word[2]:
+// RS_ERR_DEVICE once a kernel gave up a wait.  away[]: calls routed away from the streaming path
+// since the word was last seen set and streaming tried; period[]: how many of them before streaming
+// is tried again; good[]: streaming calls in a row that found the word clear.
+constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u;
 struct rs_policy {
     int32_t *word;
-    uint32_t calls[2];
+    uint32_t away[2], period[2], good[2];
 };
 
 namespace rs {
 
 // The streaming path works when the kept set is small next to the row; a row for which it does
-// not is handed to the cluster kernel in a third launch, and a call whose rows mostly end that way
-// has wasted a pass.  With a bounding top_k that takes unusual rows (ties of thousands of tokens);
-// without one (nucleus sampling alone) it is simply a flat distribution, so such a call is an
-// attempt.  The launch for the rows handed on reports "most of them: yes/no" into a word of the
-// caller's rs_policy, one word for calls with a bounding top_k and one for calls without, and
-// this function looks at the word -- without waiting for anything; a stale value only delays the
-// switch -- before it chooses the path of the next call: after a call that handed most rows on,
-// calls of that kind go straight to the cluster kernel and one in 256 streams again.  Without a
-// policy, calls with a bounding top_k always stream and calls without never do.
+// not is done by its finishing workgroup alone, from the logits, which takes several times as long
+// as the general kernel needs for a whole call of moderate size.  With a bounding top_k that takes
+// unusual rows (ties of thousands of tokens); without one (nucleus sampling alone) it is simply a
+// flat distribution, so such a call is an attempt.  The kernels report "a row went the slow way:
+// yes/no" into a word of the caller's rs_policy, one word for calls with a bounding top_k and one
+// for calls without, and this function looks at the word -- without waiting for anything; a stale
+// value only delays the switch -- before it chooses the path of the next call.  While the word is
+// set, calls of that kind go to the general kernel, and streaming is tried again after 64 of them;
+// each try that fails doubles that number (up to 1024), and as many good streaming calls in a row
+// as the last stay away lasted put it back to 64: a workload whose rows are always too flat pays
+// for one slow call in a thousand, a rare slow row costs a handful of calls on the general kernel.
+// Without a policy, calls with a bounding top_k always stream and calls without never do.
 //
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
@@ -234,10 +240,19 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     // Larger calls with penalties: the streaming pass with a pass over the penalties behind it, from
     // kPenStreamMin tokens on (measured crossover with the general kernel), long slices only.
     rs_policy *pol = opt ? opt->policy : nullptr;
-    // after a call of this kind that handed most rows on: straight to the general kernel, one in 256 tries again
+    // after a call of this kind with a slow row: the general kernel for a while, then another try
     auto routed_away = [&](int kind) {
-        if (!pol || *(volatile int32_t *)(pol->word + kind) == 0) return false;
-        return (++pol->calls[kind] & 255u) != 0u;
+        if (!pol) return false;
+        if (*(volatile int32_t *)(pol->word + kind) == 0) {
+            if (pol->period[kind] > kAwayFirst && ++pol->good[kind] >= pol->period[kind]) pol->period[kind] = kAwayFirst;
+            pol->away[kind] = 0;
+            return false;
+        }
+        pol->good[kind] = 0;
+        if (++pol->away[kind] <= pol->period[kind]) return true;
+        pol->away[kind] = 0;                                  // this call streams again; a failure sets the word anew
+        pol->period[kind] = min(pol->period[kind] * 2u, kAwayMost);
+        return false;
     };
     if (pen && bounded && stream_r(B, V) == kStreamLongR && stream_parts(V, kStreamLongR) >= 2u) {
         if (force == RS_PATH_STREAM || force == RS_PATH_ATTEMPT) return kPathStream;
@@ -348,7 +363,8 @@ int rs_policy_create(rs_policy **out)
     *out = nullptr;
     rs_policy *pol = new (std::nothrow) rs_policy;
     if (!pol) return RS_ERR_LAUNCH;
-    pol->word = nullptr; pol->calls[0] = 0; pol->calls[1] = 0;
+    pol->word = nullptr;
+    for (int i = 0; i < 2; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
     if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
         delete pol;
         return RS_ERR_LAUNCH;

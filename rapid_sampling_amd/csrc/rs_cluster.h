@@ -589,15 +589,28 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
 {
     Slice<R, PEN> sl;
     slice_setup(p, sl, row, part, p.G);
+    // the call's first thread reports on the streaming call before it, if there was one (report_begin)
+    const bool reporter = blockIdx.x == 0 && threadIdx.x == 0 && p.host_words != nullptr;
+    PrevCall prev;
+    prev.slow_rows = 0; prev.meta = 0;
+    if (reporter) prev = report_begin(p);
     draw_rand(p, s, row);
     const float lmax = slice_load(p, sl);
+    if (reporter) report_end(p, prev, false);
     if (!slice_level1(p, s, sl, lmax)) return false;
     return slice_finish(p, s, sl);
 }
 
-// Workgroups take their (row, slice) from a ticket counter, so that logical
-// ids follow the order in which workgroups actually start: a workgroup only
-// ever waits for lower tickets, whose holders are running or done.
+// Workgroups take their (row, slice) from a ticket counter, so that logical ids follow the order in
+// which workgroups actually start and a row's workgroups are the next ones to start.  The workgroups
+// of a row wait for EACH OTHER (every exchange is all-to-all within the row, so a low ticket waits for
+// higher ones too): the waits end because a row has at most 256 workgroups and a workgroup, once
+// started, runs to its end without giving up its compute unit -- the dispatcher starts workgroups in
+// ticket order as room becomes free, so all workgroups of the oldest unfinished row are resident or
+// next in line.  That needs room for one whole row of workgroups on the GPU: 256 compute units with
+// at least one workgroup each hold it; a device partitioned below that, or shared with another
+// process's long-running kernels, can starve a row -- the waits are bounded for that case and end in
+// RS_ERR_DEVICE rather than a hang.
 template <int R, bool PEN>
 __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
 {

@@ -31,7 +31,7 @@ struct alignas(256) WsHeader {
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows of the running (or last) streaming call that the finishing workgroups did the slow way
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
-    uint32_t last_call;   // batch size | kind << 31 of the last streaming call (kind: 0 top_k bounds the kept set, 1 not)
+    uint32_t last_call;   // 1 | kind << 31 after a streaming call that no later call has reported on yet (kind: 0 top_k bounds the kept set, 1 not), else 0
     uint32_t pad[58];
 };
 
@@ -287,6 +287,30 @@ __device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr)
     a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
     if (s.host_words) __hip_atomic_store(s.host_words + 2, (int32_t)RS_ERR_DEVICE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     s.abort = 1;
+}
+
+// Routing report of the streaming path.  A row that the finishing workgroup has to do the slow way
+// (alone, from the logits, in several passes) costs several times what the general kernel takes for
+// the whole call, so one such row is reason enough to send the next calls of that kind to the
+// general kernel.  Slow rows are counted in the workspace header and the first of a call sets the
+// word of the caller's policy at once (finish_row); that a call went WELL is said by the first
+// thread of the next call on the workspace, streaming or not, which collects the count (its memory
+// round trip overlaps with the thread's loads of the logits) and clears the word.
+struct PrevCall { uint32_t slow_rows, meta; };
+__device__ __forceinline__ PrevCall report_begin(const Params &p)
+{
+    PrevCall pc;
+    pc.slow_rows = __hip_atomic_exchange(&p.hdr->n_need, 0u, __ATOMIC_RELAXED, RS_AGENT);
+    pc.meta = a_load(&p.hdr->last_call);                 // 1 | kind << 31 of a streaming call not yet reported on, else 0
+    return pc;
+}
+// `streaming`: the reporting call is a streaming call itself, to be reported on by the next one
+__device__ __forceinline__ void report_end(const Params &p, const PrevCall &pc, const bool streaming)
+{
+    if (streaming) a_store(&p.hdr->last_call, 1u | (p.report << 31));
+    else if (pc.meta) a_store(&p.hdr->last_call, 0u);
+    if (p.host_words && pc.meta)
+        __hip_atomic_store(p.host_words + (pc.meta >> 31), pc.slow_rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 __device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)

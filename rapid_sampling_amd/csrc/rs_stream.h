@@ -49,28 +49,6 @@ struct LdsA {
     uint32_t cov, n, cut, over;
 };
 
-// Routing report of the streaming path.  Rows that the finishing workgroups had to do the slow way
-// are counted in the workspace header; the first thread of the next streaming call collects the
-// count (its memory round trip overlaps with the thread's loads of the logits) and tells the
-// caller's policy whether that was most of the rows of that call -- a call that goes badly says so
-// itself, at once (finish_row), a call that goes well is vouched for by the next one.
-struct PrevCall { uint32_t slow_rows, meta; };
-__device__ __forceinline__ PrevCall report_begin(const Params &p)
-{
-    PrevCall pc;
-    pc.slow_rows = __hip_atomic_exchange(&p.hdr->n_need, 0u, __ATOMIC_RELAXED, RS_AGENT);
-    pc.meta = a_load(&p.hdr->last_call);                 // batch size | kind << 31 of that call, 0 = none yet
-    return pc;
-}
-__device__ __forceinline__ void report_end(const Params &p, const PrevCall &pc)
-{
-    a_store(&p.hdr->last_call, (uint32_t)p.B | (p.report << 31));
-    if (p.host_words && pc.meta) {
-        const uint32_t rows = pc.meta & 0x7FFFFFFFu;
-        __hip_atomic_store(p.host_words + (pc.meta >> 31), pc.slow_rows * 2u > rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
-}
-
 #ifndef RS_STREAM_WAVES
 #define RS_STREAM_WAVES 3
 #endif
@@ -360,7 +338,7 @@ __global__ void __launch_bounds__(NT, (R <= 4 ? 5 : RS_STREAM_WAVES)) stream_ker
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    if (reporter) report_end(p, prev);
+    if (reporter) report_end(p, prev, true);
     slice_count_and_stash<R, NT, kRep, false>(p, v, s, eb, lmax, row, part, base4, nv);
 }
 
@@ -720,9 +698,9 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     const uint64_t top_k = (uint64_t)p.top_k;
     Found f = hist_find_level1<false>(s, top_k, p.top_p, lane, wave);
     const u128 D = s.D, P = s.P;
-    // What the stashes cannot finish, this workgroup does alone from the logits (three-launch path).
-    // Such rows are counted, and once they are most of the call's the caller's policy is told at once
-    // (that calls went well is reported by the next streaming call, see finish_kernel).
+    // What the stashes cannot finish, this workgroup does alone from the logits.  Such rows are
+    // counted, and the first of a call tells the caller's policy at once (that a call went well is
+    // reported by the call after it, see report_begin).
     auto slow = [&]() -> bool {
         if (drawer) {                                    // the row is finished here: this draw is used up
             rng_st[2] = rs[2] + 1u;
@@ -731,7 +709,7 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         finish_row_slow(p, s, t, row, xmax, p.inj_u ? 0ull : t.rand64);
         if (tid == 0) {
             const uint32_t c = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
-            if ((c + 1u) * 2u > (uint32_t)p.B && c * 2u <= (uint32_t)p.B && p.host_words)
+            if (c == 0u && p.host_words)                 // the call's first such row tells the caller's policy at once
                 __hip_atomic_store(p.host_words + p.report, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
         return true;
@@ -1014,7 +992,7 @@ __global__ void __launch_bounds__(kThreads, 2) stream_pen_kernel(const Params p,
     Slice<R, true> sl;
     slice_setup(p, sl, row, part, G);
     const float lmax = slice_load(p, sl);
-    if (reporter) report_end(p, prev);
+    if (reporter) report_end(p, prev, true);
     slice_count_and_stash<R, kThreads, kRep, false>(p, v, s, sl.eb, lmax, row, part, sl.base4, sl.nv);
 }
 

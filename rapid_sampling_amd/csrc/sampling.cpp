@@ -344,6 +344,27 @@ int64_t policy_state(std::optional<int64_t> device)
     return st;
 }
 
+// Forgets what the current stream's calls have learnt about routing: synchronises the stream, sets
+// the workspace up again (so that the next streaming call does not report on the last one) and
+// replaces the policy object.  For measurements that change workload on one stream and want each
+// workload from a clean start; a service with one workload per stream never needs it.
+void reset_routing(std::optional<int64_t> device)
+{
+    const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+    auto like = at::empty({1}, at::TensorOptions().dtype(at::kChar).device(dev));
+    void *stream = current_stream(like);
+    if (is_capturing(stream)) throw std::runtime_error("rapid_sampling: reset_routing while the stream is being captured");
+    Entry &e = entry_for((int)dev.index(), stream);
+    if (!e.ws.defined()) return;
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) throw std::runtime_error("rapid_sampling: stream synchronisation failed");
+    rs_policy *fresh = nullptr;
+    if (rs_policy_create(&fresh) != RS_OK) throw std::runtime_error("rapid_sampling: could not allocate the pinned host words of the workspace");
+    if (e.policy) rs_policy_destroy(e.policy);
+    e.policy = fresh;
+    init_workspace(e, stream);
+}
+
 // Shortens (milliseconds > 0) or restores (0) the bound of the kernels' waits on the current
 // stream's workspace.  For tests of the error path.
 void set_wait_limit(int64_t milliseconds, std::optional<int64_t> device)
@@ -411,6 +432,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("workspace_status", &workspace_status, py::arg("device") = py::none());
     m.def("policy_state", &policy_state, py::arg("device") = py::none());
     m.def("force_path", &force_path, py::arg("name"));
+    m.def("reset_routing", &reset_routing, py::arg("device") = py::none());
     m.def("debug_workspace", &debug_workspace, py::arg("device") = py::none());
     m.def("set_wait_limit", &set_wait_limit, py::arg("milliseconds"), py::arg("device") = py::none());
     m.attr("STATE_BYTES_PER_ROW") = RS_STATE_BYTES_PER_ROW;

@@ -769,24 +769,30 @@ def test_python_module_drop_in_calls(torch_cuda, oracle):
 
 def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     """top_k disabled, top_p < 1: the wait-free path is an attempt.  With a policy it is made; peaked rows
-    finish on it from the stashes (diag.rounds == 0).  A call whose rows mostly had to be done the slow
-    way (flat rows: the finishing workgroup goes through the logits again, diag.rounds == 8) says so in
-    the policy's report word at once, and the next calls go straight to the general kernel; that a call
-    went well is reported by the streaming call after it.  Without a policy no attempts are made.  Every
-    result equals the oracle's whatever the route."""
+    finish on it from the stashes (diag.rounds == 0).  A call with a row that had to be done the slow
+    way (a flat row: the finishing workgroup goes through the logits again, diag.rounds == 8) says so in
+    the policy's report word at once, and the next calls go to the general kernel; streaming is tried
+    again after 64 of them, then 128, 256, ...; that a call went well is reported by the call after it,
+    whichever kernel that is.  Without a policy no attempts are made.  Every result equals the
+    oracle's whatever the route."""
     torch = torch_cuda
     import ctypes as C
     from tests import capi
-    B, V = 600, 65536                                    # too many slices for the one-launch path: three launches, routed
+    B, V = 600, 65536
     peaked = H.logits_normal(B, V, 3.0, seed=90)
     flat = H.logits_uniform(B, V, seed=91)
+    mixed = peaked.copy()
+    mixed[7] = flat[7]                                   # one flat row among 600
     rc, c, k, p = capi.normalize(1.0, -1, 0.3, V, B, 1)
     assert k == V
     u_np = H.uniforms(B, 92)
     u = torch.from_numpy(u_np).cuda()
     ref_peaked = oracle.sample_batch(peaked, c, k, p, injected_u=u_np)
     ref_flat = oracle.sample_batch(flat, c, k, p, injected_u=u_np)
-    lg_peaked, lg_flat = torch.from_numpy(peaked).cuda(), torch.from_numpy(flat).cuda()
+    ref_mixed = (ref_peaked[0].copy(), ref_peaked[1].copy())
+    ref_mixed[0][7] = ref_flat[0][7]
+    ref_mixed[1][7] = ref_flat[1][7]
+    lg_peaked, lg_flat, lg_mixed = (torch.from_numpy(a).cuda() for a in (peaked, flat, mixed))
 
     def policy(smp):
         return smp.policy_state()
@@ -801,23 +807,38 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)
     _check(res, *ref_peaked, "attempt on peaked rows")
     assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
-    res = smp.sample(lg_flat, c, k, p, uniforms=u)       # attempted, every row handed on
-    _check(res, *ref_flat, "attempt on flat rows")
-    assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 1
+    res = smp.sample(lg_mixed, c, k, p, uniforms=u)      # attempted, one row done the slow way
+    _check(res, *ref_mixed, "attempt with one flat row")
+    assert res["diag"]["rounds"][7] == 8 and (np.delete(res["diag"]["rounds"], 7) == 0).all() and policy(smp) == 1
     for i in range(3):                                   # no further attempts for now, peaked or not
         res = smp.sample(lg_peaked, c, k, p, uniforms=u)
         _check(res, *ref_peaked, "after a failed attempt %d" % i)
         assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 1
-    for i in range(520):                                 # one call in 256 tries again; the second such call vouches for the first
+    for i in range(64):                                  # 64 calls away, a try that goes well, the call after it says so
         res = smp.sample(lg_peaked, c, k, p, uniforms=u, want_diag=False)
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
     assert policy(smp) == 0
+    res = smp.sample(lg_peaked, c, k, p, uniforms=u)
+    assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
+    # rows that are always too flat: the next try after 128 calls on the general kernel (a failed try doubles the stay)
+    streamed = []
+    for i in range(135):
+        res = smp.sample(lg_flat, c, k, p, uniforms=u)
+        assert res["rc"] == 0 and np.array_equal(res["out"], ref_flat[0])
+        if (res["diag"]["rounds"] == 8).all():
+            streamed.append(i)
+        else:
+            assert (res["diag"]["rounds"] < 8).all() and (res["diag"]["rounds"] >= 1).all()
+        assert policy(smp) == 1
+    assert streamed == [0, 129], streamed
     assert smp.status() == 0
+    smp.close()
+    smp = capi.Sampler(B, V, with_policy=True, init=True)
 
     # The same for calls WITH a bounding top_k, which stream unless told otherwise: rows whose every
     # other token ties at the top cannot be finished from the stashes (the tie is larger than any
-    # stash, and it is not the whole row) and are handed on, the report says so (bit 1), the next
-    # calls skip the streaming pass, and one in 64 streams again.
+    # stash, and it is not the whole row) and are done the slow way, the report says so (bit 1), the
+    # next calls skip the streaming pass, and after 64 of them streaming is tried again.
     ties = np.zeros((B, V), dtype=np.float32)
     ties[:, ::2] = 1.0
     rc, c, k, p = capi.normalize(1.0, 10, 1.0, V, B, 1)
@@ -827,13 +848,13 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)
     _check(res, *ref_peaked, "bounded, peaked rows")
     assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
-    res = smp.sample(lg_ties, c, k, p, uniforms=u)       # streamed, every row handed on
+    res = smp.sample(lg_ties, c, k, p, uniforms=u)       # streamed, every row done the slow way
     _check(res, *ref_ties, "bounded, rows of ties")
     assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 2
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)     # not streamed
     _check(res, *ref_peaked, "bounded, after rows of ties")
     assert (res["diag"]["rounds"] >= 1).all() and policy(smp) == 2
-    for i in range(520):
+    for i in range(66):
         res = smp.sample(lg_peaked, c, k, p, uniforms=u, want_diag=False)
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_peaked[0])
     assert policy(smp) == 0
