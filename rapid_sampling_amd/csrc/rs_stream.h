@@ -23,8 +23,8 @@ namespace rs {
 //                   tokens at or above it (or, for flat rows, the stashes
 //                   whole), resolves the threshold on them and picks.  A row
 //                   that cannot be finished from the stashes (a huge tie, a
-//                   nucleus of thousands of tokens) is put on a list, and the
-//                   cluster kernel then runs for the listed rows.
+//                   nucleus of thousands of tokens) it does alone, from the
+//                   logits (finish_row_slow).
 // Lanes of a wave that add to one LDS address are served one after the other, and rows often put
 // most of their tokens into a few bins.  So each bin is kept in kRep copies (lane l adds to copy
 // l % kRep), and e is not clamped before it is counted: the histogram spans all 512 values of
@@ -52,7 +52,7 @@ struct LdsA {
 #ifndef RS_STREAM_WAVES
 #define RS_STREAM_WAVES 3
 #endif
-// Stores of per-slice data: plain for the three-launch streaming path (the kernel boundary makes
+// Stores of per-slice data: plain for the streaming path of separate launches (the kernel boundary makes
 // them visible), device-scope atomic stores for the one-launch path, whose finishing workgroup
 // reads them while the kernel is still running.
 template <bool FUSED, typename T> __device__ __forceinline__ void put(T *p, T v)
@@ -584,11 +584,11 @@ __device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t
 }
 
 // Finishes a row from what its slices published.  Returns true when the row is done (token written),
-// false when it cannot be finished from the stashes: the three-launch path (FUSED = false) has then
-// put the row on the list for the cluster kernel; on the one-launch path (FUSED = true: the caller is
-// the last workgroup of the row to publish, the data was written by workgroups of this same launch
-// and is read with device-scope atomic loads) the caller tells the row's other workgroups, and the
-// row's histogram is left in place for them.
+// false when it cannot be finished from the stashes: only on the one-launch path (FUSED = true: the
+// caller is the last workgroup of the row to publish, the data was written by workgroups of this same
+// launch and is read with device-scope atomic loads), where the caller then tells the row's other
+// workgroups and the row's histogram is left in place for them.  With FUSED = false such a row is
+// done here the slow way, from the logits.
 template <int SLICE_LOG2, bool FUSED>     // SLICE_LOG2: log2 of the tokens per slice of the view
 __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v, Lds &s, LdsB &t, const uint32_t row)
 {

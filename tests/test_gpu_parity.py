@@ -248,7 +248,7 @@ def test_streaming_path_mixed_rows(torch_cuda, oracle):
     lg[8, 20000:20600] = 9.0                             # a tie of 600 tokens at the top
     for (k, p) in [(50, 0.9), (1024, 0.95), (1, 1.0), (1000, 0.2), (7, 1.0), (1024, 1.0)]:
         _run_case(torch_cuda, oracle, capi, lg, 0.9, k, p, u_np=H.uniforms(10, 91), what="stream mixed k=%s p=%s" % (k, p))
-    # which rows the streaming path finished itself (diag.rounds == 0) and which it handed on
+    # which rows the streaming path finished from the stashes (diag.rounds == 0) and which the slow way
     rc, c, k, p = capi.normalize(0.9, 50, 0.9, V, 10, 1)
     res = capi.Sampler(10, V).sample(torch_cuda.from_numpy(lg).cuda(), c, k, p, path="stream",
                                      uniforms=torch_cuda.from_numpy(H.uniforms(10, 91)).cuda())
@@ -320,7 +320,7 @@ def test_streaming_path_flat_distributions(torch_cuda, oracle):
     rounds = res["diag"]["rounds"]
     assert all(rounds[i] == 0 for i in (1, 2, 3, 4, 6)), rounds     # finished from the stashes
     assert rounds[0] == 0, rounds                                   # all equal: one tie, recognised as such
-    # handed on: a row so flat that even a level-2 sub-bin holds more tokens than a stash
+    # the slow way: a row so flat that even a level-2 sub-bin holds more tokens than a stash
     assert rounds[5] >= 1, rounds
 
 
