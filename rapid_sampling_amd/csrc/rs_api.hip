@@ -119,8 +119,11 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
     const int maxR = pen ? 16 : 32;
     auto parts = [&](int R) { return (V4 + (uint32_t)(kThreads * R) - 1) / (uint32_t)(kThreads * R); };
     if (force_r) {
+        // (a row of more than 64 workgroups only while the whole launch fits the GPU at once: one XCD
+        // holds 64 workgroups of the largest variants, and a row's workgroups wait for each other)
         const int R = force_r;
-        if ((R == 1 || R == 2 || R == 4 || R == 8 || R == 16 || R == 32) && R <= maxR && parts(R) <= (uint32_t)kMaxParts)
+        if ((R == 1 || R == 2 || R == 4 || R == 8 || R == 16 || R == 32) && R <= maxR && parts(R) <= (uint32_t)kMaxParts &&
+            (parts(R) <= 64u || (uint64_t)B * parts(R) <= 512u))
             return {R, parts(R)};
     }
     // Measured on MI355X: a cluster works best with at most ~64 workgroups (each exchange costs
@@ -485,14 +488,19 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         const uint32_t est = 2u * max(kk + 512u, whole <= (uint32_t)kFinCap ? whole : 0u);
         v.list_cap = 2048u;
         while (v.list_cap < est && v.list_cap < (uint32_t)kFinCap) v.list_cap *= 2u;
-        // the one-launch path keeps a list of 2048 tokens in LDS it holds anyway; a longer one costs every
-        // workgroup of the call dynamic LDS (fewer workgroups per CU), so it is only taken when even a
-        // well-behaved row would not fit 2048 (a row that then needs more falls back inside the kernel)
-        if (path == kPathFused && est / 2u <= 2048u) v.list_cap = 2048u;
+        // The one-launch path keeps its list, 2048 tokens, in static LDS it holds anyway, and never more
+        // (a row that needs more falls back inside the kernel).  Its workgroups wait for each other, and
+        // the hardware binds workgroup b to XCD b mod 8 before it starts: towards the end of a launch
+        // the workgroups still to start may all belong to one XCD, and if that XCD's compute units were
+        // all held by waiting workgroups of the row they belong to, nobody would ever move.  So a row
+        // (at most 64 slices here) must be smaller than what ONE XCD holds: 32 CUs x 2 or 3 workgroups
+        // with static LDS alone -- with a 64 KB list in dynamic LDS it was 32 x 1, and rows of 33 and
+        // more slices could, rarely, starve until their waits gave up.
+        if (path == kPathFused) v.list_cap = 2048u;
         p.report = path == kPathAttempt ? 1u : 0u;
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (path == kPathFused)
-            return launch_fused(sr, pen, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+            return launch_fused(sr, pen, (uint32_t)B, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         if (pen) {
             // penalties: read by the streaming pass (and by the finishing workgroup of a row it has to
             // do the slow way), rewritten by one pass over them at the end

@@ -378,10 +378,11 @@ __device__ __forceinline__ bool slice_finish(const Params &p, Lds &s, Slice<R, P
                     w0 = a_load(&rc->A[2 * tid]); w1 = a_load(&rc->A[2 * tid + 1]);
                     valid += (w0 & w1 & kValid) != 0;
                 }
-                guard.tick(s, p.hdr);
+                guard.tick(s, p.hdr, 3u);
                 const uint32_t total = block_sum_u32(s, valid, lane, wave);
                 if (total == ncand + G) break;
                 if (s.abort) return false;
+                if (tid == 0) { s.seen = total; s.want = ncand + G; }
             }
             if ((uint32_t)tid < G) a_mine = get_mass(w0, w1);
             // every workgroup wrote its mass after it had read the last histogram level
@@ -469,10 +470,11 @@ __device__ __forceinline__ bool slice_finish(const Params &p, Lds &s, Slice<R, P
                     w0 = a_load(&rc->A[2 * tid]); w1 = a_load(&rc->A[2 * tid + 1]);
                     valid = (w0 & w1 & kValid) != 0;
                 }
-                guard.tick(s, p.hdr);
+                guard.tick(s, p.hdr, 4u);
                 const uint32_t total = block_sum_u32(s, valid, lane, wave);
                 if (total == G) break;
                 if (s.abort) return false;
+                if (tid == 0) { s.seen = total; s.want = G; }
             }
             clear_used();
             before = block_sum_u128(s, (uint32_t)tid < part ? get_mass(w0, w1) : (u128)0, lane, wave);
@@ -531,7 +533,7 @@ __device__ __forceinline__ bool slice_finish(const Params &p, Lds &s, Slice<R, P
                 uint32_t spins = 0, v;
                 while ((v = a_load(&rc->index_p1)) == 0u) {
                     if ((++spins & 1023u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(p.hdr)) {
-                        give_up(s, p.hdr);
+                        give_up(s, p.hdr, 5u);
                         break;
                     }
                 }
@@ -589,6 +591,7 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
 {
     Slice<R, PEN> sl;
     slice_setup(p, sl, row, part, p.G);
+    if (threadIdx.x == 0) { s.who = row << 16 | part; s.seen = 0; s.want = 0; }
     // the call's first thread reports on the streaming call before it, if there was one (report_begin)
     const bool reporter = blockIdx.x == 0 && threadIdx.x == 0 && p.host_words != nullptr;
     PrevCall prev;

@@ -32,7 +32,8 @@ struct alignas(256) WsHeader {
     uint32_t n_need;      // rows of the running (or last) streaming call that the finishing workgroups did the slow way
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
     uint32_t last_call;   // 1 | kind << 31 after a streaming call that no later call has reported on yet (kind: 0 top_k bounds the kept set, 1 not), else 0
-    uint32_t pad[58];
+    uint32_t gave_up[4];  // the first wait that gave up since the workspace was set up: site, row << 16 | slice, what it had, what it waited for
+    uint32_t pad[54];
 };
 
 // How long a workgroup waits for its peers before it gives up (wall-clock ticks).
@@ -214,6 +215,7 @@ struct Lds {
     uint32_t ctr;
     int      abort;
     int32_t *host_words;     // Params::host_words, for the code that gives up a wait
+    uint32_t who, seen, want; // for the same: row << 16 | slice of this workgroup; what its current wait has and waits for
 };
 
 __device__ __forceinline__ uint32_t block_max_u32(Lds &s, uint32_t v, int lane, int wave)
@@ -267,7 +269,7 @@ __device__ __forceinline__ void block_sum2_u128(Lds &s, u128 &a, u128 &b, int la
 // A wait that ran out of time: the sticky error word of the workspace, the caller's pinned host
 // word if there is one (readable without synchronising), and the flag that makes the workgroup leave.
 struct Lds;
-__device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr);
+__device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr, uint32_t site);
 
 // Bounded wait bookkeeping: thread 0 looks at the wall clock now and then; the
 // verdict is read by everyone after a workgroup barrier, so it is uniform.
@@ -276,14 +278,20 @@ struct SpinGuard {
     uint32_t spins;
     __device__ __forceinline__ void start() { t0 = (uint64_t)wall_clock64(); spins = 0; }
     // call by every thread once per polling round, before the round's __syncthreads
-    __device__ __forceinline__ void tick(Lds &s, WsHeader *hdr)
+    __device__ __forceinline__ void tick(Lds &s, WsHeader *hdr, uint32_t site)
     {
-        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(hdr)) give_up(s, hdr);
+        if (threadIdx.x == 0 && (++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(hdr)) give_up(s, hdr, site);
     }
 };
 
-__device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr)
+// Sites of the waits: 1 a histogram level of the cluster, 2 its level 1, 3 the gathered tokens, 4 the
+// kept masses, 5 the sampled index, 6 the verdict of the one-launch path.
+__device__ __forceinline__ void give_up(Lds &s, WsHeader *hdr, uint32_t site)
 {
+    uint32_t none = 0u;
+    if (__hip_atomic_compare_exchange_strong(&hdr->gave_up[0], &none, site, __ATOMIC_RELAXED, __ATOMIC_RELAXED, RS_AGENT)) {
+        a_store(&hdr->gave_up[1], s.who); a_store(&hdr->gave_up[2], s.seen); a_store(&hdr->gave_up[3], s.want);
+    }
     a_store(&hdr->error, (int32_t)RS_ERR_DEVICE);
     if (s.host_words) __hip_atomic_store(s.host_words + 2, (int32_t)RS_ERR_DEVICE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     s.abort = 1;
@@ -358,10 +366,11 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
             s.g[b] = w;
             c += pack_count(w);
         }
-        guard.tick(s, hdr);
+        guard.tick(s, hdr, 1u);
         const uint32_t total = block_sum_u32(s, c, lane, wave);
         if (total == expected) return true;
         if (s.abort) return false;
+        if (threadIdx.x == 0) { s.seen = total; s.want = expected; }
     }
 }
 
@@ -398,7 +407,7 @@ __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G,
             nkey = ~key;
             c += key == 0u ? 1u << 24 : 0u;
         }
-        guard.tick(s, hdr);
+        guard.tick(s, hdr, 2u);
         c = wave_sum(c); key = wave_max_u32(key); nkey = wave_max_u32(nkey);
         __syncthreads();
         if (lane == 0) { s.u32[wave] = c; s.u32[kWaves + wave] = key; s.u32[2 * kWaves + wave] = nkey; }
@@ -411,6 +420,7 @@ __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G,
         }
         if (total == expected) break;
         if (s.abort) return -1;
+        if (tid == 0) { s.seen = total; s.want = expected; }
     }
     kmin = ~kmin;
     kmax_out = kmax;
@@ -629,7 +639,6 @@ hipError_t launch_stream_pen(uint32_t B, size_t finish_lds_bytes, hipStream_t st
 hipError_t launch_penalty_pass(hipStream_t st, const Params &p);
 hipError_t launch_stream(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
                          const StreamView &v);
-hipError_t launch_fused(int slice_r, bool pen, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
-                        const StreamView &v);
+hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v);
 
 }  // namespace rs

@@ -1119,7 +1119,6 @@ __global__ void __launch_bounds__(kThreads, 2) fused_kernel(const Params p, cons
     constexpr int kSliceLog2 = R == 16 ? 14 : R == 8 ? 13 : 12;
     static_assert(R == 4 || R == 8 || R == 16, "slices of 4096, 8192 or 16384 tokens");
     __shared__ FusedLds<R, PEN> u;
-    extern __shared__ __align__(16) unsigned char fused_dyn[];
     const int tid = threadIdx.x;
     const uint32_t G = v.G;
     // logical id: the hardware's while the whole launch fits the GPU at once, else a ticket, so that
@@ -1158,13 +1157,13 @@ __global__ void __launch_bounds__(kThreads, 2) fused_kernel(const Params p, cons
     __syncthreads();                                     // the LDS of the streaming pass is given up here
     Lds &s = u.f.s;
     LdsB &t = u.f.t;
-    if (tid == 0) { s.abort = 0; s.host_words = p.host_words; }
+    if (tid == 0) { s.abort = 0; s.host_words = p.host_words; s.who = row << 16 | part; s.seen = 0; s.want = 0; }
     uint32_t verdict = 0;
     if (last) {
-        // the token list: the cluster rounds' histogram copies (not in use while a row is finished from
-        // the stashes) when it fits them, else dynamic LDS
+        // the token list: the cluster rounds' histogram copies, which are not in use while a row is
+        // finished from the stashes (no dynamic LDS in this kernel: see rs_sample_ex)
         static_assert(sizeof(s.hr) == 2048 * sizeof(uint64_t), "room for a list of 2048 tokens");
-        t.list = v.list_cap <= 2048u ? s.hr : reinterpret_cast<uint64_t *>(fused_dyn);
+        t.list = s.hr;
         const bool done = finish_row<kSliceLog2, true>(p, v, s, t, row);
         __syncthreads();
         verdict = done && t.result != 0u ? t.result : kVerdictFallback;
@@ -1176,7 +1175,7 @@ __global__ void __launch_bounds__(kThreads, 2) fused_kernel(const Params p, cons
             uint32_t spins = 0, w;
             while ((w = a_load(&rc->verdict)) == 0u) {
                 __builtin_amdgcn_s_sleep(2);
-                if ((++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(p.hdr)) { give_up(s, p.hdr); break; }
+                if ((++spins & 255u) == 0 && (uint64_t)wall_clock64() - t0 > spin_limit(p.hdr)) { give_up(s, p.hdr, 6u); break; }
             }
             s.bc32[7] = w;
         }

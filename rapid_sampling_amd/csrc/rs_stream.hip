@@ -37,13 +37,12 @@ hipError_t launch_penalty_pass(hipStream_t st, const Params &p)
     return hipGetLastError();
 }
 
-hipError_t launch_fused(int slice_r, bool pen, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
-                        const StreamView &v)
+hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v)
 {
     const dim3 grid(B * v.G), block(kThreads);
-    const size_t dyn = v.list_cap <= 2048u ? 0 : finish_lds_bytes;      // a short list lives in static LDS
-#define RS_FUSED(Rv) do { if (pen) hipLaunchKernelGGL((fused_kernel<Rv, true>), grid, block, dyn, st, p, v);          \
-                          else hipLaunchKernelGGL((fused_kernel<Rv, false>), grid, block, dyn, st, p, v); } while (0)
+    if (v.list_cap > 2048u) return hipErrorInvalidValue;      // the list lives in static LDS
+#define RS_FUSED(Rv) do { if (pen) hipLaunchKernelGGL((fused_kernel<Rv, true>), grid, block, 0, st, p, v);          \
+                          else hipLaunchKernelGGL((fused_kernel<Rv, false>), grid, block, 0, st, p, v); } while (0)
     switch (slice_r) {
     case 4:  RS_FUSED(4); break;
     case 8:  RS_FUSED(8); break;

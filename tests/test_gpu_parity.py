@@ -616,6 +616,40 @@ def test_c4_penalty_chain(torch_cuda, oracle, steps):
     assert smp.status() == 0
 
 
+
+def test_one_launch_path_rows_of_more_slices_than_an_xcd_has_compute_units(torch_cuda, oracle):
+    """The workgroups of the one-launch path wait for each other, and the hardware binds workgroup b to
+    XCD b mod 8 before it starts.  With its token list in dynamic LDS the kernel ran one workgroup per
+    compute unit, 32 per XCD, and a row of 47 slices whose last workgroups all belonged to one XCD could
+    starve until its waits gave up (one call in some hundred, always the last row).  The list now always
+    lives in static LDS.  The shape and the sequence of calls that showed it, 300 times over, with a wait
+    limit of 50 ms so that a starved row would show at once."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 11, 191104
+    rng = np.random.default_rng(5)
+    rows = []
+    for _ in range(B):
+        r = rng.standard_normal(V, dtype=np.float32)
+        lo = int(rng.integers(0, V))
+        n = int(rng.integers(1, V // 2))
+        r[lo: lo + n] = float(r.max()) + float(rng.choice([0.0, 0.25, 2.0]))     # a run of ties at the top
+        rows.append(r)
+    lg = np.stack(rows)
+    rc, c, k, p = capi.normalize(0.5, 1000, 0.0, V, B, 1)                        # top_p 0: greedy
+    u_np = H.uniforms(B, 77)
+    ref_out, ref_diag = oracle.sample_batch(lg, c, k, p, injected_u=u_np)
+    smp = capi.Sampler(B, V)
+    smp.set_wait_limit(50)
+    lgt, u = torch.from_numpy(lg).cuda(), torch.from_numpy(u_np).cuda()
+    for it in range(300):
+        for path in ("cluster", "stream", "optimistic", "fused"):
+            res = smp.sample(lgt, c, k, p, uniforms=u, path=path, want_diag=(it % 50 == 0))
+            assert res["rc"] == 0 and np.array_equal(res["out"], ref_out), "iteration %d path %s" % (it, path)
+            if it % 50 == 0:
+                _check(res, ref_out, ref_diag, "iteration %d path %s" % (it, path))
+        assert smp.status() == 0, "iteration %d" % it
+
 @pytest.mark.parametrize("B,V,steps", [(96, 152064, 3), (128, 1048576, 2)])
 def test_penalties_at_scale_streaming_pass(torch_cuda, oracle, B, V, steps):
     """Calls with penalties too large for the one-launch path (more workgroups than the GPU holds at once)
