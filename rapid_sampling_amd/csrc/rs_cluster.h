@@ -607,13 +607,15 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
 // Workgroups take their (row, slice) from a ticket counter, so that logical ids follow the order in
 // which workgroups actually start and a row's workgroups are the next ones to start.  The workgroups
 // of a row wait for EACH OTHER (every exchange is all-to-all within the row, so a low ticket waits for
-// higher ones too): the waits end because a row has at most 256 workgroups and a workgroup, once
-// started, runs to its end without giving up its compute unit -- the dispatcher starts workgroups in
-// ticket order as room becomes free, so all workgroups of the oldest unfinished row are resident or
-// next in line.  That needs room for one whole row of workgroups on the GPU: 256 compute units with
-// at least one workgroup each hold it; a device partitioned below that, or shared with another
-// process's long-running kernels, can starve a row -- the waits are bounded for that case and end in
-// RS_ERR_DEVICE rather than a hang.
+// higher ones too).  The waits end because a workgroup, once started, runs to its end without giving
+// up its compute unit; because the workgroups that have started are, at any time, all of the earlier
+// rows (which finish and leave) and the first part of one unfinished row; and because the rest of
+// that row can always start: the hardware binds workgroup b of a launch to XCD b mod 8 before it
+// starts, so towards the end of a launch the workgroups still to start may all belong to one XCD, and
+// a row must therefore have fewer workgroups than ONE XCD holds (32 compute units x at least 2
+// workgroups of this kernel: the host cuts rows into at most 64).  A device partitioned below that,
+// or shared with other long-running kernels, can starve a row -- the waits are bounded for that case
+// and end in RS_ERR_DEVICE rather than a hang.
 template <int R, bool PEN>
 __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
 {
