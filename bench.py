@@ -12,7 +12,9 @@ stream the kernel runs on).  Next to it, in the same JSON line:
 
   latency    the launch-plus-one-read floor kernel timed the same way, the
              ratio to it, the wall-clock "call + synchronize" time the
-             reference's own bench measures (reference bench.py:84-92), and
+             reference's own bench measures (reference bench.py:84-92) for the
+             call and for the floor kernel (what a launch and a synchronize
+             cost on this host whatever the kernel does), and
              `readme_point`: the one point the reference publishes
              (README.md:21-31: same shape, logits U[0,1)*4)
   roofline   the bandwidth-bound configuration (BASELINE.json configs[4]):
@@ -182,6 +184,7 @@ def main():
     floor_us, _ = event_times_us(torch, floor, min(args.steps, 2000), min(args.warmup, 100))
     floor_p50 = statistics.median(floor_us)
     sync_us = sync_call_us(torch, call, 200)
+    floor_sync_us = sync_call_us(torch, floor, 200)
     b2b_us = block_time_us(torch, call, min(args.steps, 2000), 20)
     floor_b2b_us = block_time_us(torch, floor, min(args.steps, 2000), 20)
 
@@ -221,6 +224,7 @@ def main():
             "floor_p50_us": round(floor_p50, 3), "floor_back_to_back_us": round(floor_b2b_us, 3),
             "ratio_to_floor": round(p50 / floor_p50, 3),
             "call_plus_sync_p50_us": round(statistics.median(sync_us), 2),
+            "floor_call_plus_sync_p50_us": round(statistics.median(floor_sync_us), 2),
             "reference_call_plus_sync_us": 220.3,
             "reference_note": "reference README.md:21-31: same B, V, top_p, top_k, logits U[0,1)*4, unnamed NVIDIA GPU",
             "readme_point": {

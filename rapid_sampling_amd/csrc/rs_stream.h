@@ -47,7 +47,6 @@ struct LdsA {
     uint32_t sub[128];           // level-2 counts inside a boundary bin too large for the stash
     uint32_t u32[16];
     uint32_t cov, n, cut, over;
-    uint32_t ngrp;               // float4 groups staged so far
 };
 
 #ifndef RS_STREAM_WAVES
@@ -177,7 +176,6 @@ __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const
         }
     }
     if (tid < 128) s.sub[tid] = 0;
-    if (tid == 128) s.ngrp = 0;
     __syncthreads();
     if (s.over != 0xFFFFFFFFu) {
         // The bin in which the count reaches stash_k holds far more tokens than asked for (a flat
@@ -225,21 +223,33 @@ __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const
     // 2^-40: dead tokens are no candidates.
 
     // Candidates (bits >= cut) are at most n <= kStashCap, so at most that many float4 groups
-    // hold one.  A thread copies each of its groups with a candidate into LDS at the next free
-    // place (a counter in LDS: few groups hold one, so few lanes ever ask); the tokens of those
-    // groups are then gone through densely.  The histogram, whose memory this is, is done with.
+    // hold one.  Each thread copies its groups with a candidate into LDS at an offset from a scan
+    // of the per-thread counts; the tokens of those groups are then gone through densely.
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+        mine += max(max(eb[j * 4], eb[j * 4 + 1]), max(eb[j * 4 + 2], eb[j * 4 + 3])) >= cut ? 1u : 0u;
+    uint32_t o = wave_inclusive_scan(mine);
+    if (lane == kWave - 1) s.u32[wave] = o;
+    __syncthreads();
+    uint32_t ngroups = 0;
+#pragma unroll
+    for (int w = 0; w < (NT / kWave); ++w) {
+        if (w < wave) o += s.u32[w];
+        ngroups += s.u32[w];
+    }
+    o -= mine;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         if (max(max(eb[j * 4], eb[j * 4 + 1]), max(eb[j * 4 + 2], eb[j * 4 + 3])) >= cut) {
-            const uint32_t o = atomicAdd(&s.ngrp, 1u);
             if (o < (uint32_t)kStashCap) {
                 s.grp[o] = make_uint4(eb[j * 4], eb[j * 4 + 1], eb[j * 4 + 2], eb[j * 4 + 3]);
                 s.gidx[o] = (base4 + (uint32_t)j * NT) * 4;
             }
+            ++o;
         }
     }
     __syncthreads();
-    const uint32_t ngroups = s.ngrp;
     // Write the candidates out grouped by bin, largest e first, so that the finishing
     // workgroup can take a prefix.
     uint64_t *st = v.stash + ((size_t)row * G + part) * kStashCap;
