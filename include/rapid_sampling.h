@@ -118,6 +118,16 @@ int rs_workspace_set_wait_limit(void *workspace_device, uint32_t milliseconds, v
 int rs_workspace_status(const void *workspace_device, int32_t *status, void *stream);
 
 /*
+ * Where the first wait that gave up was (synchronises `stream`; no counterpart
+ * in the reference).  where[0] = the wait (0 none; 1 a histogram level,
+ * 2 the first level's totals, 3 the candidates of a level, 4 the masses,
+ * 5 the index, 6 the verdict of the one-launch kernel), where[1] =
+ * row << 16 | slice of the workgroup that gave up, where[2] and where[3] = what
+ * it had seen and what it waited for.  Cleared by rs_workspace_init.
+ */
+int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *stream);
+
+/*
  * Routing state of the streaming path and an asynchronous error report, owned
  * by the caller (optional; one per workspace).  No counterpart in the
  * reference.

@@ -360,6 +360,16 @@ int rs_workspace_status(const void *ws, int32_t *status, void *stream)
     return RS_OK;
 }
 
+int rs_workspace_where(const void *ws, uint32_t where[4], void *stream)
+{
+    if (!ws || !where) return RS_ERR_NULL;
+    const WsHeader *h = (const WsHeader *)ws;
+    if (hipMemcpyAsync(where, h->gave_up, sizeof h->gave_up, hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+        return RS_ERR_LAUNCH;
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return RS_ERR_LAUNCH;
+    return RS_OK;
+}
+
 int rs_policy_create(rs_policy **out)
 {
     if (!out) return RS_ERR_NULL;

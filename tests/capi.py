@@ -60,6 +60,8 @@ def lib():
         L.rs_workspace_init.argtypes = [vp, sz, vp]
         L.rs_workspace_status.restype = C.c_int
         L.rs_workspace_status.argtypes = [vp, C.POINTER(i32), vp]
+        L.rs_workspace_where.restype = C.c_int
+        L.rs_workspace_where.argtypes = [vp, C.POINTER(C.c_uint32), vp]
         L.rs_philox_init.restype = C.c_int
         L.rs_philox_init.argtypes = [vp, C.c_uint64, i32, vp]
         L.rs_sample.restype = C.c_int
@@ -143,6 +145,13 @@ class Sampler:
         rc = lib().rs_workspace_status(self.ws.data_ptr(), C.byref(st), self.stream())
         assert rc == 0
         return st.value
+
+    def where(self):
+        """(wait, row, slice, seen, wanted) of the first wait that gave up; wait 0 = none."""
+        w = (C.c_uint32 * 4)()
+        rc = lib().rs_workspace_where(self.ws.data_ptr(), w, self.stream())
+        assert rc == 0
+        return int(w[0]), int(w[1]) >> 16, int(w[1]) & 0xffff, int(w[2]), int(w[3])
 
     def sample(self, logits, c, top_k, top_p, *, rng=None, uniforms=None, penalties=None,
                presence=0.0, repetition=0.0, decay=1.0, want_diag=True, want_e=False, path=None, force_r=None,

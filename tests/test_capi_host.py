@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     L = capi.lib()
     names = _declared_functions()
     assert {"rs_sample", "rs_philox_init", "rs_workspace_bytes", "rs_workspace_init", "rs_normalize_args",
-            "rs_workspace_status", "rs_error_string", "rs_version", "rs_floor_read"} <= set(names)
+            "rs_workspace_status", "rs_workspace_where", "rs_error_string", "rs_version", "rs_floor_read"} <= set(names)
     for n in names:
         assert hasattr(L, n), n
     assert L.rs_version() >= 100

@@ -966,9 +966,11 @@ def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
     assert res["rc"] == 0                       # the launch itself is fine
     assert smp.policy_error() == -9             # reported to the host without a device read
     assert smp.status() == -9                   # RS_ERR_DEVICE, sticky
+    wait, row, slc, seen, want = smp.where()    # the first wait that gave up: a histogram that never added up
+    assert wait in (1, 2) and row < B and seen != want, (wait, row, slc, seen, want)
     smp.reinit()
     assert smp.policy_error(clear=True) == -9 and smp.policy_error() == 0
-    assert smp.status() == 0
+    assert smp.status() == 0 and smp.where()[0] == 0
     res = smp.sample(lg, c, k, p, uniforms=u)
     _check(res, ref_out, ref_diag, "after re-initialisation")
     assert smp.status() == 0 and smp.policy_error() == 0
