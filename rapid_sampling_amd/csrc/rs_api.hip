@@ -142,13 +142,18 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
 
 
 // Streaming geometry: workgroups of 256 threads; slices of 16384 tokens (16 float4 per thread), or
-// of 4096 tokens (4 float4) for calls of up to kStreamSmall tokens in rows of up to 262144, where a
-// shorter slice shortens the one wave of workgroups the whole pass consists of (longer rows would
-// be cut into more slices than a finishing workgroup handles quickly).
+// of 4096 tokens (4 float4) while the call's short slices all fit the device at once (256 CUs x 6
+// workgroups of that kernel; measured: up to there the short slices win 1-2.5 us per call, one more
+// workgroup than that and they lose) in rows of up to 262144 tokens (longer rows would be cut into
+// more slices than a finishing workgroup handles quickly).
 constexpr int kStreamNT = 256;
-constexpr uint64_t kStreamSmall = 1ull << 22;
-static int stream_r(int32_t B, int32_t V) { return (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144 ? 4 : kStreamLongR; }
+constexpr uint32_t kStreamSmallParts = 1536;
+constexpr uint64_t kFusedSmall = 1ull << 22;
 static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
+static int stream_r(int32_t B, int32_t V)
+{
+    return V <= 262144 && (uint64_t)B * stream_parts(V, 4) <= kStreamSmallParts ? 4 : kStreamLongR;
+}
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 struct StreamLayout { size_t hdr, cum, shist, stash, end; };
 static StreamLayout stream_layout(size_t parts, size_t base)
@@ -162,14 +167,16 @@ static StreamLayout stream_layout(size_t parts, size_t base)
     return l;
 }
 // Bytes of per-slice data a workspace for (B, V) sets aside: enough for the long slices of (B, V)
-// itself and for the short slices of any call of at most B rows that takes them (at most
-// kStreamSmall tokens: fewer than kStreamSmall / 4096 + B slices), so that the size grows with
-// B and with V and a workspace for the largest B and V serves every smaller call.
+// itself and for the short slices of any call of at most B rows that takes them (the streaming
+// path: at most kStreamSmallParts of them; the one-launch path: calls of at most kFusedSmall
+// tokens, fewer than kFusedSmall / 4096 + B slices), so that the size grows with B and with V and
+// a workspace for the largest B and V serves every smaller call.
 static size_t stream_bytes(int32_t B, int32_t V)
 {
     const size_t longs = stream_layout((size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader)).end;
     size_t small_parts = (size_t)B * stream_parts(V, 4);
-    const size_t cap = (size_t)(kStreamSmall / 4096) + (size_t)B;
+    const size_t cap = (size_t)kStreamSmallParts + (size_t)B;
+    static_assert(kStreamSmallParts >= kFusedSmall / 4096, "room for either kind of small call");
     if (small_parts > cap) small_parts = cap;
     const size_t shorts = stream_layout(small_parts, sizeof(WsHeader)).end;
     return longs > shorts ? longs : shorts;
@@ -214,12 +221,12 @@ constexpr uint64_t kPenStreamMin = 1ull << 23;
 // Its workgroups hold their compute units until their row is finished, so a call pays twice once it
 // has more workgroups than the GPU holds at a time (256 CUs x 3, x 2 for the longest slices with
 // penalties: registers): the shortest slice that keeps the call within that is taken.  Calls of up
-// to kStreamSmall tokens may use any of the three lengths (the workspace has room for their short
+// to kFusedSmall tokens may use any of the three lengths (the workspace has room for their short
 // slices), larger ones the long slices only.  `any_size` (forced by the caller): longest slices
 // whatever the number of workgroups.
 static int fused_r(int32_t B, int32_t V, bool pen, bool any_size)
 {
-    const bool small_call = (uint64_t)B * (uint64_t)V <= kStreamSmall && V <= 262144;
+    const bool small_call = (uint64_t)B * (uint64_t)V <= kFusedSmall && V <= 262144;
     const int choices[3] = {4, 8, 16};
     for (int i = small_call ? 0 : 2; i < 3; ++i) {
         const int R = choices[i];
@@ -286,7 +293,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 400; }
+int rs_version(void) { return 401; }
 
 const char *rs_error_string(int code)
 {
