@@ -141,18 +141,24 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
 }
 
 
-// Streaming geometry: workgroups of 256 threads; slices of 16384 tokens (16 float4 per thread), or
-// of 4096 tokens (4 float4) while the call's short slices all fit the device at once (256 CUs x 6
-// workgroups of that kernel; measured: up to there the short slices win 1-2.5 us per call, one more
-// workgroup than that and they lose) in rows of up to 262144 tokens (longer rows would be cut into
-// more slices than a finishing workgroup handles quickly).
+// Streaming geometry: workgroups of 256 threads.  Rows of up to 262144 tokens are cut into slices of
+// 4096 tokens (4 float4 per thread) while all of the call's slices fit the device at once, else into
+// slices of 8192 tokens while those do (256 CUs x 6 workgroups of either kernel = 1536), else into
+// slices of 16384.  Measured over forty shapes of 4-13M tokens: a pass that is one wave of workgroups
+// is 0.5-2.5 us per call faster with the shorter slices, and slower from the first workgroup beyond
+// that.  Longer rows always take slices of 16384 tokens (they would be cut into more slices than a
+// finishing workgroup handles quickly).
 constexpr int kStreamNT = 256;
 constexpr uint32_t kStreamSmallParts = 1536;
 constexpr uint64_t kFusedSmall = 1ull << 22;
 static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
-static int stream_r(int32_t B, int32_t V)
+// `pen`: the pass that also reads penalties exists for the long slices only
+static int stream_r(int32_t B, int32_t V, bool pen = false)
 {
-    return V <= 262144 && (uint64_t)B * stream_parts(V, 4) <= kStreamSmallParts ? 4 : kStreamLongR;
+    if (V > 262144) return kStreamLongR;
+    if ((uint64_t)B * stream_parts(V, 4) <= kStreamSmallParts) return 4;
+    if (!pen && (uint64_t)B * stream_parts(V, 8) <= kStreamSmallParts) return 8;
+    return kStreamLongR;
 }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 struct StreamLayout { size_t hdr, cum, shist, stash, end; };
@@ -167,10 +173,10 @@ static StreamLayout stream_layout(size_t parts, size_t base)
     return l;
 }
 // Bytes of per-slice data a workspace for (B, V) sets aside: enough for the long slices of (B, V)
-// itself and for the short slices of any call of at most B rows that takes them (the streaming
-// path: at most kStreamSmallParts of them; the one-launch path: calls of at most kFusedSmall
-// tokens, fewer than kFusedSmall / 4096 + B slices), so that the size grows with B and with V and
-// a workspace for the largest B and V serves every smaller call.
+// itself and for the shorter slices of any call of at most B rows that takes them (the streaming
+// path: at most kStreamSmallParts of them, of 4096 or of 8192 tokens; the one-launch path: calls of
+// at most kFusedSmall tokens, fewer than kFusedSmall / 4096 + B slices), so that the size grows
+// with B and with V and a workspace for the largest B and V serves every smaller call.
 static size_t stream_bytes(int32_t B, int32_t V)
 {
     const size_t longs = stream_layout((size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader)).end;
@@ -264,7 +270,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         pol->period[kind] = min(pol->period[kind] * 2u, kAwayMost);
         return false;
     };
-    if (pen && bounded && stream_r(B, V) == kStreamLongR && stream_parts(V, kStreamLongR) >= 2u) {
+    if (pen && bounded && stream_r(B, V, true) == kStreamLongR && stream_parts(V, kStreamLongR) >= 2u) {
         if (force == RS_PATH_STREAM || force == RS_PATH_ATTEMPT) return kPathStream;
         if (force == RS_PATH_AUTO && (uint64_t)B * (uint64_t)V >= kPenStreamMin && !routed_away(0)) return kPathStream;
     }
@@ -293,7 +299,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 401; }
+int rs_version(void) { return 402; }
 
 const char *rs_error_string(int code)
 {
@@ -486,7 +492,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path != kPathCluster) {
-        const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V);
+        const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V, pen);
         StreamView v;
         v.G = stream_parts(V, sr);
         const StreamLayout l = stream_layout((size_t)B * v.G, sizeof(WsHeader));
@@ -578,7 +584,7 @@ int rs_floor_read(const float *logits, int64_t row_stride, int32_t *out, int32_t
         else hipLaunchKernelGGL((floor_kernel<Rv, false>), grid, dim3(kThreads), 0, st, logits, row_stride, out, V, G); } while (0)
     if (variant >= 2) {
         // the streaming pass's own geometry
-        if (stream_r(B, V) == 4) RS_FLOOR(4); else RS_FLOOR(kStreamLongR);
+        if (stream_r(B, V) == 4) RS_FLOOR(4); else if (stream_r(B, V) == 8) RS_FLOOR(8); else RS_FLOOR(kStreamLongR);
     } else {
         switch (choose_geometry(B, V, false, 0).R) {
         case 1:  RS_FLOOR(1); break;

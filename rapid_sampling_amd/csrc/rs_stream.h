@@ -31,9 +31,10 @@ namespace rs {
 // bits >> 21, the dead tokens (below 2^-40, often most of a row) spread over the bins below
 // kBin0 by their own exponents, where nobody looks at them again.  The histogram is done with
 // before the candidates are staged, and shares their memory.
-// Eight copies for long slices; two for the short slices of small calls, where clearing and
-// folding the copies would cost more than the few tokens of a thread.
-template <int R> constexpr int stream_copies() { return R >= 8 ? 8 : 2; }
+// Eight copies for long slices; four for the middle ones, which keeps their histogram smaller than
+// the candidate staging it shares memory with (six workgroups per CU); two for the short slices of
+// small calls, where clearing and folding the copies would cost more than the few tokens of a thread.
+template <int R> constexpr int stream_copies() { return R > 8 ? 8 : R == 8 ? 4 : 2; }
 template <int kRep>
 struct LdsA {
     union {
@@ -277,7 +278,7 @@ __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const
 }
 
 template <int R, int NT, int DT>     // NT threads, each with R groups of four tokens of the slice; DT the logits' type
-__global__ void __launch_bounds__(NT, (R <= 4 ? 5 : RS_STREAM_WAVES)) stream_kernel(const Params p, const StreamView v)
+__global__ void __launch_bounds__(NT, (R <= 8 ? 5 : RS_STREAM_WAVES)) stream_kernel(const Params p, const StreamView v)
 {
     constexpr int kRep = stream_copies<R>();
     __shared__ LdsA<kRep> s;

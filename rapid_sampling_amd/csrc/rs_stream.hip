@@ -14,6 +14,11 @@ hipError_t launch_stream(int slice_r, int32_t dtype, uint32_t B, size_t finish_l
         else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);
         else hipLaunchKernelGGL((stream_kernel<4, kStreamNT, RS_DTYPE_F16>), sgrid, sblock, 0, st, p, v);
         hipLaunchKernelGGL((finish_kernel<12>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v);
+    } else if (slice_r == 8) {
+        if (dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<8, kStreamNT, RS_DTYPE_F32>), sgrid, sblock, 0, st, p, v);
+        else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<8, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);
+        else hipLaunchKernelGGL((stream_kernel<8, kStreamNT, RS_DTYPE_F16>), sgrid, sblock, 0, st, p, v);
+        hipLaunchKernelGGL((finish_kernel<13>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v);
     } else {
         if (dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<kStreamLongR, kStreamNT, RS_DTYPE_F32>), sgrid, sblock, 0, st, p, v);
         else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<kStreamLongR, kStreamNT, RS_DTYPE_BF16>), sgrid, sblock, 0, st, p, v);

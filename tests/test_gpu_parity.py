@@ -397,6 +397,25 @@ def test_cluster_levels_with_slices_that_hold_no_boundary_tokens(torch_cuda, ora
             _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="contiguous ties k=%s p=%s T=%s #%d" % (k, p, t, rep))
 
 
+@pytest.mark.parametrize("fmt", ["float32", "bfloat16", "float16"])
+def test_streaming_path_middle_slices(torch_cuda, oracle, fmt):
+    """Calls whose 4096-token slices no longer fit the device at once but whose 8192-token slices do
+    (here 52 rows of 150 000 tokens: 1924 short slices, 988 middle ones) take the streaming pass with
+    slices of 8192 tokens: rows of every kind the seeded generator makes, the last slice ragged, in
+    all three logit formats, through every path."""
+    torch = torch_cuda
+    from tests import capi
+    dtype = None if fmt == "float32" else getattr(torch, fmt)
+    rng = np.random.default_rng(8192)
+    B, V = 52, 150000
+    lg = np.stack([_random_row(rng, b % 11, V) for b in range(B)])
+    if dtype is not None:
+        lg = torch.from_numpy(lg).to(dtype).float().numpy()
+    for (k, p, t) in [(50, 0.9, 0.8), (-1, 0.3, 1.0), (1024, 0.95, 1.5)]:
+        _run_case(torch, oracle, capi, lg, t, k, p, u_np=H.uniforms(B, 8192), dtype=dtype,
+                  what="middle slices %s k=%s p=%s T=%s" % (fmt, k, p, t))
+
+
 @pytest.mark.parametrize("fmt", ["bfloat16", "float16"])
 def test_half_precision_logits(torch_cuda, oracle, fmt):
     """Logits handed over as bfloat16 or float16 (rs_sample_dtype; an extension, the reference takes
