@@ -146,8 +146,8 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
 // slices of 8192 tokens while those do (256 CUs x 6 workgroups of either kernel = 1536), else into
 // slices of 16384.  Measured over forty shapes of 4-13M tokens: a pass that is one wave of workgroups
 // is 0.5-2.5 us per call faster with the shorter slices, and slower from the first workgroup beyond
-// that.  Longer rows always take slices of 16384 tokens (they would be cut into more slices than a
-// finishing workgroup handles quickly).
+// that.  Longer rows take slices of 16384 tokens (they would be cut into more slices than a
+// finishing workgroup handles quickly) unless the call is only a few of them.
 constexpr int kStreamNT = 256;
 constexpr uint32_t kStreamSmallParts = 1536;
 constexpr uint64_t kFusedSmall = 1ull << 22;
@@ -155,7 +155,15 @@ static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStre
 // `pen`: the pass that also reads penalties exists for the long slices only
 static int stream_r(int32_t B, int32_t V, bool pen = false)
 {
-    if (V > 262144) return kStreamLongR;
+    if (V > 262144) {
+        // a few long rows: shorter slices while a row has at most 128 of them and the call at most 512
+        // (measured at 524288 and 1048576 tokens: 1-3.7 us faster up to there, slower beyond)
+        for (int R = 4; R <= 8 && !pen; R *= 2) {
+            const uint32_t g = stream_parts(V, R);
+            if (g <= 128u && (uint64_t)B * g <= 512u) return R;
+        }
+        return kStreamLongR;
+    }
     if ((uint64_t)B * stream_parts(V, 4) <= kStreamSmallParts) return 4;
     if (!pen && (uint64_t)B * stream_parts(V, 8) <= kStreamSmallParts) return 8;
     return kStreamLongR;
@@ -299,7 +307,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 402; }
+int rs_version(void) { return 403; }
 
 const char *rs_error_string(int code)
 {

@@ -416,6 +416,19 @@ def test_streaming_path_middle_slices(torch_cuda, oracle, fmt):
                   what="middle slices %s k=%s p=%s T=%s" % (fmt, k, p, t))
 
 
+@pytest.mark.parametrize("B,V", [(2, 1048576), (2, 524288), (3, 528384), (1, 1000000)])
+def test_streaming_path_few_long_rows(torch_cuda, oracle, B, V):
+    """A few rows of more than 262144 tokens are cut into up to 128 slices of 4096 or 8192 tokens
+    (instead of 16384): rows of several kinds, a ragged last slice, a nucleus, a bounding top_k and
+    both, through every path."""
+    from tests import capi
+    rng = np.random.default_rng(V + B)
+    lg = np.stack([_random_row(rng, (2, 6, 4, 8)[b % 4], V) for b in range(B)])
+    for (k, p, t) in [(50, 0.9, 0.8), (-1, 0.3, 1.0), (1000, 1.0, 1.2)]:
+        _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=H.uniforms(B, 77),
+                  what="few long rows B=%d V=%d k=%s p=%s T=%s" % (B, V, k, p, t))
+
+
 @pytest.mark.parametrize("fmt", ["bfloat16", "float16"])
 def test_half_precision_logits(torch_cuda, oracle, fmt):
     """Logits handed over as bfloat16 or float16 (rs_sample_dtype; an extension, the reference takes
