@@ -307,7 +307,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 403; }
+int rs_version(void) { return 404; }
 
 const char *rs_error_string(int code)
 {

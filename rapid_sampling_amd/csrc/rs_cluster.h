@@ -627,12 +627,19 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
         sample_slice<R, PEN>(p, s, blockIdx.x, 0u);
         return;
     }
+    // A launch that the device holds all at once needs no tickets: every workgroup is resident whatever
+    // the order they start in, and a few hundred fetch-adds on one word, served one after the other,
+    // would hold the last workgroups back by microseconds.
+    constexpr uint32_t kResident = 256u * (uint32_t)min_waves<R, PEN>();
     if (threadIdx.x == 0) {
         s.abort = 0; s.host_words = p.host_words;
-        const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
-        // every workgroup of the launch takes exactly one ticket: after the last one the counter
-        // is not touched again, and is put back for the next call
-        if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);
+        uint32_t t = blockIdx.x;
+        if (gridDim.x > kResident) {
+            t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
+            // every workgroup of the launch takes exactly one ticket: after the last one the counter
+            // is not touched again, and is put back for the next call
+            if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);
+        }
         s.bc32[0] = t;
     }
     __syncthreads();
