@@ -604,18 +604,19 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
     return slice_finish(p, s, sl);
 }
 
-// Workgroups take their (row, slice) from a ticket counter, so that logical ids follow the order in
-// which workgroups actually start and a row's workgroups are the next ones to start.  The workgroups
-// of a row wait for EACH OTHER (every exchange is all-to-all within the row, so a low ticket waits for
-// higher ones too).  The waits end because a workgroup, once started, runs to its end without giving
-// up its compute unit; because the workgroups that have started are, at any time, all of the earlier
-// rows (which finish and leave) and the first part of one unfinished row; and because the rest of
-// that row can always start: the hardware binds workgroup b of a launch to XCD b mod 8 before it
-// starts, so towards the end of a launch the workgroups still to start may all belong to one XCD, and
-// a row must therefore have fewer workgroups than ONE XCD holds (32 compute units x at least 2
-// workgroups of this kernel: the host cuts rows into at most 64).  A device partitioned below that,
-// or shared with other long-running kernels, can starve a row -- the waits are bounded for that case
-// and end in RS_ERR_DEVICE rather than a hang.
+// The workgroups of a row wait for EACH OTHER (every exchange is all-to-all within the row).  A launch
+// that the device holds all at once (256 CUs x the workgroups per CU the launch bounds guarantee)
+// uses the hardware's workgroup ids: every workgroup becomes resident whatever else runs, so every
+// wait ends.  A larger launch hands out (row, slice) from a ticket counter, so that logical ids
+// follow the order in which workgroups actually start and a row's workgroups are the next ones to
+// start: then the workgroups that have started are, at any time, all of the earlier rows (which
+// finish and leave) and the first part of one unfinished row, and the rest of that row can always
+// start -- the hardware binds workgroup b of a launch to XCD b mod 8 before it starts, so towards the
+// end of a launch the workgroups still to start may all belong to one XCD, and a row must therefore
+// have fewer workgroups than ONE XCD holds (32 compute units x at least 2 workgroups of this kernel:
+// the host cuts rows into at most 64).  A device partitioned below 256 CUs, or shared with other
+// long-running kernels, can starve a row -- the waits are bounded for that case and end in
+// RS_ERR_DEVICE rather than a hang.
 template <int R, bool PEN>
 __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
 {

@@ -1132,8 +1132,8 @@ __global__ void __launch_bounds__(kThreads, 2) fused_kernel(const Params p, cons
     __shared__ FusedLds<R, PEN> u;
     const int tid = threadIdx.x;
     const uint32_t G = v.G;
-    // logical id: the hardware's while the whole launch fits the GPU at once, else a ticket, so that
-    // a row's workgroups are always the next ones to start
+    // logical id: the hardware's while the device holds the whole launch at once (every call routed here
+    // by itself does), else a ticket, so that a row's workgroups are always the next ones to start
     uint32_t id = blockIdx.x;
     constexpr uint32_t kResident = 256u * (R == 16 && PEN ? 2u : 3u);     // workgroups of this kernel the device holds at once
     if (gridDim.x > kResident) {
