@@ -316,7 +316,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 405; }
+int rs_version(void) { return 406; }
 
 const char *rs_error_string(int code)
 {

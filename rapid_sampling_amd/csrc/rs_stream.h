@@ -702,17 +702,20 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     // What the stashes cannot finish, this workgroup does alone from the logits.  Such rows are
     // counted, and the first of a call tells the caller's policy at once (that a call went well is
     // reported by the call after it, see report_begin).
+    auto tell_policy = [&]() {
+        if (tid == 0) {
+            const uint32_t c = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
+            if (c == 0u && p.host_words)                 // the call's first such row tells the caller's policy at once
+                __hip_atomic_store(p.host_words + p.report, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+    };
     auto slow = [&]() -> bool {
         if (drawer) {                                    // the row is finished here: this draw is used up
             rng_st[2] = rs[2] + 1u;
             if (rs[2] + 1u == 0u) rng_st[3] = rs[3] + 1u;
         }
         finish_row_slow(p, s, t, row, xmax, p.inj_u ? 0ull : t.rand64);
-        if (tid == 0) {
-            const uint32_t c = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
-            if (c == 0u && p.host_words)                 // the call's first such row tells the caller's policy at once
-                __hip_atomic_store(p.host_words + p.report, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        }
+        tell_policy();
         return true;
     };
 
@@ -783,6 +786,14 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         }
         subset = true;
     }
+
+    // A nucleus of thousands of tokens is finished here all the same, but one workgroup going through
+    // such a list a dozen times takes longer than the general kernel needs for the whole call (measured:
+    // 128 rows of 50304, about 4000 tokens each, 54 against 36 us; the two meet at about 2400 tokens
+    // there and, the general kernel's time growing with the row, at about 4700 for rows of 100256): a
+    // call that is only an attempt (no top_k bounds the kept set) says so to the caller's policy.
+    const uint32_t long_list = max(2048u, (uint32_t)p.V / 20u);
+    if (!FUSED && p.report == 1u && total > long_list) tell_policy();
 
     // gather the tokens, re-based to the row's frame: a thread takes a run of consecutive list
     // entries, so that it looks up its first slice once and walks on from there
