@@ -649,16 +649,19 @@ def test_c4_penalty_chain(torch_cuda, oracle, steps):
 
 
 
-def test_one_launch_path_rows_of_more_slices_than_an_xcd_has_compute_units(torch_cuda, oracle):
+@pytest.mark.parametrize("B", [11, 21])
+def test_one_launch_path_rows_of_more_slices_than_an_xcd_has_compute_units(torch_cuda, oracle, B):
     """The workgroups of the one-launch path wait for each other, and the hardware binds workgroup b to
     XCD b mod 8 before it starts.  With its token list in dynamic LDS the kernel ran one workgroup per
     compute unit, 32 per XCD, and a row of 47 slices whose last workgroups all belonged to one XCD could
     starve until its waits gave up (one call in some hundred, always the last row).  The list now always
-    lives in static LDS.  The shape and the sequence of calls that showed it, 300 times over, with a wait
-    limit of 50 ms so that a starved row would show at once."""
+    lives in static LDS.  The shape and the sequence of calls that showed it (11 rows: 517 workgroups,
+    which the device holds at once, so they keep the hardware's ids), and the same with 21 rows (987
+    workgroups: more than it holds, so they draw tickets), 300 times over, with a wait limit of 50 ms
+    so that a starved row would show at once."""
     torch = torch_cuda
     from tests import capi
-    B, V = 11, 191104
+    V = 191104
     rng = np.random.default_rng(5)
     rows = []
     for _ in range(B):
