@@ -316,7 +316,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 406; }
+int rs_version(void) { return 407; }
 
 const char *rs_error_string(int code)
 {

@@ -607,16 +607,14 @@ __device__ __forceinline__ bool sample_slice(const Params &p, Lds &s, const uint
 // The workgroups of a row wait for EACH OTHER (every exchange is all-to-all within the row).  A launch
 // that the device holds all at once (256 CUs x the workgroups per CU the launch bounds guarantee)
 // uses the hardware's workgroup ids: every workgroup becomes resident whatever else runs, so every
-// wait ends.  A larger launch hands out (row, slice) from a ticket counter, so that logical ids
-// follow the order in which workgroups actually start and a row's workgroups are the next ones to
-// start: then the workgroups that have started are, at any time, all of the earlier rows (which
-// finish and leave) and the first part of one unfinished row, and the rest of that row can always
-// start -- the hardware binds workgroup b of a launch to XCD b mod 8 before it starts, so towards the
-// end of a launch the workgroups still to start may all belong to one XCD, and a row must therefore
-// have fewer workgroups than ONE XCD holds (32 compute units x at least 2 workgroups of this kernel:
-// the host cuts rows into at most 64).  A device partitioned below 256 CUs, or shared with other
-// long-running kernels, can starve a row -- the waits are bounded for that case and end in
-// RS_ERR_DEVICE rather than a hang.
+// wait ends.  A larger launch hands out (row, slice) by tickets (take_ticket), so that logical ids
+// follow the order in which workgroups actually start: the hardware binds workgroup b of a launch to
+// XCD b mod 8 before it starts, each XCD draws from a counter of its own, and the ids it holds at any
+// time are the lowest of its residue not yet finished -- so the earliest unfinished row has, on every
+// XCD, its workgroups running or next to start, and finishes; then the next one.  A row puts an
+// eighth of its workgroups (at most 8 of 64) on each XCD, far fewer than an XCD holds.  A device
+// partitioned below 256 CUs, or shared with other long-running kernels, can starve a row -- the waits
+// are bounded for that case and end in RS_ERR_DEVICE rather than a hang.
 template <int R, bool PEN>
 __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel(const Params p)
 {
@@ -635,12 +633,7 @@ __global__ void __launch_bounds__(kThreads, (min_waves<R, PEN>())) sample_kernel
     if (threadIdx.x == 0) {
         s.abort = 0; s.host_words = p.host_words;
         uint32_t t = blockIdx.x;
-        if (gridDim.x > kResident) {
-            t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
-            // every workgroup of the launch takes exactly one ticket: after the last one the counter
-            // is not touched again, and is put back for the next call
-            if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);
-        }
+        if (gridDim.x > kResident) t = take_ticket(p.hdr);
         s.bc32[0] = t;
     }
     __syncthreads();

@@ -26,7 +26,7 @@ constexpr uint64_t kValid     = 1ull << 63;   // marks a written exchange word
 constexpr uint32_t kVerdictFallback = 0xFFFFFFFFu;   // the finishing workgroup could not finish the row from the stashes
 
 struct alignas(256) WsHeader {
-    uint32_t ticket;      // next logical workgroup id of the running launch
+    uint32_t unused0;
     uint32_t finished;    // workgroups that have left the running launch
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows of the running (or last) streaming call that the finishing workgroups did the slow way
@@ -34,7 +34,12 @@ struct alignas(256) WsHeader {
     uint32_t last_call;   // 1 | kind << 31 after a streaming call that no later call has reported on yet (kind: 0 top_k bounds the kept set, 1 not), else 0
     uint32_t gave_up[4];  // the first wait that gave up since the workspace was set up: site, row << 16 | slice, what it had, what it waited for
     uint32_t pad[54];
+    // Logical workgroup ids of a launch larger than the device holds at once: eight counters, one per
+    // workgroup id modulo 8, each on a cache line of its own (take_ticket).
+    uint32_t ticket[8][64];
 };
+static_assert(sizeof(WsHeader) == 2304, "tests that spoil a workspace leave its header alone: tests/capi.py HEADER_BYTES");
+
 
 // How long a workgroup waits for its peers before it gives up (wall-clock ticks).
 __device__ __forceinline__ uint64_t spin_limit(const WsHeader *hdr)
@@ -95,6 +100,28 @@ struct Params {
 // counter: completeness is visible in the data itself.
 template <typename T> __device__ __forceinline__ T a_load(const T *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, RS_AGENT); }
 template <typename T> __device__ __forceinline__ void a_store(T *p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, RS_AGENT); }
+
+// Logical id of this workgroup in a launch larger than the device holds at once: ids follow the order
+// in which workgroups start.  One counter for the whole launch would be a few thousand fetch-adds on
+// one word, served at about 12 ns each whatever else the memory system does (a launch of 1024
+// workgroups: 13 us until the last one has its id; of 4096: 48 us); eight counters on cache lines of
+// their own, chosen by the hardware's workgroup id modulo 8, are served side by side (3 and 8 us).
+// Class c hands out the ids congruent to c modulo 8, in the order its workgroups start, and there
+// are exactly as many workgroups in a class as ids of that residue below the launch size, so every
+// id is taken once.  The hardware binds workgroup b to XCD b mod 8, so an XCD's workgroups draw from
+// one counter and hold, at any time, the lowest ids of their class not yet finished: the earliest
+// unfinished row has all its workgroups running or next to start on every XCD.
+__device__ __forceinline__ uint32_t take_ticket(WsHeader *hdr)
+{
+    const uint32_t c = blockIdx.x & 7u;
+    const uint32_t mine = (gridDim.x - c + 7u) >> 3;     // workgroups of this class in the launch
+    const uint32_t n = __hip_atomic_fetch_add(&hdr->ticket[c][0], 1u, __ATOMIC_RELAXED, RS_AGENT);
+    // every workgroup takes exactly one: after the class's last the counter is not touched again,
+    // and is put back for the next call
+    if (n == mine - 1u) a_store(&hdr->ticket[c][0], 0u);
+    return n * 8u + c;
+}
+
 template <typename T> __device__ __forceinline__ void a_add(T *p, T v) { __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, RS_AGENT); }
 __device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

@@ -1149,9 +1149,7 @@ __global__ void __launch_bounds__(kThreads, 2) fused_kernel(const Params p, cons
     constexpr uint32_t kResident = 256u * (R == 16 && PEN ? 2u : 3u);     // workgroups of this kernel the device holds at once
     if (gridDim.x > kResident) {
         if (tid == 0) {
-            const uint32_t t = __hip_atomic_fetch_add(&p.hdr->ticket, 1u, __ATOMIC_RELAXED, RS_AGENT);
-            if (t == gridDim.x - 1) a_store(&p.hdr->ticket, 0u);     // the last ticket of the launch
-            u.a.u32[8] = t;
+            u.a.u32[8] = take_ticket(p.hdr);
         }
         __syncthreads();
         id = u.a.u32[8];

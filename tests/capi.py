@@ -85,6 +85,9 @@ def normalize(temperature, top_k, top_p, V, B=1, T=1):
     return rc, c.value, k.value, p.value
 
 
+HEADER_BYTES = 2304          # the workspace's launch header (sizeof(rs::WsHeader)); tests that spoil a workspace leave it alone
+
+
 def workspace_bytes(B, V):
     n = C.c_size_t()
     rc = lib().rs_workspace_bytes(B, V, C.byref(n))

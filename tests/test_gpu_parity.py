@@ -993,7 +993,7 @@ def test_bounded_wait_reports_error_and_recovers(torch_cuda, oracle):
     smp = capi.Sampler(B, V, with_policy=True, init=True)
     lg, u = torch.from_numpy(lg_np).cuda(), torch.from_numpy(u_np).cuda()
     smp.set_wait_limit(20)
-    smp.ws[256:] = 1
+    smp.ws[capi.HEADER_BYTES:] = 1
     torch.cuda.synchronize()
     assert smp.policy_error() == 0
     print("poisoned workspace, expecting a bounded wait to give up", flush=True)
@@ -1018,6 +1018,7 @@ def test_python_module_raises_after_a_failed_call_and_recovers(torch_cuda, oracl
     workspace up again, and the call after that is correct.  workspace_status() tells at once."""
     torch = torch_cuda
     import rapid_sampling_amd as sample
+    from tests import capi
     B, V = 2, 32768                                  # small enough to take the general kernel, several workgroups per row
     lg_np = H.logits_normal(B, V, 2.0, seed=82)
     c, k, p = oracle.normalize(1.0, -1, 0.9, V, B, 1)
@@ -1034,7 +1035,7 @@ def test_python_module_raises_after_a_failed_call_and_recovers(torch_cuda, oracl
         for check in ("next call", "status"):
             sample.set_wait_limit(20)
             ws = sample._sample.debug_workspace()
-            ws[256:] = 1
+            ws[capi.HEADER_BYTES:] = 1
             side.synchronize()
             print("poisoned module workspace:", check, flush=True)
             sample.batch_sampling_temperature_topk_topp(lg, st, 1.0, -1, 0.9, uniforms=u)      # gives up; no exception yet
