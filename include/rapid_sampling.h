@@ -137,7 +137,10 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * which takes several times as long as the general kernel needs for a whole
  * call of moderate size: with a bounding top_k (<= 1024) that takes unusual
  * rows (ties of thousands of tokens), without one (top_p < 1 alone) a flat
- * distribution.  Calls that are given a policy report "a row went the slow
+ * distribution (a call without a bounding top_k also counts a row as slow
+ * when it is finished from a list of more than V/20, at least 2048, tokens:
+ * the general kernel is faster for such calls).  Calls that are given a
+ * policy report "a row went the slow
  * way: yes/no" to a word of pinned host memory inside it (yes at once, no by
  * the next call on the workspace), and rs_sample_ex reads that word, without
  * waiting, before it routes the next call: while it is set, calls of that
