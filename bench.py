@@ -292,6 +292,16 @@ def main():
                                    "achieved": round(bytes_flat / (t_flat * 1e-6) / 1e9, 1),
                                    "rows_per_s": round(Bb * Tb / (t_flat * 1e-6), 1)},
         }
+        # the same rows with plain temperature sampling (top_k = V, top_p = 1: every live token kept)
+        def call_plain():
+            return sample.batch_sampling_temperature_topk_topp(big, st_b, 1.0, -1, 1.0)
+
+        t_plain = block_time_us(torch, call_plain, args.bandwidth_steps, 3)
+        result["roofline"]["plain_temperature"] = {
+            "us_per_call": round(t_plain, 2), "achieved": round(bytes_btv / (t_plain * 1e-6) / 1e9, 1),
+            "frac": round(bytes_btv / (t_plain * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "the same (128,4,1048576) call with top_k -1, top_p 1.0: rs::stream_kernel counts only (no stashes), "
+                    "rs::finish_kernel picks the slice from the slices' masses and reads that slice once more"}
         # extension: the same rows handed over as bfloat16 (half the algorithmic bytes); (128, 1M), T = 1
         half = big[:, Tb - 1, :].to(torch.bfloat16)
         st_h = sample.setup_rand(1, Bb)

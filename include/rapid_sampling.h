@@ -52,7 +52,10 @@ typedef struct rs_row_diag {
     uint32_t left_bits;   /* same as thr_bits                                 */
     uint32_t thr_bits;    /* bit pattern of the smallest kept e               */
     uint32_t rounds;      /* histogram levels summed over the cluster; 0 = row
-                             finished by the streaming path                   */
+                             finished by the streaming path, 8 = by its
+                             finishing workgroup alone from the logits, 9 = a
+                             call that keeps every token (top_k = V, top_p = 1)
+                             on the streaming path                            */
     uint32_t n_gt;        /* tokens with e >  threshold                       */
     uint32_t n_eq;        /* tokens with e == threshold                       */
     int32_t  index;       /* sampled token                                    */
@@ -204,7 +207,10 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  * top_k <= 1024 the one-launch streaming kernel while the call fits the GPU at
  * once), two for calls of at least 2^17 tokens without penalties whose kept
  * set is expected to be small (a wait-free pass over the logits and a per-row
- * finish; see rs_policy), or three for calls of at least 2^23 tokens with
+ * finish; see rs_policy; plain temperature sampling -- top_k = V, top_p = 1,
+ * every token kept -- takes these two launches as well: the pass only counts,
+ * and the finish reads one slice of the row again), or three for calls of at
+ * least 2^23 tokens with
  * penalties and top_k <= 1024 (the same two and a pass that rewrites the
  * penalties); results are identical either way.  No environment variable is
  * read.
@@ -245,7 +251,8 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
  * rs_sample_dtype with explicit options (NULL = all defaults, which makes it
  * rs_sample_dtype).  `path` forces the way through the library (tests,
  * benchmarks): RS_PATH_CLUSTER the general one-launch kernel, RS_PATH_STREAM
- * the streaming path when top_k <= 1024 (else the general kernel),
+ * the streaming path when top_k <= 1024 or the call keeps every token (else
+ * the general kernel),
  * RS_PATH_ATTEMPT the streaming path whatever top_k is (penalties take the
  * general kernel on these three), RS_PATH_FUSED the streaming pass and the
  * finish in one launch (any call whose rows span at least two slices, with or

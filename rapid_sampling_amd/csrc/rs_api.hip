@@ -237,8 +237,15 @@ namespace rs {
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
-enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3 };
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4 };
 constexpr uint64_t kPenStreamMin = 1ull << 23;
+// Plain temperature sampling (top_k = V, top_p = 1: every live token is kept) has no kept set to
+// stash, but the streaming pass's bins alone say which slice holds the target: one pass at
+// bandwidth that only counts, plus a second look at one slice per row, beats the general kernel's
+// three exchanges for rows of 32768 tokens and more at every size measured from 131072 tokens per
+// call on (13.5 against 16.0 us for one row of 262144, 113 against 280 us for 128 rows of 1048576,
+// 70 against 84 us for 1024 rows of 32768); many short rows (2048 of 4096: 74 against 51 us) are
+// better off with the general kernel, which does such a row in one workgroup without exchanges.
 
 // Slice length of the one-launch path (float4 groups per thread), 0 when the call does not suit it.
 // Its workgroups hold their compute units until their row is finished, so a call pays twice once it
@@ -293,10 +300,13 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     }
     if (pen) return kPathCluster;
     if (force == RS_PATH_CLUSTER) return kPathCluster;
+    const bool keep_all = top_k == V && !(top_p < 1.0f);
+    if (keep_all && (force == RS_PATH_STREAM || force == RS_PATH_ATTEMPT)) return kPathKeep;
     if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
     if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
     if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
-    if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // everything is kept: nothing a stash could hold
+    if (keep_all && V >= 32768) return kPathKeep;              // shorter rows: one workgroup of the general kernel does a row in one go
+    if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // a top_k of thousands and no nucleus: more than the stashes hold
     if (!pol) return bounded ? kPathStream : kPathCluster;
     return routed_away(bounded ? 0 : 1) ? kPathCluster : bounded ? kPathStream : kPathAttempt;
 }
@@ -316,7 +326,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 407; }
+int rs_version(void) { return 408; }
 
 const char *rs_error_string(int code)
 {
@@ -505,7 +515,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.top_k = top_k; p.top_p = top_p;
     p.stash_k = (uint32_t)top_k; p.report = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
-    p.defer_pen = 0;
+    p.defer_pen = 0; p.keep_all = 0u;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path != kPathCluster) {
@@ -538,6 +548,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         // more slices could, rarely, starve until their waits gave up.
         if (path == kPathFused) v.list_cap = 2048u;
         p.report = path == kPathAttempt ? 1u : 0u;
+        if (path == kPathKeep) { p.keep_all = 1u; p.stash_k = 1u; v.list_cap = 2048u; }
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (path == kPathFused)
             return launch_fused(sr, pen, (uint32_t)B, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;

@@ -139,6 +139,30 @@ __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const
         uint64_t *rowbins = FUSED ? (p.ctl_end - 1 - row)->h[0] : (p.ctl_end - 1 - row)->rowhist;
         if (w) a_add(&rowbins[((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u], w);
     }
+    if (!FUSED && p.keep_all) {
+        // every live token is kept: the bins and their mass (in this slice's frame, left where the
+        // stash would begin) are all the finishing workgroup needs of this slice
+        if (wave == 0) {
+            u128 ms = 0;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                const int b = kSB - 1 - 3 * lane - i;
+                const uint64_t w = b >= 0 ? bin_total(b) : 0ull;
+                if (w) ms += pack_mass(w, (kBin0 + (uint32_t)b) >> 2);
+            }
+            const u128 tot = wave_inclusive_scan(ms);
+            if (lane == kWave - 1) {
+                uint64_t *st = v.stash + ((size_t)row * G + part) * kStashCap;
+                st[0] = (uint64_t)tot; st[1] = (uint64_t)(tot >> 64);
+            }
+        }
+        if (tid == 0) {
+            PartHdr ph;
+            ph.mkey = k; ph.cov = 0u; ph.n = 0u; ph.cut = 0u;
+            v.hdr[(size_t)row * G + part] = ph;
+        }
+        return k;
+    }
 
     // What to stash: the bins from the top down to the first one at which the count reaches
     // stash_k (that bin too if it fits).  With stash_k = top_k the row's top_k tokens are certainly
@@ -339,7 +363,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : RS_STREAM_WAVES)) stream_ker
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    if (reporter) report_end(p, prev, true);
+    if (reporter) report_end(p, prev, p.keep_all == 0u);     // a call that keeps everything has no rows to report on
     slice_count_and_stash<R, NT, kRep, false>(p, v, s, eb, lmax, row, part, base4, nv);
 }
 
@@ -400,7 +424,14 @@ __device__ __forceinline__ uint32_t bucket_step(Lds &s, LdsB &t, uint32_t nlist,
 // by token.  A few passes of one workgroup over one row take tens of microseconds (a row of a
 // million tokens: more than a hundred): fine for the odd row, and calls whose rows mostly end here
 // are routed to the cluster kernel by the caller's policy.  Same integers as every other path.
-__device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float xmax, const uint64_t rand64)
+//
+// KEEP_DIAG: the call keeps every live token (top_k = V, top_p = 1) and its token is picked from the
+// slices' masses (keep_pick); what is left to do here is the diagnostics record, which names the
+// threshold -- the smallest live token of the row -- and how many tokens tie there: one pass over
+// the row, paid by callers that ask for the record (tests, mostly).  keep_live: live tokens of the row.
+template <bool KEEP_DIAG = false>
+__device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float xmax, const uint64_t rand64,
+                                                const uint32_t keep_live = 0u)
 {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t V4 = (uint32_t)p.V >> 2;
@@ -439,6 +470,35 @@ __device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t
         }
     };
     const uint64_t top_k = (uint64_t)p.top_k;
+    if constexpr (KEEP_DIAG) {
+        uint32_t mn = 0xFFFFFFFFu, cnt = 0u;
+        row_pass(0u, V4, [&](uint32_t, uint32_t b) {
+            if (b >= kEMinBits) {
+                if (b < mn) { mn = b; cnt = 1u; }
+                else if (b == mn) ++cnt;
+            }
+        });
+        const uint32_t wm = ~wave_max_u32(~mn);
+        __syncthreads();
+        if (lane == 0) s.u32[wave] = wm;
+        __syncthreads();
+        uint32_t bm = s.u32[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) bm = min(bm, s.u32[w]);
+        const uint32_t ci = wave_inclusive_scan(mn == bm ? cnt : 0u);
+        __syncthreads();
+        if (lane == kWave - 1) s.u32[wave] = ci;
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t n_eq = 0;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) n_eq += s.u32[w];
+            const u128 D = s.D;
+            tie_and_target(p, row, rand64, xmax, D, s.P, bm, keep_live - n_eq, n_eq, D - (u128)n_eq * w_of_bits(bm), 9u, true);
+        }
+        __syncthreads();
+        return;
+    }
 
     // level 1 (dead tokens, below 2^-40, are left out)
     __syncthreads();
@@ -577,6 +637,58 @@ __device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t
                 if (acc >= r) { pick = idx; found = true; }
             };
             step(i4 * 4u, b.x); step(i4 * 4u + 1u, b.y); step(i4 * 4u + 2u, b.z); step(i4 * 4u + 3u, b.w);
+        }
+        p.out[row] = (int32_t)pick;
+        if (p.diag) p.diag[row].index = (int32_t)pick;
+        t.result = pick + 1u;
+    }
+}
+
+// The token of a row of a call that keeps everything: the slice that begins at token lo_idx holds
+// the target, r is the target's offset inside the slice.  Thread t owns the slice's float4 groups
+// [t N, (t + 1) N) -- consecutive tokens, so the running sum over the threads is the running sum
+// over the tokens -- and sums their weights; a scan finds the one thread whose tokens hold the
+// target, and that thread walks its own tokens, which it still has in its registers.  One look at
+// the slice, no atomics.  (No penalties on this path.)
+template <int SLICE_LOG2>
+__device__ __forceinline__ void keep_pick(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float M, const uint32_t lo_idx, const u128 r)
+{
+    constexpr int N = 1 << (SLICE_LOG2 - 10);
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const uint32_t V4 = (uint32_t)p.V >> 2;
+    const char *lrow = logits_row(p, row);
+    const uint32_t g0 = (lo_idx >> 2) + (uint32_t)tid * N;
+    auto weight = [](uint32_t b) -> uint64_t { return b >= kEMinBits ? w_of_bits(b) : 0ull; };
+    float4 l[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) l[j] = load_logits4(lrow, min(g0 + (uint32_t)j, V4 - 1u), p.dtype);
+    uint4 b[N];
+    u128 mine = 0;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        if (g0 + (uint32_t)j < V4) {
+            b[j] = make_uint4(e_bits_of(sf(l[j].x * p.c), M), e_bits_of(sf(l[j].y * p.c), M), e_bits_of(sf(l[j].z * p.c), M), e_bits_of(sf(l[j].w * p.c), M));
+            mine += (u128)weight(b[j].x) + weight(b[j].y) + weight(b[j].z) + weight(b[j].w);
+        } else b[j] = make_uint4(0u, 0u, 0u, 0u);                    // past the end of the row: no weight
+    }
+    u128 inc = wave_inclusive_scan(mine);
+    __syncthreads();
+    if (lane == kWave - 1) s.q128[wave] = inc;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) inc += s.q128[w];
+    u128 acc = inc - mine;
+    if (acc < r && r <= inc) {
+        uint32_t pick = g0 * 4u;
+        bool found = false;
+        auto step = [&](uint32_t idx, uint32_t bits) {
+            if (found) return;
+            acc += weight(bits);
+            if (acc >= r) { pick = idx; found = true; }
+        };
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const uint32_t i = (g0 + (uint32_t)j) * 4u;
+            step(i, b[j].x); step(i + 1u, b[j].y); step(i + 2u, b[j].z); step(i + 3u, b[j].w);
         }
         p.out[row] = (int32_t)pick;
         if (p.diag) p.diag[row].index = (int32_t)pick;
@@ -740,6 +852,46 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
             if (p.diag) p.diag[row].index = (int32_t)lo_i;
             t.result = lo_i + 1u;
         }
+        return true;
+    }
+
+    if (!FUSED && p.keep_all) {
+        // Every live token is kept with its full weight (S = D).  Each slice's mass, moved into the
+        // row's frame, is exact (a bin is dead in the row's frame as a whole or not at all: frames
+        // differ by whole octaves); a scan over the slices finds the one that holds the target, and
+        // only that slice's logits are looked at again.
+        if (drawer) {
+            rng_st[2] = rs[2] + 1u;
+            if (rs[2] + 1u == 0u) rng_st[3] = rs[3] + 1u;
+        }
+        u128 mine = 0;
+        if ((uint32_t)tid < G && dl < 41u) {                          // 41 octaves and more below: nothing of the slice is live
+            const uint64_t *sm = v.stash + ((size_t)row * G + tid) * kStashCap;
+            mine = (u128)sm[0] | ((u128)sm[1] << 64);
+            if (dl) {
+                // the slice's lowest 4 dl bins are dead in the row's frame; the rest is a multiple of 2^dl
+                const uint64_t *sh = v.shist + ((size_t)row * G + tid) * kSB;
+                u128 low = 0;
+                for (uint32_t b = 0; b < 4u * dl; ++b) {
+                    const uint64_t w = sh[b];
+                    if (w) low += pack_mass(w, (kBin0 + b) >> 2);
+                }
+                mine = (mine - low) >> dl;
+            }
+        }
+        const u128 r = p.inj_u ? ceil_mul(p.inj_u[row], D) : r_from_bits(t.rand64, D);
+        u128 inc = wave_inclusive_scan(mine);
+        if (lane == kWave - 1) s.q128[wave] = inc;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) inc += s.q128[w];
+        const u128 exc = inc - mine;
+        if (exc < r && r <= inc) { t.bucket = (uint32_t)tid; s.bc128[1] = r - exc; }
+        __syncthreads();
+        const uint32_t g = t.bucket;
+        const u128 r_in = s.bc128[1];
+        __syncthreads();
+        if (p.diag) finish_row_slow<true>(p, s, t, row, xmax, p.inj_u ? 0ull : t.rand64, f.cnt_above + f.cnt_bin);
+        keep_pick<SLICE_LOG2>(p, s, t, row, M, g << SLICE_LOG2, r_in);
         return true;
     }
 

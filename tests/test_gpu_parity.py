@@ -429,6 +429,41 @@ def test_streaming_path_few_long_rows(torch_cuda, oracle, B, V):
                   what="few long rows B=%d V=%d k=%s p=%s T=%s" % (B, V, k, p, t))
 
 
+@pytest.mark.parametrize("B,V", [(11, 50304), (4, 262144), (40, 152064), (2, 1048576), (3, 528384), (1, 4096)])
+def test_streaming_path_keeps_everything(torch_cuda, oracle, B, V):
+    """Plain temperature sampling (top_k = V, top_p = 1): every live token is kept, so there is no
+    kept set to stash.  The streaming pass only counts; the finishing workgroup takes each slice's mass
+    from the slice's bins (moved into the row's frame), finds the slice that holds the target and looks
+    at that slice's logits once more.  Rows of every kind (ties, masks, slices whose maxima lie
+    hundreds of octaves apart, most of the row dead, NaN and Inf), ragged last slices, every slice
+    length, several temperatures; _run_case forces the path (twice) next to the general kernel and
+    compares the token, every diagnostic (the threshold is the smallest live token, its ties counted)
+    and the e of every token.  Then the same calls the way a caller makes them (no diagnostics, random
+    numbers from the Philox state): the tokens and the advanced states must equal the general kernel's."""
+    from tests import capi
+    torch = torch_cuda
+    rng = np.random.default_rng(V * 31 + B)
+    lg = np.stack([_random_row(rng, (2, 9, 6, 4, 0, 8, 10, 1, 7, 5, 3)[b % 11], V) for b in range(B)])
+    for t in (1.0, 0.7, 3.0):
+        _run_case(torch, oracle, capi, lg, t, -1, 1.0, u_np=H.uniforms(B, int(t * 10) + V % 97),
+                  what="keep all B=%d V=%d T=%s" % (B, V, t))
+    rc, c, k, p = capi.normalize(1.0, -1, 1.0, V, B, 1)
+    assert rc == 0 and k == V
+    lgd = torch.from_numpy(lg).cuda()
+    smp = capi.Sampler(B, V)
+    rounds = smp.sample(lgd, c, k, p, uniforms=torch.from_numpy(H.uniforms(B, 3)).cuda(), path="stream")["diag"]["rounds"]
+    assert ((rounds == 9) | (rounds == 0)).all() and (rounds == 9).any(), rounds    # 0: a row of equal logits, by division
+    rng_ref = oracle.rng_init(1234 + V, B)
+    ref = np.stack([oracle.sample_batch(lg, c, k, p, rng=rng_ref)[0] for _ in range(3)])
+    for path in ("cluster", "stream", None):
+        st = torch.empty(B * 64, dtype=torch.int8, device="cuda")
+        assert capi.lib().rs_philox_init(st.data_ptr(), 1234 + V, B, smp.stream()) == 0
+        res = [smp.sample(lgd, c, k, p, rng=st, want_diag=False, path=path)["out"] for _ in range(3)]
+        assert smp.status() == 0
+        assert np.array_equal(np.stack(res), ref), path
+        assert np.array_equal(st.cpu().numpy().view(np.uint32).reshape(B, 16), rng_ref), path
+
+
 @pytest.mark.parametrize("fmt", ["bfloat16", "float16"])
 def test_half_precision_logits(torch_cuda, oracle, fmt):
     """Logits handed over as bfloat16 or float16 (rs_sample_dtype; an extension, the reference takes
