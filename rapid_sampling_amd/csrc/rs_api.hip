@@ -515,7 +515,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.top_k = top_k; p.top_p = top_p;
     p.stash_k = (uint32_t)top_k; p.report = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
-    p.defer_pen = 0; p.keep_all = 0u;
+    p.defer_pen = 0;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path != kPathCluster) {
@@ -548,7 +548,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         // more slices could, rarely, starve until their waits gave up.
         if (path == kPathFused) v.list_cap = 2048u;
         p.report = path == kPathAttempt ? 1u : 0u;
-        if (path == kPathKeep) { p.keep_all = 1u; p.stash_k = 1u; v.list_cap = 2048u; }
+        if (path == kPathKeep) { p.stash_k = 1u; v.list_cap = 2048u; }
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (path == kPathFused)
             return launch_fused(sr, pen, (uint32_t)B, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
@@ -559,7 +559,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
             if (launch_stream_pen((uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
             return launch_penalty_pass(st, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         }
-        return launch_stream(sr, logits_dtype, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+        return launch_stream(sr, logits_dtype, path == kPathKeep, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
     }
     return launch_sample(pen, g.R, grid, (hipStream_t)stream, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
 }

@@ -85,8 +85,6 @@ struct Params {
     uint32_t     report;       // which of the two report words a streaming call writes: 0 top_k bounds the kept set, 1 not
     int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1] routing reports, [2] error; or null
     int32_t      defer_pen;    // penalties enter x but are left as they are: a later pass over them applies decay and one-hot add
-    uint32_t     keep_all;     // streaming call that keeps every live token (top_k = V, top_p = 1): no stashes, the token is
-                               // picked from the slices' masses and one more look at a single slice
     int64_t      row_stride;
     int32_t      B, V;
     uint32_t     G;            // workgroups per row
@@ -666,7 +664,7 @@ struct StreamView {
 hipError_t launch_sample(bool pen, int R, dim3 grid, hipStream_t st, const Params &p);
 hipError_t launch_stream_pen(uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
 hipError_t launch_penalty_pass(hipStream_t st, const Params &p);
-hipError_t launch_stream(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
+hipError_t launch_stream(int slice_r, int32_t dtype, bool keep, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
                          const StreamView &v);
 hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v);
 

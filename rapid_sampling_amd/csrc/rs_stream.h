@@ -70,7 +70,7 @@ template <bool FUSED, typename T> __device__ __forceinline__ T get(const T *p)
 // in eb), the packed histogram added to the row's and kept under the slice's own name, cumulative
 // counts, and the stash of its largest tokens with the value down to which it is complete.
 // Returns the key of the slice's maximum.
-template <int R, int NT, int kRep, bool FUSED>
+template <int R, int NT, int kRep, bool FUSED, bool KEEP = false>     // KEEP: a call that keeps every live token (top_k = V, top_p = 1)
 __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const StreamView &v, LdsA<kRep> &s, uint32_t (&eb)[R * 4],
                                                           const float lmax, const uint32_t row, const uint32_t part,
                                                           const uint32_t base4, const int nv)
@@ -139,7 +139,7 @@ __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const
         uint64_t *rowbins = FUSED ? (p.ctl_end - 1 - row)->h[0] : (p.ctl_end - 1 - row)->rowhist;
         if (w) a_add(&rowbins[((uint32_t)(int)mm * 4u + (uint32_t)tid - 160u) & 511u], w);
     }
-    if (!FUSED && p.keep_all) {
+    if constexpr (KEEP) {
         // every live token is kept: the bins and their mass (in this slice's frame, left where the
         // stash would begin) are all the finishing workgroup needs of this slice
         if (wave == 0) {
@@ -301,7 +301,7 @@ __device__ __forceinline__ uint32_t slice_count_and_stash(const Params &p, const
     return k;
 }
 
-template <int R, int NT, int DT>     // NT threads, each with R groups of four tokens of the slice; DT the logits' type
+template <int R, int NT, int DT, bool KEEP = false>     // NT threads, each with R groups of four tokens of the slice; DT the logits' type
 __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : RS_STREAM_WAVES)) stream_kernel(const Params p, const StreamView v)
 {
     constexpr int kRep = stream_copies<R>();
@@ -363,8 +363,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : RS_STREAM_WAVES)) stream_ker
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    if (reporter) report_end(p, prev, p.keep_all == 0u);     // a call that keeps everything has no rows to report on
-    slice_count_and_stash<R, NT, kRep, false>(p, v, s, eb, lmax, row, part, base4, nv);
+    if (reporter) report_end(p, prev, !KEEP);                // a call that keeps everything has no rows to report on
+    slice_count_and_stash<R, NT, kRep, false, KEEP>(p, v, s, eb, lmax, row, part, base4, nv);
 }
 
 struct LdsB {
@@ -702,7 +702,7 @@ __device__ __forceinline__ void keep_pick(const Params &p, Lds &s, LdsB &t, cons
 // launch and is read with device-scope atomic loads), where the caller then tells the row's other
 // workgroups and the row's histogram is left in place for them.  With FUSED = false such a row is
 // done here the slow way, from the logits.
-template <int SLICE_LOG2, bool FUSED>     // SLICE_LOG2: log2 of the tokens per slice of the view
+template <int SLICE_LOG2, bool FUSED, bool KEEP = false>     // SLICE_LOG2: log2 of the tokens per slice of the view
 __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v, Lds &s, LdsB &t, const uint32_t row)
 {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
@@ -855,7 +855,7 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         return true;
     }
 
-    if (!FUSED && p.keep_all) {
+    if constexpr (KEEP) {
         // Every live token is kept with its full weight (S = D).  Each slice's mass, moved into the
         // row's frame, is exact (a bin is dead in the row's frame as a whole or not at all: frames
         // differ by whole octaves); a scan over the slices finds the one that holds the target, and
@@ -1125,14 +1125,14 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     return true;
 }
 
-template <int SLICE_LOG2>
+template <int SLICE_LOG2, bool KEEP = false>
 __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const StreamView v)
 {
     __shared__ Lds s;
     __shared__ LdsB t;
     extern __shared__ __align__(16) unsigned char finish_dyn[];
-    t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value
-    finish_row<SLICE_LOG2, false>(p, v, s, t, blockIdx.x);
+    t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value (KEEP: no list, not used)
+    finish_row<SLICE_LOG2, false, KEEP>(p, v, s, t, blockIdx.x);
 }
 
 
