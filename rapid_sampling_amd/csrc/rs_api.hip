@@ -243,7 +243,7 @@ constexpr uint64_t kPenStreamMin = 1ull << 23;
 // stash, but the streaming pass's bins alone say which slice holds the target: one pass at
 // bandwidth that only counts, plus a second look at one slice per row, beats the general kernel's
 // three exchanges for rows of 32768 tokens and more at every size measured from 131072 tokens per
-// call on (13.5 against 16.0 us for one row of 262144, 113 against 280 us for 128 rows of 1048576,
+// call on (13.5 against 16.0 us for one row of 262144, 107 against 280 us for 128 rows of 1048576,
 // 70 against 84 us for 1024 rows of 32768); many short rows (2048 of 4096: 74 against 51 us) are
 // better off with the general kernel, which does such a row in one workgroup without exchanges.
 
@@ -326,7 +326,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 408; }
+int rs_version(void) { return 409; }
 
 const char *rs_error_string(int code)
 {

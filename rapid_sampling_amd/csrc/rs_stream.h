@@ -645,54 +645,71 @@ __device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t
 }
 
 // The token of a row of a call that keeps everything: the slice that begins at token lo_idx holds
-// the target, r is the target's offset inside the slice.  Thread t owns the slice's float4 groups
-// [t N, (t + 1) N) -- consecutive tokens, so the running sum over the threads is the running sum
-// over the tokens -- and sums their weights; a scan finds the one thread whose tokens hold the
-// target, and that thread walks its own tokens, which it still has in its registers.  One look at
-// the slice, no atomics.  (No penalties on this path.)
+// the target, r is the target's offset inside the slice.  The slice is gone through in chunks of
+// 64 float4 groups (256 consecutive tokens, one KB that a wave loads in one go): chunk c belongs
+// to wave c mod 4, which sums its tokens' weights (two 64-bit wave sums of the weights' halves);
+// one wave scans the chunk totals for the chunk that holds the target, loads that chunk again,
+// scans its 64 groups, and the lane whose group holds the target walks its four tokens.  No
+// atomics, no list.  (An earlier version gave every thread 16 consecutive groups: its loads, 64
+// cache lines per instruction and every line touched by 8 instructions, cost a microsecond per
+// group.)  No penalties on this path.
 template <int SLICE_LOG2>
 __device__ __forceinline__ void keep_pick(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float M, const uint32_t lo_idx, const u128 r)
 {
-    constexpr int N = 1 << (SLICE_LOG2 - 10);
+    constexpr int N = 1 << (SLICE_LOG2 - 10);                      // chunks per wave
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const char *lrow = logits_row(p, row);
-    const uint32_t g0 = (lo_idx >> 2) + (uint32_t)tid * N;
-    auto weight = [](uint32_t b) -> uint64_t { return b >= kEMinBits ? w_of_bits(b) : 0ull; };
+    const uint32_t g0 = lo_idx >> 2;
+    auto weight = [&](float l) -> uint64_t {
+        const uint32_t b = e_bits_of(sf(l * p.c), M);
+        return b >= kEMinBits ? w_of_bits(b) : 0ull;
+    };
     float4 l[N];
 #pragma unroll
-    for (int j = 0; j < N; ++j) l[j] = load_logits4(lrow, min(g0 + (uint32_t)j, V4 - 1u), p.dtype);
-    uint4 b[N];
-    u128 mine = 0;
+    for (int j = 0; j < N; ++j) l[j] = load_logits4(lrow, min(g0 + (uint32_t)((j * kWaves + wave) * kWave + lane), V4 - 1u), p.dtype);
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-        if (g0 + (uint32_t)j < V4) {
-            b[j] = make_uint4(e_bits_of(sf(l[j].x * p.c), M), e_bits_of(sf(l[j].y * p.c), M), e_bits_of(sf(l[j].z * p.c), M), e_bits_of(sf(l[j].w * p.c), M));
-            mine += (u128)weight(b[j].x) + weight(b[j].y) + weight(b[j].z) + weight(b[j].w);
-        } else b[j] = make_uint4(0u, 0u, 0u, 0u);                    // past the end of the row: no weight
-    }
-    u128 inc = wave_inclusive_scan(mine);
-    __syncthreads();
-    if (lane == kWave - 1) s.q128[wave] = inc;
-    __syncthreads();
-    for (int w = 0; w < wave; ++w) inc += s.q128[w];
-    u128 acc = inc - mine;
-    if (acc < r && r <= inc) {
-        uint32_t pick = g0 * 4u;
-        bool found = false;
-        auto step = [&](uint32_t idx, uint32_t bits) {
-            if (found) return;
-            acc += weight(bits);
-            if (acc >= r) { pick = idx; found = true; }
-        };
-#pragma unroll
-        for (int j = 0; j < N; ++j) {
-            const uint32_t i = (g0 + (uint32_t)j) * 4u;
-            step(i, b[j].x); step(i + 1u, b[j].y); step(i + 2u, b[j].z); step(i + 3u, b[j].w);
+        uint64_t a = 0, b = 0;
+        if (g0 + (uint32_t)((j * kWaves + wave) * kWave + lane) < V4) {            // past the end of the row: no weight
+            const uint64_t w0 = weight(l[j].x), w1 = weight(l[j].y), w2 = weight(l[j].z), w3 = weight(l[j].w);
+            a = (w0 & 0xFFFFFFFFull) + (w1 & 0xFFFFFFFFull) + (w2 & 0xFFFFFFFFull) + (w3 & 0xFFFFFFFFull);
+            b = (w0 >> 32) + (w1 >> 32) + (w2 >> 32) + (w3 >> 32);
         }
-        p.out[row] = (int32_t)pick;
-        if (p.diag) p.diag[row].index = (int32_t)pick;
-        t.result = pick + 1u;
+        a = wave_sum(a); b = wave_sum(b);
+        if (lane == 0) { t.blo[j * kWaves + wave] = a; t.bhi[j * kWaves + wave] = b; }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const u128 mine = lane < N * kWaves ? (u128)t.blo[lane] + ((u128)t.bhi[lane] << 32) : (u128)0;
+        const u128 inc = wave_inclusive_scan(mine);
+        const u128 exc = inc - mine;
+        if (exc < r && r <= inc) { t.bucket = (uint32_t)lane; s.bc128[1] = r - exc; }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const uint32_t g = g0 + t.bucket * (uint32_t)kWave + (uint32_t)lane;
+        const u128 r2 = s.bc128[1];
+        uint64_t w[4] = {0ull, 0ull, 0ull, 0ull};
+        if (g < V4) {
+            const float4 q = load_logits4(lrow, g, p.dtype);
+            w[0] = weight(q.x); w[1] = weight(q.y); w[2] = weight(q.z); w[3] = weight(q.w);
+        }
+        const u128 mine = (u128)w[0] + w[1] + w[2] + w[3];
+        const u128 inc = wave_inclusive_scan(mine);
+        u128 acc = inc - mine;
+        if (acc < r2 && r2 <= inc) {
+            uint32_t pick = g * 4u + 3u;
+            bool found = false;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                acc += w[q];
+                if (!found && acc >= r2) { pick = g * 4u + (uint32_t)q; found = true; }
+            }
+            p.out[row] = (int32_t)pick;
+            if (p.diag) p.diag[row].index = (int32_t)pick;
+            t.result = pick + 1u;
+        }
     }
 }
 
