@@ -25,6 +25,9 @@ namespace rs {
 //                   that cannot be finished from the stashes (a huge tie, a
 //                   nucleus of thousands of tokens) it does alone, from the
 //                   logits (finish_row_slow).
+// A call that keeps every live token (top_k = V, top_p = 1) runs both kernels as a variant (KEEP):
+// the pass stops behind the histogram and leaves each slice's mass, the finishing workgroup picks
+// the slice from the masses and reads that one slice again (keep_pick).
 // Lanes of a wave that add to one LDS address are served one after the other, and rows often put
 // most of their tokens into a few bins.  So each bin is kept in kRep copies (lane l adds to copy
 // l % kRep), and e is not clamped before it is counted: the histogram spans all 512 values of
