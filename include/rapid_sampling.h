@@ -142,8 +142,11 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * rows (ties of thousands of tokens), without one (top_p < 1 alone) a flat
  * distribution (a call without a bounding top_k also counts a row as slow
  * when it is finished from a list of more than V/20, at least 2048, tokens:
- * the general kernel is faster for such calls).  Calls that are given a
- * policy report "a row went the slow
+ * the general kernel is faster for such calls; a call of fewer than 2^24
+ * tokens with a bounding top_k counts a row as slow when its stashes hold
+ * more tokens than the finishing workgroup's list and have to be gone through
+ * twice more -- flat rows cut into many slices -- for the same reason).  Calls
+ * that are given a policy report "a row went the slow
  * way: yes/no" to a word of pinned host memory inside it (yes at once, no by
  * the next call on the workspace), and rs_sample_ex reads that word, without
  * waiting, before it routes the next call: while it is set, calls of that

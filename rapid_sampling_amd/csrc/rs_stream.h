@@ -936,44 +936,15 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         t.take[tid] = inc;
         __syncthreads();
     };
-    take_prefix(mtake);
-    bool subset = false;                                               // plan B in force
-    uint32_t cutrow = 0;
-    if (t.fail || t.take[kThreads - 1] != total) {
-        // Plan B (flat distributions: the boundary bin holds thousands of tokens, but top_k is small):
-        // take the stashes whole.  Together they hold every token of the row at or above
-        // cutrow = the largest of the slices' cuts, so a threshold found among those is the row's.
-        uint32_t mycut = 0;
-        if ((uint32_t)tid < G) {
-            // a cut that lands below 2^-40 in the row's frame: what the stash lacks is dead there
-            mycut = max(rebase_bits(ph.cut, dl), kEMinBits);
-        }
-        cutrow = block_max_u32(s, mycut, lane, wave);
-        take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
-        total = t.take[kThreads - 1];
-        if (total > v.list_cap || total == 0u) {
-            // not resolvable from the stashes
-            if (FUSED) return false;
-            return slow();
-        }
-        subset = true;
-    }
-
-    // A nucleus of thousands of tokens is finished here all the same, but one workgroup going through
-    // such a list a dozen times takes longer than the general kernel needs for the whole call (measured:
-    // 128 rows of 50304, about 4000 tokens each, 54 against 36 us; the two meet at about 2400 tokens
-    // there and, the general kernel's time growing with the row, at about 4700 for rows of 100256): a
-    // call that is only an attempt (no top_k bounds the kept set) says so to the caller's policy.
-    const uint32_t long_list = max(2048u, (uint32_t)p.V / 20u);
-    if (!FUSED && p.report == 1u && total > long_list) tell_policy();
-
-    // gather the tokens, re-based to the row's frame: a thread takes a run of consecutive list
-    // entries, so that it looks up its first slice once and walks on from there
-    {
+    // fn(i, e in the row's frame, token) for the first n entries of the stashes' prefixes as t.take has
+    // them (entry i belongs to the first slice whose inclusive prefix exceeds i): a thread takes a run of
+    // consecutive entries, so that it looks up its first slice once and walks on from there, eight
+    // loads in flight
+    auto stashed = [&](const uint32_t n_all, auto fn) {
         constexpr int kBatch = 8;
-        const uint32_t per = (total + kThreads - 1u) / kThreads;
+        const uint32_t per = (n_all + kThreads - 1u) / kThreads;
         uint32_t i = (uint32_t)tid * per;
-        const uint32_t iend = min(total, i + per);
+        const uint32_t iend = min(n_all, i + per);
         uint32_t g = 0, gbase = 0, gend = 0;
         if (i < iend) {
             uint32_t lo_g = 0, hi_g = G - 1;                           // first slice whose prefix exceeds i
@@ -986,9 +957,7 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         if (per == 1u) {                                               // a short list: one entry, no walking
             if (i < iend) {
                 const uint64_t e = get<FUSED>(&v.stash[((size_t)row * G + g) * kStashCap + (i - gbase)]);
-                uint32_t b = rebase_bits((uint32_t)(e >> 32), t.delta[g]);
-                if (b < cutrow) b = 0;
-                t.list[i] = ((uint64_t)b << 32) | (uint32_t)e;
+                fn(i, rebase_bits((uint32_t)(e >> 32), t.delta[g]), (uint32_t)e);
             }
             i = iend;
         }
@@ -1007,14 +976,99 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
             }
 #pragma unroll
             for (int u = 0; u < kBatch; ++u)
-                if ((uint32_t)u < n) {
-                    uint32_t b = rebase_bits((uint32_t)(e[u] >> 32), t.delta[sl[u]]);
-                    if (b < cutrow) b = 0;                             // plan B: below the complete part; 0 matches nothing
-                    t.list[i + (uint32_t)u] = ((uint64_t)b << 32) | (uint32_t)e[u];
-                }
+                if ((uint32_t)u < n) fn(i + (uint32_t)u, rebase_bits((uint32_t)(e[u] >> 32), t.delta[sl[u]]), (uint32_t)e[u]);
             i += n;
         }
+    };
+    take_prefix(mtake);
+    bool subset = false;                                               // plan B in force
+    bool listed = false;                                               // the list has been filled already
+    uint32_t cutrow = 0;
+    if (t.fail || t.take[kThreads - 1] != total) {
+        // Plan B (flat distributions: the boundary bin holds thousands of tokens, but top_k is small):
+        // take the stashes whole.  Together they hold every token of the row at or above
+        // cutrow = the largest of the slices' cuts, so a threshold found among those is the row's.
+        uint32_t mycut = 0;
+        if ((uint32_t)tid < G) {
+            // a cut that lands below 2^-40 in the row's frame: what the stash lacks is dead there
+            mycut = max(rebase_bits(ph.cut, dl), kEMinBits);
+        }
+        cutrow = block_max_u32(s, mycut, lane, wave);
+        take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
+        total = t.take[kThreads - 1];
+        if (!FUSED && total > v.list_cap && (uint32_t)p.top_k <= v.list_cap / 2u) {
+            // More stashed tokens than the list holds (a flat row cut into many slices, each of which
+            // stashed several times its share of top_k).  The kept set is at most top_k tokens, so only
+            // the stashed tokens down to some value T at or above which there are at least top_k of
+            // them are needed: T from a count of the stashed tokens in steps of 1/512 octave below the
+            // row's largest (one pass over the stashes, which sit in the L2), the tokens at or above T
+            // into the list by a second pass.  T is at or above cutrow, so the list is complete above T.
+            const uint32_t topkey = e_bits_of(xmax, M) >> 14;
+            uint32_t *cnt = reinterpret_cast<uint32_t *>(t.blo);                // 512 counters
+            cnt[tid] = 0u; cnt[tid + kThreads] = 0u;
+            if (tid == 0) { s.ctr = 0u; s.bc32[4] = 0xFFFFFFFFu; s.bc32[5] = 0u; }
+            __syncthreads();
+            stashed(total, [&](uint32_t, uint32_t b, uint32_t) {
+                if (b >= cutrow) atomicAdd(&cnt[min(511u, topkey - (b >> 14))], 1u);
+            });
+            __syncthreads();
+            if (wave == 0) {
+                uint32_t c8 = 0;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) c8 += cnt[lane * 8 + q];
+                const uint32_t inc = wave_inclusive_scan(c8);
+                uint32_t run = inc - c8;
+                if (run < (uint32_t)p.top_k && (uint32_t)p.top_k <= inc) {
+                    bool done = false;
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        run += cnt[lane * 8 + q];
+                        if (!done && run >= (uint32_t)p.top_k) { s.bc32[4] = (uint32_t)(lane * 8 + q); s.bc32[5] = run; done = true; }
+                    }
+                }
+            }
+            __syncthreads();
+            const uint32_t step = s.bc32[4], nge = s.bc32[5];
+            if (step >= 511u || nge > v.list_cap) return slow();              // fewer than top_k at or above cutrow, or one value thousands of times
+            cutrow = max(cutrow, (topkey - step) << 14);
+            stashed(total, [&](uint32_t, uint32_t b, uint32_t idx) {
+                if (b >= cutrow) {
+                    const uint32_t o = atomicAdd(&s.ctr, 1u);
+                    if (o < v.list_cap) t.list[o] = ((uint64_t)b << 32) | idx;
+                }
+            });
+            __syncthreads();
+            total = nge;
+            subset = true; listed = true;
+            // Two more passes over the stashes make this finish slower than the general kernel's whole
+            // call while the call is of moderate size (measured: 64 flat rows of 131072 with top_k 1000,
+            // 51 against 38 us; 128 rows of 262144, 77 against 117): such a call says so to the caller's
+            // policy, as it did when these rows still went the slow way.
+            if ((uint64_t)p.B * (uint64_t)p.V < (1ull << 24)) tell_policy();
+        } else {
+        if (total > v.list_cap || total == 0u) {
+            // not resolvable from the stashes
+            if (FUSED) return false;
+            return slow();
+        }
+        subset = true;
+        }
     }
+
+    // A nucleus of thousands of tokens is finished here all the same, but one workgroup going through
+    // such a list a dozen times takes longer than the general kernel needs for the whole call (measured:
+    // 128 rows of 50304, about 4000 tokens each, 54 against 36 us; the two meet at about 2400 tokens
+    // there and, the general kernel's time growing with the row, at about 4700 for rows of 100256): a
+    // call that is only an attempt (no top_k bounds the kept set) says so to the caller's policy.
+    const uint32_t long_list = max(2048u, (uint32_t)p.V / 20u);
+    if (!FUSED && p.report == 1u && total > long_list) tell_policy();
+
+    // gather the tokens, re-based to the row's frame
+    if (!listed)
+        stashed(total, [&](uint32_t i, uint32_t b, uint32_t idx) {
+            if (b < cutrow) b = 0;                                     // plan B: below the complete part; 0 matches nothing
+            t.list[i] = ((uint64_t)b << 32) | idx;
+        });
     __syncthreads();
     uint32_t exb = f.bin >> 2;
     if (subset) {

@@ -429,6 +429,29 @@ def test_streaming_path_few_long_rows(torch_cuda, oracle, B, V):
                   what="few long rows B=%d V=%d k=%s p=%s T=%s" % (B, V, k, p, t))
 
 
+@pytest.mark.parametrize("B,V,k", [(4, 262144, 1000), (3, 262144, 1024), (24, 100256, 1000), (2, 1048576, 600), (6, 152064, 700)])
+def test_streaming_path_flat_rows_more_stashed_than_listed(torch_cuda, oracle, B, V, k):
+    """Flat rows (the reference's benchmark generators U[0,1), U[0,1)*4, N(0,1)/2) with a top_k of
+    several hundred, cut into many slices: the boundary bin holds tens of thousands of tokens, every
+    slice stashes several times its share of top_k, and the stashes together hold more tokens than
+    the finishing workgroup's list.  It then counts the stashed tokens in steps of 1/512 octave below
+    the row's largest, takes those down to the step at which there are top_k of them, and goes on from
+    there: such rows finish on the streaming path (diag.rounds == 0), with a nucleus or without."""
+    from tests import capi
+    torch = torch_cuda
+    rng = np.random.default_rng(V + k)
+    gens = [lambda: rng.random(V, dtype=np.float32), lambda: rng.random(V, dtype=np.float32) * np.float32(4),
+            lambda: rng.standard_normal(V, dtype=np.float32) * np.float32(0.5)]
+    lg = np.stack([gens[b % 3]() for b in range(B)])
+    for (p, t) in [(1.0, 1.0), (0.9, 1.0), (0.3, 0.7)]:
+        _run_case(torch, oracle, capi, lg, t, k, p, u_np=H.uniforms(B, k + int(p * 10)),
+                  what="flat rows B=%d V=%d k=%d p=%s T=%s" % (B, V, k, p, t))
+    rc, c, kk, pp = capi.normalize(1.0, k, 1.0, V, B, 1)
+    smp = capi.Sampler(B, V)
+    res = smp.sample(torch.from_numpy(lg).cuda(), c, kk, pp, uniforms=torch.from_numpy(H.uniforms(B, 1)).cuda(), path="stream")
+    assert (res["diag"]["rounds"] == 0).all(), res["diag"]["rounds"]
+
+
 @pytest.mark.parametrize("B,V", [(11, 50304), (4, 262144), (40, 152064), (2, 1048576), (3, 528384), (1, 4096)])
 def test_streaming_path_keeps_everything(torch_cuda, oracle, B, V):
     """Plain temperature sampling (top_k = V, top_p = 1): every live token is kept, so there is no
