@@ -326,7 +326,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 410; }
+int rs_version(void) { return 411; }
 
 const char *rs_error_string(int code)
 {

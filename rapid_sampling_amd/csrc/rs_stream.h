@@ -996,9 +996,11 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         cutrow = block_max_u32(s, mycut, lane, wave);
         take_prefix((uint32_t)tid < G ? min(ph.n, (uint32_t)kStashCap) : 0u);
         total = t.take[kThreads - 1];
-        if (!FUSED && total > v.list_cap && (uint32_t)p.top_k <= v.list_cap / 2u) {
+        if (!FUSED && total > min(v.list_cap, max(2048u, 3u * (uint32_t)p.top_k)) && (uint32_t)p.top_k <= v.list_cap / 2u) {
             // More stashed tokens than the list holds (a flat row cut into many slices, each of which
-            // stashed several times its share of top_k).  The kept set is at most top_k tokens, so only
+            // stashed several times its share of top_k), or several times top_k of them (going through
+            // a list of thousands a dozen times costs more than these two passes: 128 flat rows of
+            // 100256 with top_k 1000, 60 against 70 us).  The kept set is at most top_k tokens, so only
             // the stashed tokens down to some value T at or above which there are at least top_k of
             // them are needed: T from a count of the stashed tokens in steps of 1/512 octave below the
             // row's largest (one pass over the stashes, which sit in the L2), the tokens at or above T
