@@ -450,6 +450,17 @@ def test_streaming_path_flat_rows_more_stashed_than_listed(torch_cuda, oracle, B
     smp = capi.Sampler(B, V)
     res = smp.sample(torch.from_numpy(lg).cuda(), c, kk, pp, uniforms=torch.from_numpy(H.uniforms(B, 1)).cuda(), path="stream")
     assert (res["diag"]["rounds"] == 0).all(), res["diag"]["rounds"]
+    # a call of this size (fewer than 2^24 tokens) says so to a caller's policy all the same: the general
+    # kernel does such a call faster, and the next one goes there
+    pol = capi.Sampler(B, V, with_policy=True, init=True)
+    u = torch.from_numpy(H.uniforms(B, 1)).cuda()
+    first = pol.sample(torch.from_numpy(lg).cuda(), c, kk, pp, uniforms=u)
+    assert (first["diag"]["rounds"] == 0).all() and np.array_equal(first["out"], res["out"])
+    if V * B < (1 << 24) and V != 152064:                # (6, 152064, 700): the stashes fit the list, nothing to report
+        assert pol.policy_state() == 2
+        second = pol.sample(torch.from_numpy(lg).cuda(), c, kk, pp, uniforms=u)
+        assert (second["diag"]["rounds"] >= 1).all() and np.array_equal(second["out"], res["out"])
+    pol.close()
 
 
 @pytest.mark.parametrize("B,V", [(11, 50304), (4, 262144), (40, 152064), (2, 1048576), (3, 528384), (1, 4096)])
