@@ -36,6 +36,7 @@ extern "C" {
 #define RS_ERR_LAUNCH      -8   /* the HIP runtime refused the launch                         */
 #define RS_ERR_DEVICE      -9   /* a kernel gave up waiting for its peer workgroups           */
 #define RS_ERR_SCRATCH     -10  /* rs_sample_static: the call needs more than RS_STATIC_SCRATCH_BYTES */
+#define RS_ERR_UNSUPPORTED -11  /* the current device is not a whole MI355X (256 compute units)     */
 
 /* Bytes of RNG state per row.  Same size as the reference's
  * curandStatePhilox4_32_10_t record (sampling.cu:9,141) so that the opaque
@@ -268,6 +269,7 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
 #define RS_PATH_STREAM  2
 #define RS_PATH_ATTEMPT 3
 #define RS_PATH_FUSED   4
+#define RS_PATH_WIDE    5
 typedef struct rs_options {
     int32_t    path;
     int32_t    slice_r;
@@ -292,14 +294,27 @@ int rs_sample_ex(const void *logits_device, int32_t logits_dtype, int64_t row_st
  * The workspace is a static array in device memory inside the library,
  * RS_STATIC_SCRATCH_BYTES (32 MiB) on every GPU the library is used on, held
  * until the process ends.  A call whose rs_workspace_bytes(B, V) exceeds that
- * size is refused with RS_ERR_SCRATCH before anything is launched (64 rows of
- * 152064 tokens need 16 MiB, 32 rows of 131072 tokens 14 MiB; 128 rows of
- * 1048576 tokens, 105 MB, do not fit).  The call allocates nothing and
- * synchronises nothing: it enqueues one small kernel that clears the launch
- * header and the B row records the call is about to use (so it also recovers
- * by itself after an RS_ERR_DEVICE), then exactly what rs_sample_ex enqueues.
- * The address of the array is looked up once per device, on the first call
- * made while that device is current.
+ * size is refused with RS_ERR_SCRATCH (64 rows of 152064 tokens need 16 MiB,
+ * 32 rows of 131072 tokens 14 MiB; 128 rows of 1048576 tokens, 105 MB, do not
+ * fit).  Every check that can refuse a call -- arguments, alignment, size, the
+ * device -- is made before anything is launched.  The call allocates nothing
+ * and synchronises nothing: it enqueues one small kernel that clears the
+ * launch counters of the array's header and the B row records the call is
+ * about to use, then exactly what rs_sample_ex enqueues; so a call starts from
+ * clean records whatever the one before it left, also after RS_ERR_DEVICE.
+ * The sticky error word of the array, the place of the first wait that gave
+ * up, the wait limit and the words of the routing report survive that clearing:
+ * with `options->policy` the reports work as they do with a workspace of the
+ * caller's own, and without one a caller learns of a kernel that gave up a
+ * wait from rs_static_status (the call that gave up returned RS_OK and left
+ * garbage in out_device, as rs_sample_ex does).
+ *
+ * The address of the array is looked up once per device, with
+ * hipGetSymbolAddress, on the first call made while that device is current --
+ * which must therefore happen outside stream capture: call rs_static_prepare()
+ * (or make one ordinary call) on each device before capturing.  The array of
+ * the CURRENT device is used; a `stream` of another device is refused
+ * (RS_ERR_ARG).
  *
  * Every call on a GPU uses that GPU's one array: calls must be ordered on one
  * stream (or otherwise serialised); calls that overlap on one GPU race.
@@ -313,6 +328,19 @@ int rs_sample_static(const void *logits_device, int32_t logits_dtype, int64_t ro
                      float log2e_inv_temp, int32_t top_k, float top_p,
                      rs_row_diag *diag_device, uint32_t *e_bits_device,
                      const rs_options *options, void *stream);
+
+/* Looks up the static array's address on the current device (no GPU work, no
+ * allocation); to be called once per device before rs_sample_static is used
+ * under stream capture.  No counterpart in the reference. */
+int rs_static_prepare(void);
+
+/*
+ * The sticky error word of the current device's static array (synchronises
+ * `stream`): *status = RS_OK or RS_ERR_DEVICE; where[4], if not NULL, as
+ * rs_workspace_where.  With clear != 0 a reported error is put back to RS_OK
+ * by a one-thread kernel on `stream`.  No counterpart in the reference.
+ */
+int rs_static_status(int32_t *status, uint32_t where[4], int32_t clear, void *stream);
 
 /*
  * Launch-plus-one-read floor: a kernel that reads every logit of the B rows once

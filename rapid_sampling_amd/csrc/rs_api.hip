@@ -16,9 +16,9 @@
 // Everything summed across tokens is an integer, so the result does not depend
 // on how a row is cut up or in which order the pieces arrive.
 //
-// Two ways through these steps:
+// Ways through these steps (choose_path below; the results are the same integers on every one):
 //
-//   cluster path (sample_kernel, one launch): a row is worked by a CLUSTER of
+//   general kernel (sample_kernel, one launch): a row is worked by a CLUSTER of
 //     G workgroups of 256 threads; each thread keeps R float4 (4R tokens) in
 //     registers for the whole call, so the row is read from HBM exactly once.
 //     The workgroups of a cluster exchange histograms, the slice maxima, the
@@ -27,13 +27,25 @@
 //     add up, words that are non-zero once written), every wait is bounded.
 //     Any top_k / top_p, penalties, any batch.
 //
-//   streaming path (stream_kernel, finish_kernel, sample_list_kernel): for
+//   streaming path (stream_kernel + finish_kernel, two launches, no waits): for
 //     calls of 2^17 tokens and more without penalties whose kept set is small
-//     next to the row (top_k <= 1024, or a small nucleus).  No workgroup waits
-//     for another: one pass over the logits leaves per-row histograms and
-//     per-slice stashes of the largest tokens, a small kernel finishes each
-//     row from them, and rows it cannot finish that way go through the
-//     cluster kernel afterwards.
+//     next to the row (top_k <= 1024, or a small nucleus), and, as a counting-only
+//     variant, for calls that keep every token.  One pass over the logits leaves
+//     per-row histograms and per-slice stashes of the largest tokens; one
+//     workgroup per row finishes the row from them.  A row it cannot finish that
+//     way it does alone, from the logits (finish_row_slow), and says so to the
+//     caller's rs_policy, which routes the next calls of that kind.
+//
+//   wide path (stream_kernel counting only + wide_kernel + wide_finish_kernel,
+//     three launches, no waits): kept sets of thousands of tokens (top_k > 1024,
+//     flat distributions under top_p).  The second pass reads the rows again with
+//     the boundary bin of the first known, counts the bin's next digit and sets
+//     aside the tokens around the place where each slice expects the threshold.
+//
+//   one-launch path (fused_kernel): the streaming pass and the finish in one
+//     grid, for calls with penalties that fit the device at once.
+//
+//   penalties at scale (stream_pen_kernel + finish_kernel + penalty_fix_kernel).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -98,12 +110,25 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint4 *dst, size_t n16, 
 
 __global__ void set_u32_kernel(uint32_t *dst, uint32_t value) { *dst = value; }
 
-// What a call reads before it writes: the launch header and its row records.
-__global__ void __launch_bounds__(256) clear_records_kernel(uint4 *hdr, uint4 *recs, size_t n16)
+// What a call reads before it writes: the launch counters of the header (workgroups that have left,
+// the eight ticket counters) and its row records.  The sticky error word, the place of the first wait
+// that gave up, the wait limit and the words of the routing report (n_need, last_call) are left as
+// they are: they are read across calls.
+__global__ void __launch_bounds__(256) clear_records_kernel(WsHeader *hdr, uint4 *recs, size_t n16)
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) recs[i] = make_uint4(0u, 0u, 0u, 0u);
-    if (blockIdx.x == 0 && threadIdx.x < sizeof(WsHeader) / 16) hdr[threadIdx.x] = make_uint4(0u, 0u, 0u, 0u);
+    if (blockIdx.x == 0) {
+        if (threadIdx.x == 0) hdr->finished = 0u;
+        for (uint32_t i = threadIdx.x; i < 8u * 64u; i += 256u) hdr->ticket[i >> 6][i & 63u] = 0u;
+    }
+}
+
+// Puts the sticky error word and the record of the first wait that gave up back to "none".
+__global__ void clear_error_kernel(WsHeader *hdr)
+{
+    hdr->error = 0;
+    hdr->gave_up[0] = 0u; hdr->gave_up[1] = 0u; hdr->gave_up[2] = 0u; hdr->gave_up[3] = 0u;
 }
 
 // ------------------------------------------------------------ host side ----
@@ -207,16 +232,17 @@ static size_t stream_bytes(int32_t B, int32_t V)
 
 }  // namespace rs
 
-// The caller's routing state (see rapid_sampling.h).  word[0], word[1]: "a row had to be done the
-// slow way" as last reported by a streaming call with / without a bounding top_k; word[2]:
-// RS_ERR_DEVICE once a kernel gave up a wait.  away[]: calls routed away from the streaming path
+// The caller's routing state (see rapid_sampling.h).  word[0], word[1], word[3]: "a row had to be done
+// the slow way" as last reported by a streaming call with / without a bounding top_k and by a call on
+// the wide path; word[2]: RS_ERR_DEVICE once a kernel gave up a wait.  away[]: calls routed away from the streaming path
 // since the word was last seen set and streaming tried; period[]: how many of them before streaming
 // is tried again; good[]: streaming calls in a row that found the word clear.
 constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u;
 struct rs_policy {
     int32_t *word;
-    uint32_t away[2], period[2], good[2];
+    uint32_t away[3], period[3], good[3];                // kinds: 0 streaming with a bounding top_k, 1 without, 2 the wide path
 };
+static inline int policy_word(int kind) { return kind == 2 ? 3 : kind; }    // word[2] is the error report
 
 namespace rs {
 
@@ -237,7 +263,11 @@ namespace rs {
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
-enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4 };
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5 };
+// The wide path (three launches, two reads of the logits) against the general kernel (one launch, its
+// exchanges): from this many tokens per call on the wide path is taken for kept sets the streaming
+// path cannot stash.
+constexpr uint64_t kWideMin = 1ull << 20;
 constexpr uint64_t kPenStreamMin = 1ull << 23;
 // Plain temperature sampling (top_k = V, top_p = 1: every live token is kept) has no kept set to
 // stash, but the streaming pass's bins alone say which slice holds the target: one pass at
@@ -283,7 +313,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     // after a call of this kind with a slow row: the general kernel for a while, then another try
     auto routed_away = [&](int kind) {
         if (!pol) return false;
-        if (*(volatile int32_t *)(pol->word + kind) == 0) {
+        if (*(volatile int32_t *)(pol->word + policy_word(kind)) == 0) {
             if (pol->period[kind] > kAwayFirst && ++pol->good[kind] >= pol->period[kind]) pol->period[kind] = kAwayFirst;
             pol->away[kind] = 0;
             return false;
@@ -304,11 +334,16 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (keep_all && (force == RS_PATH_STREAM || force == RS_PATH_ATTEMPT)) return kPathKeep;
     if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
     if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
+    if (force == RS_PATH_WIDE) return keep_all ? kPathKeep : kPathWide;
     if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
     if (keep_all && V >= 32768) return kPathKeep;              // shorter rows: one workgroup of the general kernel does a row in one go
-    if (!bounded && !(top_p < 1.0f)) return kPathCluster;      // a top_k of thousands and no nucleus: more than the stashes hold
-    if (!pol) return bounded ? kPathStream : kPathCluster;
-    return routed_away(bounded ? 0 : 1) ? kPathCluster : bounded ? kPathStream : kPathAttempt;
+    // kept sets the stashes cannot hold: the wide path from kWideMin tokens on, unless its rows have been
+    // going the slow way (slices that are no fair samples of their rows, ties of thousands of tokens)
+    auto wide_or_general = [&]() { return (uint64_t)B * (uint64_t)V >= kWideMin && !routed_away(2) ? kPathWide : kPathCluster; };
+    if (!bounded && !(top_p < 1.0f)) return wide_or_general(); // a top_k of thousands and no nucleus: more than the stashes hold
+    if (!pol) return bounded ? kPathStream : wide_or_general();
+    if (!routed_away(bounded ? 0 : 1)) return bounded ? kPathStream : kPathAttempt;
+    return bounded ? kPathCluster : wide_or_general();
 }
 
 static hipError_t fill_zero(void *dst, size_t bytes, hipStream_t st)
@@ -342,6 +377,7 @@ const char *rs_error_string(int code)
     case RS_ERR_LAUNCH:      return "HIP launch failed";
     case RS_ERR_DEVICE:      return "a workgroup gave up waiting for its peers";
     case RS_ERR_SCRATCH:     return "the call needs a larger workspace than the static scratch of rs_sample_static (RS_STATIC_SCRATCH_BYTES)";
+    case RS_ERR_UNSUPPORTED: return "the device is not a whole MI355X (256 compute units in 8 XCDs): the kernels' waits are only known to end on one";
     default:                 return "unknown error";
     }
 }
@@ -417,7 +453,7 @@ int rs_policy_create(rs_policy **out)
     rs_policy *pol = new (std::nothrow) rs_policy;
     if (!pol) return RS_ERR_LAUNCH;
     pol->word = nullptr;
-    for (int i = 0; i < 2; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
+    for (int i = 0; i < 3; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
     if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
         delete pol;
         return RS_ERR_LAUNCH;
@@ -438,7 +474,7 @@ int rs_policy_state(const rs_policy *pol, int32_t *state)
 {
     if (!pol || !state) return RS_ERR_NULL;
     const volatile int32_t *w = pol->word;
-    *state = (w[1] != 0 ? 1 : 0) | (w[0] != 0 ? 2 : 0);
+    *state = (w[1] != 0 ? 1 : 0) | (w[0] != 0 ? 2 : 0) | (w[3] != 0 ? 4 : 0);
     return RS_OK;
 }
 
@@ -484,6 +520,41 @@ int rs_sample_dtype(const void *logits, int32_t logits_dtype, int64_t row_stride
                         nullptr, stream);
 }
 
+// The argument checks of a sampling call; nothing is launched before they pass.
+static int check_call(const void *logits, int32_t logits_dtype, int64_t row_stride, const float *penalties, const int32_t *out,
+                      const void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                      float log2e_inv_temp, int32_t top_k, float top_p, const uint32_t *e_bits, const rs_options *opt)
+{
+    if (!logits || !out || (!rng_state && !injected_u)) return RS_ERR_NULL;
+    if (logits_dtype != RS_DTYPE_F32 && logits_dtype != RS_DTYPE_BF16 && logits_dtype != RS_DTYPE_F16) return RS_ERR_ARG;
+    if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
+    if (B <= 0) return RS_ERR_BATCH;
+    if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
+    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_WIDE || opt->slice_r < 0)) return RS_ERR_ARG;
+    if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
+        return RS_ERR_ALIGN;
+    return RS_OK;
+}
+
+// Compute units of the current device, looked up once per device (a host-side table lookup, no GPU
+// work).  Every path with waits -- the general kernel, the one-launch kernel -- sizes its launches and
+// its tickets for a whole MI355X: 256 compute units in 8 XCDs.  A partitioned device (compute-partition
+// modes) or a CU-masked process holds fewer workgroups than those launches assume, rows could starve
+// and every such call would end in a 2 s bounded wait: such a device is refused instead.
+static int device_is_whole()
+{
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cus[kMaxDevices];            // 0 = not looked up yet
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return RS_ERR_LAUNCH;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (!n) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return RS_ERR_LAUNCH;
+        cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return n == 256 ? RS_OK : RS_ERR_UNSUPPORTED;
+}
+
 int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
                  void *rng_state, const float *injected_u, int32_t B, int32_t V,
                  float presence, float repetition, float decay,
@@ -491,17 +562,15 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
                  void *workspace, size_t workspace_bytes,
                  rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
 {
-    if (!logits || !out || !workspace || (!rng_state && !injected_u)) return RS_ERR_NULL;
-    if (logits_dtype != RS_DTYPE_F32 && logits_dtype != RS_DTYPE_BF16 && logits_dtype != RS_DTYPE_F16) return RS_ERR_ARG;
-    if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
-    if (B <= 0) return RS_ERR_BATCH;
-    if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
-    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_FUSED || opt->slice_r < 0)) return RS_ERR_ARG;
-    if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
-        return RS_ERR_ALIGN;
+    if (!workspace) return RS_ERR_NULL;
+    const int bad = check_call(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, log2e_inv_temp,
+                               top_k, top_p, e_bits, opt);
+    if (bad != RS_OK) return bad;
     size_t need = 0;
     rs_workspace_bytes(B, V, &need);
     if (workspace_bytes < need || ((uintptr_t)workspace & 255)) return RS_ERR_WORKSPACE;
+    const int whole = device_is_whole();
+    if (whole != RS_OK) return whole;
 
     const bool pen = penalties != nullptr;
     const Geometry g = choose_geometry(B, V, pen, opt ? opt->slice_r : 0);
@@ -547,8 +616,13 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         // with static LDS alone -- with a 64 KB list in dynamic LDS it was 32 x 1, and rows of 33 and
         // more slices could, rarely, starve until their waits gave up.
         if (path == kPathFused) v.list_cap = 2048u;
-        p.report = path == kPathAttempt ? 1u : 0u;
+        p.report = path == kPathAttempt ? 1u : path == kPathWide ? 3u : 0u;
         if (path == kPathKeep) { p.stash_k = 1u; v.list_cap = 2048u; }
+        if (path == kPathWide) {
+            // the list holds the tokens of ONE sub-bin of the boundary bin: 1/128 of it for a smooth distribution
+            p.stash_k = 1u; v.list_cap = 4096u;
+            return launch_wide(sr, logits_dtype, (uint32_t)B, (size_t)v.list_cap * sizeof(uint64_t), st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+        }
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (path == kPathFused)
             return launch_fused(sr, pen, (uint32_t)B, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
@@ -564,17 +638,10 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     return launch_sample(pen, g.R, grid, (hipStream_t)stream, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
 }
 
-int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
-                     void *rng_state, const float *injected_u, int32_t B, int32_t V,
-                     float presence, float repetition, float decay,
-                     float log2e_inv_temp, int32_t top_k, float top_p,
-                     rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
+// The static workspace of the current device: the array's address on that device, looked up once per
+// device (every GPU holds its own copy of the array at its own address).
+static int static_base(void **out)
 {
-    size_t need = 0;
-    const int rc = rs_workspace_bytes(B, V, &need);
-    if (rc != RS_OK) return rc;
-    if (need > (size_t)RS_STATIC_SCRATCH_BYTES) return RS_ERR_SCRATCH;
-    // every GPU holds its own copy of the array at its own address: looked up once per device
     constexpr int kMaxDevices = 64;
     static std::atomic<void *> base[kMaxDevices];
     int dev = -1;
@@ -584,14 +651,66 @@ int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_strid
         if (hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch)) != hipSuccess || !ws) return RS_ERR_LAUNCH;
         base[dev].store(ws, std::memory_order_release);
     }
+    *out = ws;
+    return RS_OK;
+}
+
+int rs_static_prepare(void)
+{
+    void *ws = nullptr;
+    return static_base(&ws);
+}
+
+int rs_static_status(int32_t *status, uint32_t where[4], int32_t clear, void *stream)
+{
+    if (!status) return RS_ERR_NULL;
+    void *ws = nullptr;
+    const int rc = static_base(&ws);
+    if (rc != RS_OK) return rc;
+    int r = rs_workspace_status(ws, status, stream);
+    if (r == RS_OK && where) r = rs_workspace_where(ws, where, stream);
+    if (r == RS_OK && clear && *status != RS_OK) {
+        hipLaunchKernelGGL(clear_error_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, (WsHeader *)ws);
+        if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
+    }
+    return r;
+}
+
+int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_stride, float *penalties, int32_t *out,
+                     void *rng_state, const float *injected_u, int32_t B, int32_t V,
+                     float presence, float repetition, float decay,
+                     float log2e_inv_temp, int32_t top_k, float top_p,
+                     rs_row_diag *diag, uint32_t *e_bits, const rs_options *opt, void *stream)
+{
+    // everything that can refuse the call comes before the first launch
+    const int bad = check_call(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, log2e_inv_temp,
+                               top_k, top_p, e_bits, opt);
+    if (bad != RS_OK) return bad;
+    size_t need = 0;
+    const int rc = rs_workspace_bytes(B, V, &need);
+    if (rc != RS_OK) return rc;
+    if (need > (size_t)RS_STATIC_SCRATCH_BYTES) return RS_ERR_SCRATCH;
+    const int whole = device_is_whole();
+    if (whole != RS_OK) return whole;
+    // the array of the CURRENT device is used, so the stream must belong to that device
+    if (stream) {
+        int cur = -1;
+        hipDevice_t sdev = -1;
+        if (hipGetDevice(&cur) != hipSuccess || hipStreamGetDevice((hipStream_t)stream, &sdev) != hipSuccess) return RS_ERR_LAUNCH;
+        if ((int)sdev != cur) return RS_ERR_ARG;
+    }
+    void *ws = nullptr;
+    const int rb = static_base(&ws);
+    if (rb != RS_OK) return rb;
     // The array keeps what the last call left.  A call leaves it clean unless a wait gave up; the launch
-    // header and this call's row records are cleared all the same, by a kernel (not a memset node: the
-    // call may be under capture), so that every call starts from zero whatever came before.
+    // counters and this call's row records are cleared all the same, by a kernel (not a memset node: the
+    // call may be under capture), so that every call starts from zero whatever came before.  The sticky
+    // error word stays (rs_static_status reads and clears it), and so do the words of the routing report.
     const size_t rec_bytes = (size_t)B * sizeof(RowCtl);
     char *recs = (char *)ws + (size_t)RS_STATIC_SCRATCH_BYTES - rec_bytes;
     const size_t n16 = rec_bytes / 16;
     const uint32_t blocks = (uint32_t)(n16 / 1024 < 1 ? 1 : n16 / 1024 > 1024 ? 1024 : n16 / 1024);
-    hipLaunchKernelGGL(clear_records_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint4 *)ws, (uint4 *)recs, n16);
+    hipLaunchKernelGGL(clear_records_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (WsHeader *)ws, (uint4 *)recs, n16);
     if (hipGetLastError() != hipSuccess) return RS_ERR_LAUNCH;
     return rs_sample_ex(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, presence,
                         repetition, decay, log2e_inv_temp, top_k, top_p, ws, (size_t)RS_STATIC_SCRATCH_BYTES, diag,

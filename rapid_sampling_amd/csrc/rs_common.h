@@ -31,7 +31,7 @@ struct alignas(256) WsHeader {
     int32_t  error;       // sticky RS_ERR_DEVICE
     uint32_t n_need;      // rows of the running (or last) streaming call that the finishing workgroups did the slow way
     uint32_t spin_ticks;  // bound of a wait in units of 1024 wall-clock ticks; 0 = the default (2 s)
-    uint32_t last_call;   // 1 | kind << 31 after a streaming call that no later call has reported on yet (kind: 0 top_k bounds the kept set, 1 not), else 0
+    uint32_t last_call;   // 1 | word << 8 after a streaming call that no later call has reported on yet (word: the report word of the caller's policy the call writes, Params::report), else 0
     uint32_t gave_up[4];  // the first wait that gave up since the workspace was set up: site, row << 16 | slice, what it had, what it waited for
     uint32_t pad[54];
     // Logical workgroup ids of a launch larger than the device holds at once: eight counters, one per
@@ -82,8 +82,8 @@ struct Params {
     RowCtl      *ctl_end;      // one past the record of row 0; row r is ctl_end[-1 - r]
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     int32_t      dtype;        // RS_DTYPE_* of the logits
-    uint32_t     report;       // which of the two report words a streaming call writes: 0 top_k bounds the kept set, 1 not
-    int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1] routing reports, [2] error; or null
+    uint32_t     report;       // which report word of the caller's policy a streaming call writes: 0 top_k bounds the kept set, 1 not, 3 the wide path
+    int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1], [3] routing reports, [2] error; or null
     int32_t      defer_pen;    // penalties enter x but are left as they are: a later pass over them applies decay and one-hot add
     int64_t      row_stride;
     int32_t      B, V;
@@ -336,16 +336,16 @@ __device__ __forceinline__ PrevCall report_begin(const Params &p)
 {
     PrevCall pc;
     pc.slow_rows = __hip_atomic_exchange(&p.hdr->n_need, 0u, __ATOMIC_RELAXED, RS_AGENT);
-    pc.meta = a_load(&p.hdr->last_call);                 // 1 | kind << 31 of a streaming call not yet reported on, else 0
+    pc.meta = a_load(&p.hdr->last_call);                 // 1 | word << 8 of a streaming call not yet reported on, else 0
     return pc;
 }
 // `streaming`: the reporting call is a streaming call itself, to be reported on by the next one
 __device__ __forceinline__ void report_end(const Params &p, const PrevCall &pc, const bool streaming)
 {
-    if (streaming) a_store(&p.hdr->last_call, 1u | (p.report << 31));
+    if (streaming) a_store(&p.hdr->last_call, 1u | (p.report << 8));
     else if (pc.meta) a_store(&p.hdr->last_call, 0u);
     if (p.host_words && pc.meta)
-        __hip_atomic_store(p.host_words + (pc.meta >> 31), pc.slow_rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(p.host_words + ((pc.meta >> 8) & 3u), pc.slow_rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 __device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)
@@ -470,8 +470,8 @@ __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G,
 // scans this workgroup's own histogram s.hm and returns its mass above the
 // boundary bin in local_above.  With GIVEN_P the histogram is that of a
 // subset of the row which is complete above some value: D and P are left alone.
-template <bool LOCAL, bool GIVEN_P = false>
-__device__ __forceinline__ Found hist_find_level1(Lds &s, uint64_t top_k, float top_p, int lane, int wave)
+template <bool LOCAL, bool GIVEN_P = false, typename L = Lds>
+__device__ __forceinline__ Found hist_find_level1(L &s, uint64_t top_k, float top_p, int lane, int wave)
 {
     if (wave == 0) {
         uint32_t c[3]; u128 m[3], hl[3];
@@ -483,7 +483,7 @@ __device__ __forceinline__ Found hist_find_level1(Lds &s, uint64_t top_k, float 
             c[i] = pack_count(w);
             m[i] = w ? pack_mass(w, (uint32_t)idx >> 2) : (u128)0;
             cs += c[i]; ms += m[i];
-            if (LOCAL) {
+            if constexpr (LOCAL) {
                 const uint64_t h = idx >= (int)kBin0 ? s.hm[idx] : 0ull;
                 hl[i] = h ? pack_mass(h, (uint32_t)idx >> 2) : (u128)0;
                 hs += hl[i];
@@ -667,5 +667,6 @@ hipError_t launch_penalty_pass(hipStream_t st, const Params &p);
 hipError_t launch_stream(int slice_r, int32_t dtype, bool keep, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
                          const StreamView &v);
 hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v);
+hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
 
 }  // namespace rs

@@ -366,7 +366,8 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : RS_STREAM_WAVES)) stream_ker
             eb[j * 4 + 2] = __float_as_uint(x2); eb[j * 4 + 3] = __float_as_uint(x3);
         }
     }
-    if (reporter) report_end(p, prev, !KEEP);                // a call that keeps everything has no rows to report on
+    // a call that keeps everything has no rows to report on; the counting-only pass of the wide path does
+    if (reporter) report_end(p, prev, !KEEP || p.report == 3u);
     slice_count_and_stash<R, NT, kRep, false, KEEP>(p, v, s, eb, lmax, row, part, base4, nv);
 }
 
@@ -656,18 +657,18 @@ __device__ __forceinline__ void finish_row_slow(const Params &p, Lds &s, LdsB &t
 // atomics, no list.  (An earlier version gave every thread 16 consecutive groups: its loads, 64
 // cache lines per instruction and every line touched by 8 instructions, cost a microsecond per
 // group.)  No penalties on this path.
-template <int SLICE_LOG2>
-__device__ __forceinline__ void keep_pick(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float M, const uint32_t lo_idx, const u128 r)
+// `kept`: weight of a token from the bit pattern of its e in the row's frame (its full weight when the
+// call keeps every live token; on the wide path what the threshold and the tie weight leave of it).
+template <int SLICE_LOG2, typename WF>
+__device__ __forceinline__ void keep_pick(const Params &p, Lds &s, LdsB &t, const uint32_t row, const float M, const uint32_t lo_idx, const u128 r,
+                                          WF kept)
 {
     constexpr int N = 1 << (SLICE_LOG2 - 10);                      // chunks per wave
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const char *lrow = logits_row(p, row);
     const uint32_t g0 = lo_idx >> 2;
-    auto weight = [&](float l) -> uint64_t {
-        const uint32_t b = e_bits_of(sf(l * p.c), M);
-        return b >= kEMinBits ? w_of_bits(b) : 0ull;
-    };
+    auto weight = [&](float l) -> uint64_t { return kept(e_bits_of(sf(l * p.c), M)); };
     float4 l[N];
 #pragma unroll
     for (int j = 0; j < N; ++j) l[j] = load_logits4(lrow, min(g0 + (uint32_t)((j * kWaves + wave) * kWave + lane), V4 - 1u), p.dtype);
@@ -911,7 +912,8 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
         const u128 r_in = s.bc128[1];
         __syncthreads();
         if (p.diag) finish_row_slow<true>(p, s, t, row, xmax, p.inj_u ? 0ull : t.rand64, f.cnt_above + f.cnt_bin);
-        keep_pick<SLICE_LOG2>(p, s, t, row, M, g << SLICE_LOG2, r_in);
+        keep_pick<SLICE_LOG2>(p, s, t, row, M, g << SLICE_LOG2, r_in,
+                              [](uint32_t b) -> uint64_t { return b >= kEMinBits ? w_of_bits(b) : 0ull; });
         return true;
     }
 
@@ -1238,9 +1240,9 @@ __global__ void __launch_bounds__(kThreads, 2) stream_pen_kernel(const Params p,
 
 // pen <- fma(pen, decay, onehot * (pen == 0 ? presence : repetition)), the switch on the value before
 // the decay (reference: sampling.cu:427-437), for every row from its sampled token in p.out.
+template <int kPer>                                      // float4 groups per thread
 __global__ void __launch_bounds__(kThreads) penalty_pass_kernel(const Params p, uint32_t groups_per_row)
 {
-    constexpr int kPer = 8;                              // float4 groups per thread
     const uint32_t row = blockIdx.x / groups_per_row, part = blockIdx.x - row * groups_per_row;
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const uint32_t idx = (uint32_t)p.out[row];

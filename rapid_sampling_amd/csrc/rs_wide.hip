@@ -1,0 +1,25 @@
+// Instantiations and the launcher of the wide path.
+#include "rs_wide.h"
+
+namespace rs {
+
+hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v)
+{
+    const dim3 sgrid(B * v.G), sblock(kThreads);
+#define RS_WIDE_DT(Rv, Lv, DTv) do {                                                                    \
+        hipLaunchKernelGGL((stream_kernel<Rv, kThreads, DTv, true>), sgrid, sblock, 0, st, p, v);      \
+        hipLaunchKernelGGL((wide_kernel<Rv, DTv>), sgrid, sblock, 0, st, p, v);                        \
+        hipLaunchKernelGGL((wide_finish_kernel<Lv>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v); } while (0)
+#define RS_WIDE(Rv, Lv) do {                                                        \
+        if (dtype == RS_DTYPE_F32) RS_WIDE_DT(Rv, Lv, RS_DTYPE_F32);               \
+        else if (dtype == RS_DTYPE_BF16) RS_WIDE_DT(Rv, Lv, RS_DTYPE_BF16);        \
+        else RS_WIDE_DT(Rv, Lv, RS_DTYPE_F16); } while (0)
+    if (slice_r == 4) RS_WIDE(4, 12);
+    else if (slice_r == 8) RS_WIDE(8, 13);
+    else RS_WIDE(kStreamLongR, kStreamLongLog2);
+#undef RS_WIDE
+#undef RS_WIDE_DT
+    return hipGetLastError();
+}
+
+}  // namespace rs

@@ -386,7 +386,8 @@ void force_path(const std::string &name)
     else if (name == "stream") g_forced_path = RS_PATH_STREAM;
     else if (name == "attempt") g_forced_path = RS_PATH_ATTEMPT;
     else if (name == "fused") g_forced_path = RS_PATH_FUSED;
-    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused");
+    else if (name == "wide") g_forced_path = RS_PATH_WIDE;
+    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused | wide");
 }
 
 // The workspace tensor of the current stream (tests poison it to force the error path).

@@ -74,10 +74,11 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     # Every way through the library on this one workspace: the general kernel alone, the wait-free
     # streaming path (taken for top_k <= 1024; rows it cannot finish go on to the general kernel), the
     # same attempted whatever top_k is, the one-launch path (streaming pass and finish in one kernel,
-    # falling back inside the kernel), then the general kernel again on the workspace these leave
+    # falling back inside the kernel), the wide path (two passes over the logits and a finish, for kept
+    # sets of any size), then the general kernel again on the workspace these leave
     # behind.  All but the general kernel also return the e of every token: the kept set on that path.
     # With penalties: the one-launch path and the general kernel.
-    paths = ("cluster", "stream", "optimistic", "fused", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
+    paths = ("cluster", "stream", "optimistic", "fused", "wide", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
     for path in paths:
         pen3 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
         res3 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen3, presence=presence, repetition=repetition, decay=decay,
