@@ -264,10 +264,14 @@ namespace rs {
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
 enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5 };
-// The wide path (three launches, two reads of the logits) against the general kernel (one launch, its
-// exchanges): from this many tokens per call on the wide path is taken for kept sets the streaming
-// path cannot stash.
-constexpr uint64_t kWideMin = 1ull << 20;
+// The wide path (four launches, two reads of the logits) against the general kernel (one launch, its
+// exchanges), measured on flat rows (U[0,1), top_p 0.9) and on N(0,1.5) with top_k 10000: the wide path
+// wins from about 2^25 tokens per call on in rows of 50304 tokens and more (256 x 131072: 104 against
+// 108 us and 85 against 99; 128 x 262144: 102 against 119; 32 x 1048576: 106 against 133; 512 x 262144:
+// 280 against 395), loses below that (128 x 131072: 74 against 66) and in short rows (2048 x 32768:
+// 225 against 193).
+constexpr uint64_t kWideMin = 1ull << 25;
+constexpr int32_t kWideMinV = 49152;
 constexpr uint64_t kPenStreamMin = 1ull << 23;
 // Plain temperature sampling (top_k = V, top_p = 1: every live token is kept) has no kept set to
 // stash, but the streaming pass's bins alone say which slice holds the target: one pass at
@@ -339,7 +343,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (keep_all && V >= 32768) return kPathKeep;              // shorter rows: one workgroup of the general kernel does a row in one go
     // kept sets the stashes cannot hold: the wide path from kWideMin tokens on, unless its rows have been
     // going the slow way (slices that are no fair samples of their rows, ties of thousands of tokens)
-    auto wide_or_general = [&]() { return (uint64_t)B * (uint64_t)V >= kWideMin && !routed_away(2) ? kPathWide : kPathCluster; };
+    auto wide_or_general = [&]() { return (uint64_t)B * (uint64_t)V >= kWideMin && V >= kWideMinV && !routed_away(2) ? kPathWide : kPathCluster; };
     if (!bounded && !(top_p < 1.0f)) return wide_or_general(); // a top_k of thousands and no nucleus: more than the stashes hold
     if (!pol) return bounded ? kPathStream : wide_or_general();
     if (!routed_away(bounded ? 0 : 1)) return bounded ? kPathStream : kPathAttempt;

@@ -1,6 +1,10 @@
 // Instantiations and the launcher of the wide path.
 #include "rs_wide.h"
 
+#ifndef RS_WIDE_NT
+#define RS_WIDE_NT 512
+#endif
+
 namespace rs {
 
 hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v)
@@ -8,7 +12,8 @@ hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds
     const dim3 sgrid(B * v.G), sblock(kThreads);
 #define RS_WIDE_DT(Rv, Lv, DTv) do {                                                                    \
         hipLaunchKernelGGL((stream_kernel<Rv, kThreads, DTv, true>), sgrid, sblock, 0, st, p, v);      \
-        hipLaunchKernelGGL((wide_kernel<Rv, DTv>), sgrid, sblock, 0, st, p, v);                        \
+        hipLaunchKernelGGL(wide_plan_kernel, dim3(B), dim3(kThreads), 0, st, p, v);                    \
+        hipLaunchKernelGGL((wide_kernel<(Rv * 256 / RS_WIDE_NT), RS_WIDE_NT, DTv>), sgrid, dim3(RS_WIDE_NT), 0, st, p, v);                        \
         hipLaunchKernelGGL((wide_finish_kernel<Lv>), dim3(B), dim3(kThreads), finish_lds_bytes, st, p, v); } while (0)
 #define RS_WIDE(Rv, Lv) do {                                                        \
         if (dtype == RS_DTYPE_F32) RS_WIDE_DT(Rv, Lv, RS_DTYPE_F32);               \
