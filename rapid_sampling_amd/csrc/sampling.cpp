@@ -47,6 +47,7 @@ struct Entry {
     rs_policy *policy = nullptr;
     bool captured = false;                  // a stream capture has recorded calls that point into ws
     std::vector<at::Tensor> retired;        // outgrown workspaces a captured graph may still point into
+    std::vector<rs_policy *> retired_policies;   // replaced policies whose pinned words a captured graph's kernels may still write
 };
 
 bool is_capturing(void *stream)
@@ -333,7 +334,8 @@ int64_t workspace_status(std::optional<int64_t> device)
 }
 
 // Routing state of the current stream's workspace (rs_policy_state): bit 0 set: calls without a
-// bounding top_k currently take the general kernel, bit 1 set: so do calls with one.  -1: no workspace yet.
+// bounding top_k currently take the general kernel (or the wide path), bit 1 set: calls with one take the
+// general kernel, bit 2 set: calls that would take the wide path take the general kernel.  -1: no workspace yet.
 int64_t policy_state(std::optional<int64_t> device)
 {
     const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
@@ -360,7 +362,12 @@ void reset_routing(std::optional<int64_t> device)
     if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) throw std::runtime_error("rapid_sampling: stream synchronisation failed");
     rs_policy *fresh = nullptr;
     if (rs_policy_create(&fresh) != RS_OK) throw std::runtime_error("rapid_sampling: could not allocate the pinned host words of the workspace");
-    if (e.policy) rs_policy_destroy(e.policy);
+    // A captured graph holds the address of the old policy's pinned words (its kernels report into them on
+    // every replay): such a policy is kept, never freed, and simply no longer looked at.
+    if (e.policy) {
+        if (e.captured) e.retired_policies.push_back(e.policy);
+        else rs_policy_destroy(e.policy);
+    }
     e.policy = fresh;
     init_workspace(e, stream);
 }

@@ -299,6 +299,115 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
         assert np.array_equal(res["stream"]["out"][lo:lo + 32], ref_out), lo
 
 
+@pytest.mark.parametrize("B,T,V,top_k,top_p,gen", [(512, 1, 262144, -1, 0.9, "u1"), (128, 4, 1048576, 10000, 0.95, "n15"),
+                                                    (768, 1, 50304, 10000, 1.0, "u1")])
+def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
+    """Kept sets of thousands of tokens at scale (the reference's benchmark grid has top_k 10000 and top_p
+    0.9 on flat generators, /root/reference/bench.py:34-35, :66-72; its search costs the same whatever the
+    kept set, sampling.cu:261-329): 512 flat rows of 262144 tokens under top_p 0.9, the bandwidth
+    configuration's 128 rows of a million tokens with top_k 10000, 768 flat rows of 50304 tokens.  The
+    library takes the wide path for them by itself (diag.rounds == 7 for every row: none done the slow
+    way); every row goes through the oracle, and the general kernel must agree in every field."""
+    torch = torch_cuda
+    from tests import capi
+    g = torch.Generator(device="cuda")
+    g.manual_seed(50 + B)
+    shape = (B, T, V) if T > 1 else (B, V)
+    lg = torch.rand(shape, generator=g, device="cuda") if gen == "u1" else torch.randn(shape, generator=g, device="cuda") * 1.5
+    rc, c, k, p = capi.normalize(1.0, top_k, top_p, V, B, T)
+    u_np = H.uniforms(B, 321)
+    u = torch.from_numpy(u_np).cuda()
+    smp = capi.Sampler(B, V)
+    res = {}
+    for path in ("auto", "cluster", "wide"):
+        print("wide at scale", B, T, V, path, flush=True)
+        r = smp.sample(lg, c, k, p, uniforms=u, path=path)
+        assert r["rc"] == 0 and smp.status() == 0
+        res[path] = r
+    assert (res["auto"]["diag"]["rounds"] == 7).all(), np.unique(res["auto"]["diag"]["rounds"], return_counts=True)
+    assert (res["wide"]["diag"]["rounds"] == 7).all()
+    assert (res["cluster"]["diag"]["rounds"] < 7).all()
+    for f in FIELDS:
+        assert np.array_equal(res["auto"]["diag"][f], res["cluster"]["diag"][f]), f
+        assert np.array_equal(res["auto"]["diag"][f], res["wide"]["diag"][f]), f
+    assert np.array_equal(res["auto"]["out"], res["cluster"]["out"])
+    d = res["auto"]["diag"]
+    step = 64 if V <= 262144 else 32
+    for lo in range(0, B, step):
+        sub = (lg[lo:lo + step, T - 1, :] if T > 1 else lg[lo:lo + step]).cpu().numpy()
+        ref_out, ref_diag = oracle.sample_batch(sub, c, k, p, injected_u=u_np[lo:lo + step])
+        for f in FIELDS:
+            assert np.array_equal(d[f][lo:lo + step], ref_diag[f]), (f, lo)
+        assert np.array_equal(res["auto"]["out"][lo:lo + step], ref_out), lo
+
+
+def test_wide_path_unusual_rows(torch_cuda, oracle):
+    """Rows the wide path's second pass cannot serve the usual way, each against the oracle on every path:
+    a boundary bin that holds more than a quarter of a slice (flat rows at a temperature of 2: the waves'
+    queues overflow and the slice is gone through again from memory); sorted rows, whose slices are no
+    samples of the row at all, so that no slice's window covers the row's threshold (done the slow way,
+    diag.rounds == 8); rows of a few distinct values (ties of thousands of tokens in one sub-bin); rows
+    with masked stretches that put whole slices far below the row's frame; a tie of all tokens."""
+    torch = torch_cuda
+    from tests import capi
+    V = 131072 + 8192
+    rng = np.random.default_rng(123)
+    lg = rng.random((8, V), dtype=np.float32)
+    lg[1] = np.sort(lg[1])[::-1]                                      # descending: slice 0 holds the whole kept set
+    lg[2] = np.sort(lg[2])                                            # ascending
+    lg[3] = np.round(lg[3] * 16) / 16                                 # 17 distinct values
+    lg[4, 16384:81920] = -np.inf                                      # four slices fully masked
+    lg[5] = 0.5                                                       # one tie of all tokens
+    lg[6] = (rng.standard_normal(V) * 1.5).astype(np.float32)
+    lg[7, ::3] += 0.5                                                 # two populations
+    for (temp, k, p) in [(2.0, -1, 0.9), (1.0, 10000, 1.0), (1.0, -1, 0.5), (0.7, 3000, 0.8)]:
+        _run_case(torch, oracle, capi, lg, temp, k, p, u_np=H.uniforms(8, 61), what="wide unusual T=%g k=%d p=%g" % (temp, k, p))
+    rc, c, k, p = capi.normalize(1.0, -1, 0.5, V, 8, 1)
+    res = capi.Sampler(8, V).sample(torch.from_numpy(lg).cuda(), c, k, p, path="wide", uniforms=torch.from_numpy(H.uniforms(8, 61)).cuda())
+    rounds = res["diag"]["rounds"]
+    assert rounds[0] == 7 and rounds[4] == 7 and rounds[6] == 7 and rounds[7] == 7, rounds
+    assert rounds[1] == 8 and rounds[2] == 8, rounds                # sorted rows: the slow way
+    assert rounds[5] == 0, rounds                                   # one tie of all tokens: finished from the row's bins
+
+
+def test_wide_path_reports_slow_rows(torch_cuda, oracle):
+    """Calls on the wide path that are given a policy report rows done the slow way in a word of their own
+    (rs_policy_state bit 2): the next calls of that kind take the general kernel, the wide path is tried
+    again after 64 of them, and a call that goes well clears the word through the call after it."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 300, 131072
+    good = H.logits_uniform(B, V, seed=71)
+    bad = good.copy()
+    bad[11] = np.sort(bad[11])
+    # top_k 20000 of a sorted row: the boundary bin's tokens lie in two slices, the upper part in one and the
+    # lower part in the other, so neither slice's share says where in the bin the row's threshold is
+    rc, c, k, p = capi.normalize(1.0, 20000, 1.0, V, B, 1)
+    u_np = H.uniforms(B, 72)
+    u = torch.from_numpy(u_np).cuda()
+    ref_good = oracle.sample_batch(good, c, k, p, injected_u=u_np)
+    ref_bad = oracle.sample_batch(bad, c, k, p, injected_u=u_np)
+    lg_good, lg_bad = torch.from_numpy(good).cuda(), torch.from_numpy(bad).cuda()
+    smp = capi.Sampler(B, V, with_policy=True, init=True)
+    res = smp.sample(lg_good, c, k, p, uniforms=u)
+    _check(res, *ref_good, "wide, fair rows")
+    assert (res["diag"]["rounds"] == 7).all() and smp.policy_state() == 0
+    res = smp.sample(lg_bad, c, k, p, uniforms=u)
+    _check(res, *ref_bad, "wide, one sorted row")
+    assert res["diag"]["rounds"][11] == 8 and (np.delete(res["diag"]["rounds"], 11) == 7).all() and smp.policy_state() == 4
+    for i in range(3):
+        res = smp.sample(lg_good, c, k, p, uniforms=u)
+        _check(res, *ref_good, "after a slow row %d" % i)
+        assert (res["diag"]["rounds"] < 7).all() and smp.policy_state() == 4       # general kernel
+    for i in range(64):
+        res = smp.sample(lg_good, c, k, p, uniforms=u, want_diag=False)
+        assert res["rc"] == 0 and np.array_equal(res["out"], ref_good[0])
+    assert smp.policy_state() == 0
+    res = smp.sample(lg_good, c, k, p, uniforms=u)
+    assert (res["diag"]["rounds"] == 7).all() and smp.policy_state() == 0 and smp.status() == 0
+    smp.close()
+
+
 def test_streaming_path_flat_distributions(torch_cuda, oracle):
     """Flat rows with a small top_k: the bin in which the count reaches top_k holds thousands of tokens, so
     a slice refines its cut inside that bin and the finish works on the whole stashes (the reference's
