@@ -203,15 +203,17 @@ static int stream_r(int32_t B, int32_t V, bool pen = false)
     return kStreamLongR;
 }
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-struct StreamLayout { size_t hdr, cum, shist, stash, end; };
-static StreamLayout stream_layout(size_t parts, size_t base)
+struct StreamLayout { size_t hdr, cum, shist, stash, pens, end; };
+// `with_pens`: room for every slice's note of its non-zero penalties behind the stashes (long slices only)
+static StreamLayout stream_layout(size_t parts, size_t base, bool with_pens = false)
 {
     StreamLayout l;
     l.hdr = align256(base);
     l.cum = align256(l.hdr + parts * sizeof(PartHdr));
     l.shist = align256(l.cum + parts * kSB * sizeof(uint32_t));
     l.stash = align256(l.shist + parts * kSB * sizeof(uint64_t));
-    l.end = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
+    l.pens = align256(l.stash + parts * kStashCap * sizeof(uint64_t));
+    l.end = with_pens ? align256(l.pens + parts * kPenCap * sizeof(uint64_t)) : l.pens;
     return l;
 }
 // Bytes of per-slice data a workspace for (B, V) sets aside: enough for the long slices of (B, V)
@@ -221,7 +223,7 @@ static StreamLayout stream_layout(size_t parts, size_t base)
 // with B and with V and a workspace for the largest B and V serves every smaller call.
 static size_t stream_bytes(int32_t B, int32_t V)
 {
-    const size_t longs = stream_layout((size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader)).end;
+    const size_t longs = stream_layout((size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader), true).end;
     size_t small_parts = (size_t)B * stream_parts(V, 4);
     const size_t cap = (size_t)kStreamSmallParts + (size_t)B;
     static_assert(kStreamSmallParts >= kFusedSmall / 4096, "room for either kind of small call");
@@ -595,10 +597,12 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V, pen);
         StreamView v;
         v.G = stream_parts(V, sr);
-        const StreamLayout l = stream_layout((size_t)B * v.G, sizeof(WsHeader));
+        const bool pen_stream = pen && path == kPathStream;                  // long slices: their layout has room for the notes
+        const StreamLayout l = stream_layout((size_t)B * v.G, sizeof(WsHeader), pen_stream);
         char *w = (char *)workspace;
         v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.shist = (uint64_t *)(w + l.shist);
+        v.pens = pen_stream ? (uint64_t *)(w + l.pens) : nullptr;
         // without a bounding top_k the stashes are sized as for top_k = kStreamK: enough for a nucleus
         // of up to about a thousand tokens
         const uint32_t kk = min((uint32_t)top_k, (uint32_t)kStreamK);
@@ -631,11 +635,12 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         if (path == kPathFused)
             return launch_fused(sr, pen, (uint32_t)B, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         if (pen) {
-            // penalties: read by the streaming pass (and by the finishing workgroup of a row it has to
-            // do the slow way), rewritten by one pass over them at the end
-            p.defer_pen = 1;
+            // penalties: read and rewritten (decayed) by the streaming pass, the sampled token's patched by the
+            // finishing workgroup; slices the pass deferred are rewritten by a fix-up kernel at the end
+            // a finite decay keeps +0.0 at +0.0, which is what lets the pass skip the groups that hold nothing
+            p.defer_pen = (decay - decay == 0.0f) ? 2 : 1;
             if (launch_stream_pen((uint32_t)B, dyn, st, p, v) != hipSuccess) return RS_ERR_LAUNCH;
-            return launch_penalty_pass(st, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+            return launch_penalty_fix(st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         }
         return launch_stream(sr, logits_dtype, path == kPathKeep, (uint32_t)B, dyn, st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
     }

@@ -84,7 +84,9 @@ struct Params {
     int32_t      dtype;        // RS_DTYPE_* of the logits
     uint32_t     report;       // which report word of the caller's policy a streaming call writes: 0 top_k bounds the kept set, 1 not, 3 the wide path
     int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1], [3] routing reports, [2] error; or null
-    int32_t      defer_pen;    // penalties enter x but are left as they are: a later pass over them applies decay and one-hot add
+    int32_t      defer_pen;    // penalties enter x and are not rewritten from the registers at the end: 1 a later pass over them
+                               // applies decay and one-hot add; 2 the streaming pass writes the decayed values itself and notes
+                               // the old non-zero ones, the finish patches the sampled token (see stream_pen_kernel)
     int64_t      row_stride;
     int32_t      B, V;
     uint32_t     G;            // workgroups per row
@@ -650,8 +652,16 @@ struct PartHdr {
                           // bin cov or, when only part of a bin fitted, in bin cov - 1
 };
 
+// A slice's note of its penalties (stream_pen_kernel): word 0 = count, or kPenDeferred when the slice left its
+// penalties untouched; then count entries (old value's bits << 32 | token index in the row), the penalties
+// whose bit pattern was not +0.0 before the call.
+constexpr int      kPenCap      = 512;        // words per slice: 511 non-zero penalties among 16384 tokens, 3.1 %
+constexpr int      kPenWave     = 160;        // of which one wave (4096 tokens) can note this many
+constexpr uint64_t kPenDeferred = 1ull << 63;
+
 struct StreamView {
     PartHdr  *hdr;        // [B][G]
+    uint64_t *pens;       // [B][G][kPenCap]   penalties at scale only, else null
     uint64_t *stash;      // [B][G][kStashCap]   bits(e, slice frame) << 32 | index, by descending bin
     uint32_t *cum;        // [B][G][kSB]   tokens of the slice in this bin and the bins above it
     uint64_t *shist;      // [B][G][kSB]   the slice's own bins (slice frame), as it added them to the row's
@@ -663,7 +673,7 @@ struct StreamView {
 // Launchers, one per translation unit that instantiates the kernels.
 hipError_t launch_sample(bool pen, int R, dim3 grid, hipStream_t st, const Params &p);
 hipError_t launch_stream_pen(uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
-hipError_t launch_penalty_pass(hipStream_t st, const Params &p);
+hipError_t launch_penalty_fix(hipStream_t st, const Params &p, const StreamView &v);
 hipError_t launch_stream(int slice_r, int32_t dtype, bool keep, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
                          const StreamView &v);
 hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v);

@@ -717,6 +717,51 @@ __device__ __forceinline__ void keep_pick(const Params &p, Lds &s, LdsB &t, cons
     }
 }
 
+// Penalties at scale (stream_pen_kernel): the pass has already written every slice's decayed penalties and
+// noted the old values that were not +0.0.  A row that has to be done the slow way needs the old values
+// of all its tokens: the notes are played back, and every slice of the row is marked deferred, so that
+// the fix-up kernel rewrites the whole row once its token is known.
+__device__ __forceinline__ void pen_restore(const Params &p, const StreamView &v, const uint32_t row)
+{
+    const int tid = threadIdx.x;
+    float *pen = p.penalties + (int64_t)row * p.V;
+    for (uint32_t g = 0; g < v.G; ++g) {
+        uint64_t *rec = v.pens + ((size_t)row * v.G + g) * kPenCap;
+        const uint64_t h = rec[0];
+        if (!(h & kPenDeferred))
+            for (uint32_t i = (uint32_t)tid; i < (uint32_t)h; i += kThreads) {
+                const uint64_t e = rec[1 + i];
+                pen[(uint32_t)e] = __uint_as_float((uint32_t)(e >> 32));
+            }
+    }
+    __syncthreads();
+    if ((uint32_t)tid < v.G) v.pens[((size_t)row * v.G + tid) * kPenCap] = kPenDeferred;
+    wait_vmem();
+    __syncthreads();
+}
+
+// The sampled token's penalty: fma(old, decay, old == 0 ? presence : repetition) (reference:
+// sampling.cu:427-437), the old value from the slice's notes (+0.0 when it is not among them).  A deferred
+// slice still holds its old penalties and is rewritten whole by the fix-up kernel.
+__device__ __forceinline__ void pen_patch(const Params &p, const StreamView &v, Lds &s, const uint32_t row, const uint32_t idx, const uint32_t slice_log2)
+{
+    const int tid = threadIdx.x;
+    const uint64_t *rec = v.pens + ((size_t)row * v.G + (idx >> slice_log2)) * kPenCap;
+    const uint64_t h = rec[0];
+    if (h & kPenDeferred) return;
+    if (tid == 0) s.bc32[6] = 0u;
+    __syncthreads();
+    for (uint32_t i = (uint32_t)tid; i < (uint32_t)h; i += kThreads) {
+        const uint64_t e = rec[1 + i];
+        if ((uint32_t)e == idx) s.bc32[6] = (uint32_t)(e >> 32);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const float old = __uint_as_float(s.bc32[6]);
+        p.penalties[(int64_t)row * p.V + idx] = __builtin_fmaf(old, p.decay, old == 0.0f ? p.presence : p.repetition);
+    }
+}
+
 // Finishes a row from what its slices published.  Returns true when the row is done (token written),
 // false when it cannot be finished from the stashes: only on the one-launch path (FUSED = true: the
 // caller is the last workgroup of the row to publish, the data was written by workgroups of this same
@@ -847,6 +892,7 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
             rng_st[2] = rs[2] + 1u;
             if (rs[2] + 1u == 0u) rng_st[3] = rs[3] + 1u;
         }
+        if (!FUSED && p.penalties && p.defer_pen == 2) pen_restore(p, v, row);
         finish_row_slow(p, s, t, row, xmax, p.inj_u ? 0ull : t.rand64);
         tell_policy();
         return true;
@@ -1211,20 +1257,33 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const Params p, const 
     extern __shared__ __align__(16) unsigned char finish_dyn[];
     t.list = reinterpret_cast<uint64_t *>(finish_dyn);       // every thread writes the same value (KEEP: no list, not used)
     finish_row<SLICE_LOG2, false, KEEP>(p, v, s, t, blockIdx.x);
+    if (!KEEP && p.penalties && p.defer_pen == 2) {
+        __syncthreads();
+        pen_patch(p, v, s, blockIdx.x, t.result - 1u, SLICE_LOG2);
+    }
 }
 
 
 
 // The streaming pass for calls with penalties too large for the one-launch path: logits and penalties
 // are read once, x = sf((sf(l) - pen) * c) as in the cluster kernel, everything after that is the
-// streaming pass.  The penalties are not rewritten here (the sampled token is not known yet):
-// penalty_pass_kernel does that once every row has its token -- 16 bytes per token in all instead
-// of the 12 a single pass would move, at several times the cluster kernel's rate.
+// streaming pass.  The sampled token is not known yet, but every OTHER token's new penalty is
+// fma(pen, decay, 0), so the pass writes those from its registers -- 12 bytes per token in all, as the
+// reference's single kernel moves (sampling.cu:211,220,427-437) -- and the finishing workgroup patches the
+// one sampled token.  That needs the sampled token's old value, and a row the finishing workgroup has to do
+// the slow way needs the old values of all its tokens; penalties are non-zero only where tokens have been
+// generated, so each slice notes the old values whose bit pattern is not +0.0 (up to kPenCap - 1 of them; a
+// slice with more leaves its penalties untouched and says so, and penalty_fix_kernel rewrites such slices
+// once the tokens are known).  Groups of four that are all +0.0 stay +0.0 under a finite decay and are
+// not written at all.
 template <int R>
 __global__ void __launch_bounds__(kThreads, 2) stream_pen_kernel(const Params p, const StreamView v)
 {
     constexpr int kRep = stream_copies<R>();
     __shared__ LdsA<kRep> s;
+    __shared__ uint64_t noted[kWaves][kPenWave];
+    __shared__ uint32_t nnote[kWaves];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t G = v.G;
     const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
     const bool reporter = blockIdx.x == 0 && threadIdx.x == 0;
@@ -1235,27 +1294,77 @@ __global__ void __launch_bounds__(kThreads, 2) stream_pen_kernel(const Params p,
     slice_setup(p, sl, row, part, G);
     const float lmax = slice_load(p, sl);
     if (reporter) report_end(p, prev, true);
+    if (p.defer_pen == 2) {
+        // the penalties whose bit pattern is not +0.0, side by side into this wave's notes
+        uint32_t fill = 0;                               // wave-uniform: every lane takes part in every vote
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint32_t b4[4] = {__float_as_uint(sl.pen[j].x), __float_as_uint(sl.pen[j].y), __float_as_uint(sl.pen[j].z), __float_as_uint(sl.pen[j].w)};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bool nz = j < sl.nv && b4[q] != 0u;
+                const uint64_t vote = __ballot(nz);
+                if (nz) {
+                    const uint32_t pos = fill + __builtin_amdgcn_mbcnt_hi((uint32_t)(vote >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)vote, 0u));
+                    if (pos < (uint32_t)kPenWave) noted[wave][pos] = ((uint64_t)b4[q] << 32) | ((sl.base4 + (uint32_t)j * kThreads) * 4u + (uint32_t)q);
+                }
+                fill += (uint32_t)__popcll(vote);
+            }
+        }
+        if (lane == 0) nnote[wave] = fill;
+        __syncthreads();
+        uint32_t total = 0, before = 0;
+        bool fits = true;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const uint32_t n = nnote[w];
+            if (w < wave) before += n;
+            total += n;
+            fits = fits && n <= (uint32_t)kPenWave;
+        }
+        fits = fits && total < (uint32_t)kPenCap;
+        uint64_t *rec = v.pens + ((size_t)row * G + part) * kPenCap;
+        if (fits) {
+            for (uint32_t i = (uint32_t)lane; i < fill; i += kWave) rec[1 + before + i] = noted[wave][i];
+            if (tid == 0) rec[0] = total;
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                float4 q = sl.pen[j];
+                if (j < sl.nv && (__float_as_uint(q.x) | __float_as_uint(q.y) | __float_as_uint(q.z) | __float_as_uint(q.w)) != 0u) {
+                    q.x = __builtin_fmaf(q.x, p.decay, 0.0f); q.y = __builtin_fmaf(q.y, p.decay, 0.0f);
+                    q.z = __builtin_fmaf(q.z, p.decay, 0.0f); q.w = __builtin_fmaf(q.w, p.decay, 0.0f);
+                    sl.pn4[sl.base4 + (uint32_t)j * kThreads] = q;
+                }
+            }
+        } else if (tid == 0) rec[0] = kPenDeferred;
+    }
     slice_count_and_stash<R, kThreads, kRep, false>(p, v, s, sl.eb, lmax, row, part, sl.base4, sl.nv);
 }
 
 // pen <- fma(pen, decay, onehot * (pen == 0 ? presence : repetition)), the switch on the value before
-// the decay (reference: sampling.cu:427-437), for every row from its sampled token in p.out.
-template <int kPer>                                      // float4 groups per thread
-__global__ void __launch_bounds__(kThreads) penalty_pass_kernel(const Params p, uint32_t groups_per_row)
+// the decay (reference: sampling.cu:427-437), from the sampled token in p.out, for the slices that still
+// hold their old penalties: all of them when the streaming pass left the penalties alone (defer_pen 1),
+// else those marked deferred -- by the pass (too many non-zero penalties to note) or by the finishing
+// workgroup of a row done the slow way (which played the notes back).  One workgroup per slice; the others
+// leave after one load.
+template <int R>
+__global__ void __launch_bounds__(kThreads) penalty_fix_kernel(const Params p, const StreamView v)
 {
-    const uint32_t row = blockIdx.x / groups_per_row, part = blockIdx.x - row * groups_per_row;
+    const uint32_t G = v.G;
+    const uint32_t row = blockIdx.x / G, part = blockIdx.x - row * G;
+    if (p.defer_pen == 2 && !(v.pens[((size_t)row * G + part) * kPenCap] & kPenDeferred)) return;
     const uint32_t V4 = (uint32_t)p.V >> 2;
     const uint32_t idx = (uint32_t)p.out[row];
     float4 *pn4 = reinterpret_cast<float4 *>(p.penalties + (int64_t)row * p.V);
-    const uint32_t base4 = part * (uint32_t)(kThreads * kPer) + threadIdx.x;
-    float4 q[kPer];
+    const uint32_t base4 = part * (uint32_t)(kThreads * R) + threadIdx.x;
+    float4 q[R];
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) {
+    for (int j = 0; j < R; ++j) {
         const uint32_t i4 = base4 + (uint32_t)j * kThreads;
         if (i4 < V4) q[j] = pn4[i4];
     }
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) {
+    for (int j = 0; j < R; ++j) {
         const uint32_t i4 = base4 + (uint32_t)j * kThreads;
         if (i4 < V4) {
             float4 w = q[j];

@@ -29,10 +29,9 @@ hipError_t launch_stream_pen(uint32_t B, size_t finish_lds_bytes, hipStream_t st
     return hipGetLastError();
 }
 
-hipError_t launch_penalty_pass(hipStream_t st, const Params &p)
+hipError_t launch_penalty_fix(hipStream_t st, const Params &p, const StreamView &v)
 {
-    const uint32_t V4 = (uint32_t)p.V / 4, groups = (V4 + kThreads * 8 - 1) / (kThreads * 8);
-    hipLaunchKernelGGL((penalty_pass_kernel<8>), dim3((uint32_t)p.B * groups), dim3(kThreads), 0, st, p, groups);
+    hipLaunchKernelGGL((penalty_fix_kernel<kStreamLongR>), dim3((uint32_t)p.B * v.G), dim3(kThreads), 0, st, p, v);
     return hipGetLastError();
 }
 

@@ -867,8 +867,8 @@ def test_one_launch_path_rows_of_more_slices_than_an_xcd_has_compute_units(torch
 @pytest.mark.parametrize("B,V,steps", [(96, 152064, 3), (128, 1048576, 2)])
 def test_penalties_at_scale_streaming_pass(torch_cuda, oracle, B, V, steps):
     """Calls with penalties too large for the one-launch path (more workgroups than the GPU holds at once)
-    take the streaming pass over logits and penalties, the finish, and one pass over the penalties that
-    applies decay and the one-hot add: chained steps, tokens, diagnostics and penalties bit for bit
+    take the streaming pass over logits and penalties, which also writes the decayed penalties, and the
+    finish, which patches the sampled tokens: chained steps, tokens, diagnostics and penalties bit for bit
     against the oracle; the general kernel on the same inputs beside it."""
     torch = torch_cuda
     from tests import capi
@@ -893,6 +893,55 @@ def test_penalties_at_scale_streaming_pass(torch_cuda, oracle, B, V, steps):
         _check(res_c, ref_out, ref_diag, "general kernel, step %d" % step)
         assert torch.equal(pen_c.view(torch.int32), pen.view(torch.int32))
         assert smp.status() == 0
+
+
+def test_penalties_at_scale_unusual_rows_and_slices(torch_cuda, oracle):
+    """The single pass over the penalties at scale where it cannot simply write decayed values and patch
+    one token (reference: sampling.cu:427-437 on every kind of row): a row that has to be done the slow way
+    (half its tokens tie at the top, so the old penalties of the whole row are needed again: the slices'
+    notes are played back and the row rewritten at the end), a row of a million tokens among them, slices
+    with more non-zero penalties than they can note (left alone by the pass, rewritten at the end),
+    penalties of -0.0 (not +0.0: written, and 'zero' for the presence / repetition switch), a sampled token
+    whose old penalty was non-zero, and a decay that is not finite (nothing can be skipped).  Three chained
+    steps each, everything bit for bit against the oracle."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 10, 1048576
+    rng = np.random.default_rng(150)
+    lg_np = (rng.standard_normal((B, V)) * 1.5).astype(np.float32)
+    pen0 = H.penalties_sparse(B, V, seed=151)
+    lg_np[1, ::2] = 9.0                                               # a tie of half the row at the top: the slow way
+    pen0[1, ::2] = 0.0
+    pen0[1, 4::64] = 0.25                                             # ... some of the tied tokens penalised
+    pen0[2, 100000:140000] = rng.exponential(1.0, 40000).astype(np.float32)      # dense stretch: slices that cannot note all
+    pen0[3, ::7] = -0.0
+    top = np.argsort(lg_np[4])[-3:]
+    lg_np[4, top] += 6.0                                              # three dominant tokens, already penalised
+    pen0[4, top] = 0.5
+    pen0[5] = 0.0                                                     # nothing penalised yet
+    pen0[6] = rng.exponential(0.1, V).astype(np.float32)              # everything penalised
+    rc, c, k, p = capi.normalize(0.8, 50, 0.9, V, B, 1)
+    lg = torch.from_numpy(lg_np).cuda()
+    for decay in (0.95, float("inf")):
+        pen_ref = pen0.copy()
+        if decay != 0.95:
+            pen_ref[:] = 0.0                                          # 0 * inf: every entry becomes NaN, zeros too
+        smp = capi.Sampler(B, V)
+        pen = torch.from_numpy(pen_ref.copy()).cuda()
+        for step in range(3):
+            u_np = H.uniforms(B, 600 + step)
+            u = torch.from_numpy(u_np).cuda()
+            ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, injected_u=u_np, penalties=pen_ref,
+                                                    presence=0.1, repetition=0.2, decay=decay)
+            print("penalties at scale, unusual: decay", decay, "step", step, flush=True)
+            res = smp.sample(lg, c, k, p, uniforms=u, penalties=pen, presence=0.1, repetition=0.2, decay=decay)
+            _check(res, ref_out, ref_diag, "unusual penalties, decay %r step %d" % (decay, step))
+            got = pen.cpu().numpy().view(np.uint32)
+            bad = np.nonzero((got != pen_ref.view(np.uint32)).any(axis=1))[0]
+            assert bad.size == 0, (decay, step, bad)
+            if decay == 0.95 and step == 0:
+                assert res["diag"]["rounds"][1] == 8 and (np.delete(res["diag"]["rounds"], 1) == 0).all(), res["diag"]["rounds"]
+            assert smp.status() == 0
 
 
 def test_philox_stream_matches_oracle(torch_cuda, oracle):
