@@ -220,6 +220,7 @@ def main():
                                "Philox draws, drop-in Python call"},
         "latency": {
             "p50_us": round(p50, 3), "p10_us": round(pct(us, 0.10), 3), "p90_us": round(pct(us, 0.90), 3),
+            "p99_us": round(pct(us, 0.99), 3), "max_us": round(max(us), 3),
             "back_to_back_us": round(b2b_us, 3),
             "floor_p50_us": round(floor_p50, 3), "floor_back_to_back_us": round(floor_b2b_us, 3),
             "ratio_to_floor": round(p50 / floor_p50, 3),
@@ -229,7 +230,8 @@ def main():
             "reference_note": "reference README.md:21-31: same B, V, top_p, top_k, logits U[0,1)*4, unnamed NVIDIA GPU",
             "readme_point": {
                 "workload": "B=1, V=262144, logits U[0,1)*4 seed 4, temperature 1.0, top_k -1, top_p 0.3 (README.md:21-31)",
-                "p50_us": round(readme_p50, 3), "ratio_to_floor": round(readme_p50 / floor_p50, 3),
+                "p50_us": round(readme_p50, 3), "p99_us": round(pct(readme_us, 0.99), 3), "max_us": round(max(readme_us), 3),
+                "ratio_to_floor": round(readme_p50 / floor_p50, 3),
                 "call_plus_sync_p50_us": round(statistics.median(readme_sync), 2),
                 "path": "general kernel (the flat row's nucleus is too large for the streaming path; routed by its reports)"
                         if readme_state & 1 else "streaming path",
@@ -263,8 +265,12 @@ def main():
         # read-only kernels on the same rows: plain / non-temporal loads on the general kernel's grid
         # and on the streaming pass's grid
         floor_names = ["plain loads, 128 KiB per workgroup", "non-temporal loads, 128 KiB per workgroup",
-                       "plain loads, 64 KiB per workgroup", "non-temporal loads, 64 KiB per workgroup"]
-        t_floors = [block_time_us(torch, floor_variant(n), args.bandwidth_steps, 3) for n in range(4)]
+                       "plain loads, 64 KiB per workgroup", "non-temporal loads, 64 KiB per workgroup",
+                       "persistent grid of 2048 workgroups, 4 loads in flight", "the same, an eighth of the data per XCD",
+                       "256 KiB contiguous per workgroup, 16 loads in flight",
+                       "persistent grid of 1024 workgroups per XCD, 8 loads in flight",
+                       "persistent grid of 4096 workgroups, 2 loads in flight"]
+        t_floors = [block_time_us(torch, floor_variant(n), args.bandwidth_steps, 3) for n in range(len(floor_names))]
         t_floor = min(t_floors)
         sample._sample.force_path("cluster")             # the general single-launch kernel on the same input
         try:
@@ -329,7 +335,8 @@ def main():
             "us_per_call": round(t_pen, 2), "achieved": round(Bb * Vb * 12 / (t_pen * 1e-6) / 1e9, 1),
             "frac": round(Bb * Vb * 12 / (t_pen * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
             "note": "(128,1048576) fp32 rows (stride T*V) with a (128,1048576) penalties tensor, 2 % non-zero: "
-                    "rs::stream_pen_kernel, rs::finish_kernel, rs::penalty_pass_kernel; algorithmic bytes 12*V per row"}
+                    "rs::stream_pen_kernel (reads both, writes the decayed penalties), rs::finish_kernel (patches the sampled "
+                    "tokens), rs::penalty_fix_kernel (slices the pass deferred: none here); algorithmic bytes 12*V per row"}
         del pen_b, last
         if args.traffic_probe:
             src = big.view(-1)[: Bb * Vb]

@@ -348,8 +348,14 @@ int rs_static_status(int32_t *status, uint32_t where[4], int32_t clear, void *st
  * every thread issuing all its loads before it uses the first.  variant 0: the
  * general kernel's grid for (B,V), plain loads; 1: the same with loads marked
  * non-temporal (as the sampling kernels read the logits); 2, 3: the same two
- * on the streaming pass's grid.  Measurement aid for the B=1 latency bound and
- * for the read bandwidth the hardware delivers; no counterpart in the reference.
+ * on the streaming pass's grid; 4 to 8: other shapes of a read-only kernel,
+ * all non-temporal, which max-combine into out_device[0] only -- 4 a
+ * persistent grid of 2048 workgroups that sweeps the rows front to back with
+ * four loads per thread in flight, 5 the same with an eighth of the data per
+ * XCD, 6 contiguous 256 KiB per workgroup, 7 a persistent grid of 1024
+ * workgroups per XCD with eight loads in flight, 8 one of 4096 workgroups with
+ * two.  Measurement aid for the B=1 latency bound and for the read bandwidth
+ * the hardware delivers; no counterpart in the reference.
  */
 int rs_floor_read(const float *logits_device, int64_t row_stride, int32_t *out_device,
                   int32_t B, int32_t V, int32_t variant, void *stream);

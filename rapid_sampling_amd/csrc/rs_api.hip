@@ -89,6 +89,44 @@ __global__ void __launch_bounds__(kThreads) floor_kernel(const float *logits, in
     if (threadIdx.x == 0) atomicMax(reinterpret_cast<uint32_t *>(out + row), max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
 }
 
+// Read-only kernels of other shapes, for the read bandwidth the device delivers: a workgroup goes through
+// `per` pieces of kThreads * U float4 (U loads per thread in flight), either pieces that lie one after the
+// other (a long contiguous stretch per workgroup), or grid-strided ones (a persistent grid that sweeps
+// the rows front to back); XCD: workgroup b runs on XCD b mod 8, and the eight XCDs are given an eighth
+// of the data each, so that what one XCD's L2 sees is one contiguous stretch.
+template <int U, bool STRIDED, bool XCD>
+__global__ void __launch_bounds__(kThreads) floor_sweep_kernel(const float *logits, int64_t row_stride, int32_t *out, int32_t V,
+                                                               uint32_t pieces_per_row, uint32_t pieces, uint32_t per)
+{
+    const uint32_t V4 = (uint32_t)V >> 2;
+    uint32_t wg = blockIdx.x, nwg = gridDim.x;
+    uint32_t first = 0, span = pieces;                   // the stretch of pieces this workgroup's group of workgroups shares
+    if (XCD) {
+        const uint32_t x = blockIdx.x & 7u, share = (pieces + 7u) >> 3;
+        first = x * share; span = min(share, pieces > first ? pieces - first : 0u);
+        wg = blockIdx.x >> 3; nwg = (gridDim.x + 7u - x) >> 3;
+    }
+    float m = -3.402823466e+38f;
+    for (uint32_t i = 0; i < per; ++i) {
+        const uint32_t local = STRIDED ? wg + i * nwg : wg * per + i;
+        if (local >= span) break;
+        const uint32_t piece = first + local;
+        const uint32_t row = piece / pieces_per_row, off4 = (piece - row * pieces_per_row) * (uint32_t)(kThreads * U) + threadIdx.x;
+        const uint4 *lg = reinterpret_cast<const uint4 *>(logits + (int64_t)row * row_stride);
+        uint4 v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) v[j] = load_once(lg + min(off4 + (uint32_t)(j * kThreads), V4 - 1));
+#pragma unroll
+        for (int j = 0; j < U; ++j)
+            m = fmaxf(m, fmaxf(fmaxf(__uint_as_float(v[j].x), __uint_as_float(v[j].y)), fmaxf(__uint_as_float(v[j].z), __uint_as_float(v[j].w))));
+    }
+    __shared__ uint32_t wmax[kWaves];
+    const uint32_t k = wave_max_u32(fkey(m));
+    if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = k;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(reinterpret_cast<uint32_t *>(out), max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+}
+
 __global__ void philox_init_kernel(uint32_t *state, uint64_t seed, int32_t B)
 {
     const int b = blockIdx.x * blockDim.x + threadIdx.x;
@@ -243,6 +281,7 @@ constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u;
 struct rs_policy {
     int32_t *word;
     uint32_t away[3], period[3], good[3];                // kinds: 0 streaming with a bounding top_k, 1 without, 2 the wide path
+    uint32_t probed;                                     // calls without a bounding top_k have been tried once (as a probe)
 };
 static inline int policy_word(int kind) { return kind == 2 ? 3 : kind; }    // word[2] is the error report
 
@@ -265,7 +304,7 @@ namespace rs {
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
-enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5 };
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5, kPathProbe = 6 };
 // The wide path (four launches, two reads of the logits) against the general kernel (one launch, its
 // exchanges), measured on flat rows (U[0,1), top_p 0.9) and on N(0,1.5) with top_k 10000: the wide path
 // wins from about 2^25 tokens per call on in rows of 50304 tokens and more (256 x 131072: 104 against
@@ -317,6 +356,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     // kPenStreamMin tokens on (measured crossover with the general kernel), long slices only.
     rs_policy *pol = opt ? opt->policy : nullptr;
     // after a call of this kind with a slow row: the general kernel for a while, then another try
+    bool retry = false;                                       // routed_away() let this call through after a stay away
     auto routed_away = [&](int kind) {
         if (!pol) return false;
         if (*(volatile int32_t *)(pol->word + policy_word(kind)) == 0) {
@@ -328,6 +368,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         if (++pol->away[kind] <= pol->period[kind]) return true;
         pol->away[kind] = 0;                                  // this call streams again; a failure sets the word anew
         pol->period[kind] = min(pol->period[kind] * 2u, kAwayMost);
+        retry = true;
         return false;
     };
     if (pen && bounded && stream_r(B, V, true) == kStreamLongR && stream_parts(V, kStreamLongR) >= 2u) {
@@ -348,7 +389,16 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     auto wide_or_general = [&]() { return (uint64_t)B * (uint64_t)V >= kWideMin && V >= kWideMinV && !routed_away(2) ? kPathWide : kPathCluster; };
     if (!bounded && !(top_p < 1.0f)) return wide_or_general(); // a top_k of thousands and no nucleus: more than the stashes hold
     if (!pol) return bounded ? kPathStream : wide_or_general();
-    if (!routed_away(bounded ? 0 : 1)) return bounded ? kPathStream : kPathAttempt;
+    if (!routed_away(bounded ? 0 : 1)) {
+        if (bounded) return kPathStream;
+        // Whether the streaming path suits a workload without a bounding top_k is found out by a PROBE: the
+        // first call of that kind on a policy, and every call that tries again after a stay away, takes
+        // the wide path -- whose time does not depend on the kept set -- and its finishing workgroups report
+        // whether the rows' kept sets would have fitted the stashes.  An attempt that fails costs a pass
+        // of one workgroup over the row (hundreds of microseconds); a probe that says no costs nothing extra.
+        if (!pol->probed || retry) { pol->probed = 1u; return kPathProbe; }
+        return kPathAttempt;
+    }
     return bounded ? kPathCluster : wide_or_general();
 }
 
@@ -460,6 +510,7 @@ int rs_policy_create(rs_policy **out)
     if (!pol) return RS_ERR_LAUNCH;
     pol->word = nullptr;
     for (int i = 0; i < 3; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
+    pol->probed = 0;
     if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
         delete pol;
         return RS_ERR_LAUNCH;
@@ -590,7 +641,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.top_k = top_k; p.top_p = top_p;
     p.stash_k = (uint32_t)top_k; p.report = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
-    p.defer_pen = 0;
+    p.defer_pen = 0; p.probe = 0;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path != kPathCluster) {
@@ -624,9 +675,10 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         // with static LDS alone -- with a 64 KB list in dynamic LDS it was 32 x 1, and rows of 33 and
         // more slices could, rarely, starve until their waits gave up.
         if (path == kPathFused) v.list_cap = 2048u;
-        p.report = path == kPathAttempt ? 1u : path == kPathWide ? 3u : 0u;
+        p.report = path == kPathAttempt || path == kPathProbe ? 1u : path == kPathWide ? 3u : 0u;
+        p.probe = path == kPathProbe ? 1u : 0u;
         if (path == kPathKeep) { p.stash_k = 1u; v.list_cap = 2048u; }
-        if (path == kPathWide) {
+        if (path == kPathWide || path == kPathProbe) {
             // the list holds the tokens of ONE sub-bin of the boundary bin: 1/128 of it for a smooth distribution
             p.stash_k = 1u; v.list_cap = 4096u;
             return launch_wide(sr, logits_dtype, (uint32_t)B, (size_t)v.list_cap * sizeof(uint64_t), st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
@@ -731,10 +783,27 @@ int rs_floor_read(const float *logits, int64_t row_stride, int32_t *out, int32_t
     if (!logits || !out) return RS_ERR_NULL;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
-    if (variant < 0 || variant > 3) return RS_ERR_ARG;
+    if (variant < 0 || variant > 8) return RS_ERR_ARG;
     const uint32_t V4 = (uint32_t)V / 4;
     const bool once = (variant & 1) != 0;
     hipStream_t st = (hipStream_t)stream;
+    if (variant >= 4) {
+        // non-temporal loads throughout; pieces of kThreads * U float4
+        auto sweep = [&](auto kernel, uint32_t U, uint32_t grid_or_0, uint32_t per_or_0) {
+            const uint32_t ppr = (V4 + kThreads * U - 1) / (kThreads * U), pieces = (uint32_t)B * ppr;
+            const uint32_t grid = grid_or_0 ? min(grid_or_0, pieces) : (pieces + per_or_0 - 1) / per_or_0;
+            const uint32_t per = per_or_0 ? per_or_0 : (pieces + grid - 1) / grid + 1;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, st, logits, row_stride, out, V, ppr, pieces, per);
+        };
+        switch (variant) {
+        case 4: sweep(floor_sweep_kernel<4, true, false>, 4u, 2048u, 0u); break;     // persistent, 8 workgroups per CU, grid-strided, 4 loads in flight
+        case 5: sweep(floor_sweep_kernel<4, true, true>, 4u, 2048u, 0u); break;      // the same, an eighth of the data per XCD
+        case 6: sweep(floor_sweep_kernel<16, false, false>, 16u, 0u, 4u); break;     // 256 KiB per workgroup, contiguous, 16 loads in flight
+        case 7: sweep(floor_sweep_kernel<8, true, true>, 8u, 1024u, 0u); break;      // persistent, 4 workgroups per CU, per XCD, 8 loads in flight
+        default: sweep(floor_sweep_kernel<2, true, false>, 2u, 4096u, 0u); break;    // persistent, 16 workgroups per CU, 2 loads in flight
+        }
+        return hipGetLastError() == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+    }
 #define RS_FLOOR(Rv) do { const uint32_t G = (V4 + kThreads * Rv - 1) / (kThreads * Rv); const dim3 grid((uint32_t)B * G);                          \
         if (once) hipLaunchKernelGGL((floor_kernel<Rv, true>), grid, dim3(kThreads), 0, st, logits, row_stride, out, V, G);                     \
         else hipLaunchKernelGGL((floor_kernel<Rv, false>), grid, dim3(kThreads), 0, st, logits, row_stride, out, V, G); } while (0)

@@ -83,6 +83,7 @@ struct Params {
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     int32_t      dtype;        // RS_DTYPE_* of the logits
     uint32_t     report;       // which report word of the caller's policy a streaming call writes: 0 top_k bounds the kept set, 1 not, 3 the wide path
+    uint32_t     probe;        // wide path as a probe for the streaming path: rows whose kept set the stashes would not hold are reported as slow
     int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1], [3] routing reports, [2] error; or null
     int32_t      defer_pen;    // penalties enter x and are not rewritten from the registers at the end: 1 a later pass over them
                                // applies decay and one-hot add; 2 the streaming pass writes the decayed values itself and notes

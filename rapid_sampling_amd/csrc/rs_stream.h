@@ -367,7 +367,7 @@ __global__ void __launch_bounds__(NT, (R <= 8 ? 5 : RS_STREAM_WAVES)) stream_ker
         }
     }
     // a call that keeps everything has no rows to report on; the counting-only pass of the wide path does
-    if (reporter) report_end(p, prev, !KEEP || p.report == 3u);
+    if (reporter) report_end(p, prev, !KEEP || p.report != 0u);
     slice_count_and_stash<R, NT, kRep, false, KEEP>(p, v, s, eb, lmax, row, part, base4, nv);
 }
 

@@ -473,6 +473,13 @@ __device__ __forceinline__ void wide_finish_row(const Params &p, const StreamVie
     const uint32_t exb = f.bin >> 2;
     const uint64_t rand64 = p.inj_u ? 0ull : t.rand64;
 
+    auto tell_policy = [&]() {
+        if (tid == 0) {
+            const uint32_t c = __hip_atomic_fetch_add(&p.hdr->n_need, 1u, __ATOMIC_RELAXED, RS_AGENT);
+            if (c == 0u && p.host_words)
+                __hip_atomic_store(p.host_words + p.report, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+    };
     auto slow = [&]() {
         finish_row_slow(p, s, t, row, xmax, rand64);
         if (tid == 0) {
@@ -592,6 +599,8 @@ __device__ __forceinline__ void wide_finish_row(const Params &p, const StreamVie
     __syncthreads();
     const uint64_t w_tie = s.bc64[1];
     const u128 r = s.bc128[0];
+    // as a probe for the streaming path: would this row's kept set have fitted the stashes of an attempt?
+    if (p.probe && f.cnt_above + f.cnt_bin > 512u) tell_policy();
     auto weight = [=](uint32_t b) -> uint64_t { return (b > thr) ? w_of_bits(b) : (b == thr ? w_tie : 0ull); };
 
     // kept weight per slice: the listed tokens of slice g are entries [take[g-1], take[g])

@@ -1065,7 +1065,8 @@ def test_python_module_drop_in_calls(torch_cuda, oracle):
 
 
 def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
-    """top_k disabled, top_p < 1: the wait-free path is an attempt.  With a policy it is made; peaked rows
+    """top_k disabled, top_p < 1: the wait-free path is an attempt.  With a policy it is made, after one call
+    on the wide path that probes whether the rows' kept sets fit the stashes; peaked rows
     finish on it from the stashes (diag.rounds == 0).  A call with a row that had to be done the slow
     way (a flat row: the finishing workgroup goes through the logits again, diag.rounds == 8) says so in
     the policy's report word at once, and the next calls go to the general kernel; streaming is tried
@@ -1101,6 +1102,9 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
 
     smp = capi.Sampler(B, V, with_policy=True, init=True)
     assert policy(smp) == 0
+    res = smp.sample(lg_peaked, c, k, p, uniforms=u)     # the first call of its kind on a policy is a probe: the wide path
+    _check(res, *ref_peaked, "probe on peaked rows")
+    assert (res["diag"]["rounds"] == 7).all() and policy(smp) == 0
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)
     _check(res, *ref_peaked, "attempt on peaked rows")
     assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
@@ -1127,7 +1131,8 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
         else:
             assert (res["diag"]["rounds"] < 8).all() and (res["diag"]["rounds"] >= 1).all()
         assert policy(smp) == 1
-    assert streamed == [0, 129], streamed
+    # (the try after 128 calls is a probe on the wide path, which says no without doing any row the slow way)
+    assert streamed == [0], streamed
     assert smp.status() == 0
     smp.close()
     smp = capi.Sampler(B, V, with_policy=True, init=True)
