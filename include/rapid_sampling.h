@@ -334,6 +334,11 @@ int rs_sample_static(const void *logits_device, int32_t logits_dtype, int64_t ro
  * under stream capture.  No counterpart in the reference. */
 int rs_static_prepare(void);
 
+/* Device address of the current device's static array (RS_STATIC_SCRATCH_BYTES
+ * long), or NULL; for rs_workspace_where / rs_workspace_set_wait_limit and for
+ * tests.  No counterpart in the reference. */
+void *rs_static_workspace(void);
+
 /*
  * The sticky error word of the current device's static array (synchronises
  * `stream`): *status = RS_OK or RS_ERR_DEVICE; where[4], if not NULL, as

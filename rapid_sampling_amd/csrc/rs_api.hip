@@ -722,6 +722,12 @@ int rs_static_prepare(void)
     return static_base(&ws);
 }
 
+void *rs_static_workspace(void)
+{
+    void *ws = nullptr;
+    return static_base(&ws) == RS_OK ? ws : nullptr;
+}
+
 int rs_static_status(int32_t *status, uint32_t where[4], int32_t clear, void *stream)
 {
     if (!status) return RS_ERR_NULL;

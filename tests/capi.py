@@ -73,6 +73,12 @@ def lib():
         L.rs_sample_static.restype = C.c_int
         L.rs_sample_static.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, i32, f32, f32, f32, f32, i32, f32,
                                        vp, vp, C.POINTER(Options), vp]
+        L.rs_static_prepare.restype = C.c_int
+        L.rs_static_prepare.argtypes = []
+        L.rs_static_workspace.restype = C.c_void_p
+        L.rs_static_workspace.argtypes = []
+        L.rs_static_status.restype = C.c_int
+        L.rs_static_status.argtypes = [C.POINTER(i32), C.POINTER(C.c_uint32), i32, vp]
         L.rs_floor_read.restype = C.c_int
         L.rs_floor_read.argtypes = [vp, i64, vp, i32, i32, i32, vp]
         _lib = L
