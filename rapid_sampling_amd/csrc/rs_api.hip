@@ -272,18 +272,28 @@ static size_t stream_bytes(int32_t B, int32_t V)
 
 }  // namespace rs
 
-// The caller's routing state (see rapid_sampling.h).  word[0], word[1], word[3]: "a row had to be done
-// the slow way" as last reported by a streaming call with / without a bounding top_k and by a call on
-// the wide path; word[2]: RS_ERR_DEVICE once a kernel gave up a wait.  away[]: calls routed away from the streaming path
-// since the word was last seen set and streaming tried; period[]: how many of them before streaming
-// is tried again; good[]: streaming calls in a row that found the word clear.
+// The caller's routing state (see rapid_sampling.h).  Calls are of one of three kinds -- 0 the streaming
+// path with a bounding top_k, 1 without one (an attempt), 2 the wide path -- and of one of three size
+// classes (tokens per call below 2^20, below 2^24, from 2^24 on), and every (kind, class) has a report
+// word of its own in pinned host memory, "a row had to be done the slow way" as last reported by a call of
+// that kind and class: workloads that share a policy (a lone flat row and a batch of peaked ones on one
+// stream) do not flip each other's route.  word[2]: RS_ERR_DEVICE once a kernel gave up a wait.  away[]:
+// calls routed away since the word was last seen set and the path tried; period[]: how many of them
+// before it is tried again; good[]: calls in a row that found the word clear.
 constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u;
+constexpr int kKinds = 3, kClasses = 3;
 struct rs_policy {
     int32_t *word;
-    uint32_t away[3], period[3], good[3];                // kinds: 0 streaming with a bounding top_k, 1 without, 2 the wide path
-    uint32_t probed;                                     // calls without a bounding top_k have been tried once (as a probe)
+    uint32_t away[kKinds * kClasses], period[kKinds * kClasses], good[kKinds * kClasses];
+    uint32_t probed[kClasses];                           // calls without a bounding top_k of this class have been tried once (as a probe)
 };
-static inline int policy_word(int kind) { return kind == 2 ? 3 : kind; }    // word[2] is the error report
+static inline int size_class(int32_t B, int32_t V)
+{
+    const uint64_t n = (uint64_t)B * (uint64_t)V;
+    return n < (1ull << 20) ? 0 : n < (1ull << 24) ? 1 : 2;
+}
+static inline int policy_slot(int kind, int cls) { return kind * kClasses + cls; }
+static inline int policy_word(int kind, int cls) { return 4 + policy_slot(kind, cls); }
 
 namespace rs {
 
@@ -355,19 +365,21 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     // Larger calls with penalties: the streaming pass with a pass over the penalties behind it, from
     // kPenStreamMin tokens on (measured crossover with the general kernel), long slices only.
     rs_policy *pol = opt ? opt->policy : nullptr;
+    const int cls = size_class(B, V);
     // after a call of this kind with a slow row: the general kernel for a while, then another try
     bool retry = false;                                       // routed_away() let this call through after a stay away
     auto routed_away = [&](int kind) {
         if (!pol) return false;
-        if (*(volatile int32_t *)(pol->word + policy_word(kind)) == 0) {
-            if (pol->period[kind] > kAwayFirst && ++pol->good[kind] >= pol->period[kind]) pol->period[kind] = kAwayFirst;
-            pol->away[kind] = 0;
+        const int slot = policy_slot(kind, cls);
+        if (*(volatile int32_t *)(pol->word + policy_word(kind, cls)) == 0) {
+            if (pol->period[slot] > kAwayFirst && ++pol->good[slot] >= pol->period[slot]) pol->period[slot] = kAwayFirst;
+            pol->away[slot] = 0;
             return false;
         }
-        pol->good[kind] = 0;
-        if (++pol->away[kind] <= pol->period[kind]) return true;
-        pol->away[kind] = 0;                                  // this call streams again; a failure sets the word anew
-        pol->period[kind] = min(pol->period[kind] * 2u, kAwayMost);
+        pol->good[slot] = 0;
+        if (++pol->away[slot] <= pol->period[slot]) return true;
+        pol->away[slot] = 0;                                  // this call streams again; a failure sets the word anew
+        pol->period[slot] = min(pol->period[slot] * 2u, kAwayMost);
         retry = true;
         return false;
     };
@@ -396,7 +408,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         // the wide path -- whose time does not depend on the kept set -- and its finishing workgroups report
         // whether the rows' kept sets would have fitted the stashes.  An attempt that fails costs a pass
         // of one workgroup over the row (hundreds of microseconds); a probe that says no costs nothing extra.
-        if (!pol->probed || retry) { pol->probed = 1u; return kPathProbe; }
+        if (!pol->probed[cls] || retry) { pol->probed[cls] = 1u; return kPathProbe; }
         return kPathAttempt;
     }
     return bounded ? kPathCluster : wide_or_general();
@@ -509,8 +521,8 @@ int rs_policy_create(rs_policy **out)
     rs_policy *pol = new (std::nothrow) rs_policy;
     if (!pol) return RS_ERR_LAUNCH;
     pol->word = nullptr;
-    for (int i = 0; i < 3; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
-    pol->probed = 0;
+    for (int i = 0; i < kKinds * kClasses; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
+    for (int i = 0; i < kClasses; ++i) pol->probed[i] = 0;
     if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
         delete pol;
         return RS_ERR_LAUNCH;
@@ -531,7 +543,8 @@ int rs_policy_state(const rs_policy *pol, int32_t *state)
 {
     if (!pol || !state) return RS_ERR_NULL;
     const volatile int32_t *w = pol->word;
-    *state = (w[1] != 0 ? 1 : 0) | (w[0] != 0 ? 2 : 0) | (w[3] != 0 ? 4 : 0);
+    auto any = [&](int kind) { return w[policy_word(kind, 0)] != 0 || w[policy_word(kind, 1)] != 0 || w[policy_word(kind, 2)] != 0; };
+    *state = (any(1) ? 1 : 0) | (any(0) ? 2 : 0) | (any(2) ? 4 : 0);
     return RS_OK;
 }
 
@@ -639,7 +652,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.row_stride = row_stride; p.B = B; p.V = V; p.G = g.G;
     p.presence = presence; p.repetition = repetition; p.decay = decay; p.c = log2e_inv_temp;
     p.top_k = top_k; p.top_p = top_p;
-    p.stash_k = (uint32_t)top_k; p.report = 0;
+    p.stash_k = (uint32_t)top_k; p.report = 0; p.attempt = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
     p.defer_pen = 0; p.probe = 0;
     dim3 grid((uint32_t)B * g.G);
@@ -675,7 +688,9 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         // with static LDS alone -- with a 64 KB list in dynamic LDS it was 32 x 1, and rows of 33 and
         // more slices could, rarely, starve until their waits gave up.
         if (path == kPathFused) v.list_cap = 2048u;
-        p.report = path == kPathAttempt || path == kPathProbe ? 1u : path == kPathWide ? 3u : 0u;
+        const int kind = path == kPathAttempt || path == kPathProbe ? 1 : path == kPathWide ? 2 : 0;
+        p.report = path == kPathKeep ? 0u : (uint32_t)policy_word(kind, size_class(B, V));
+        p.attempt = path == kPathAttempt ? 1u : 0u;
         p.probe = path == kPathProbe ? 1u : 0u;
         if (path == kPathKeep) { p.stash_k = 1u; v.list_cap = 2048u; }
         if (path == kPathWide || path == kPathProbe) {

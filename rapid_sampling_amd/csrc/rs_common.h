@@ -82,9 +82,10 @@ struct Params {
     RowCtl      *ctl_end;      // one past the record of row 0; row r is ctl_end[-1 - r]
     uint32_t     stash_k;      // streaming pass: tokens a slice aims to stash (<= top_k)
     int32_t      dtype;        // RS_DTYPE_* of the logits
-    uint32_t     report;       // which report word of the caller's policy a streaming call writes: 0 top_k bounds the kept set, 1 not, 3 the wide path
+    uint32_t     report;       // index of the report word of the caller's policy a streaming call writes (4..12: kind of call x size class), 0 none
+    uint32_t     attempt;      // the call has no bounding top_k: its streaming pass is an attempt
     uint32_t     probe;        // wide path as a probe for the streaming path: rows whose kept set the stashes would not hold are reported as slow
-    int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [0], [1], [3] routing reports, [2] error; or null
+    int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [2] error, [4..12] routing reports; or null
     int32_t      defer_pen;    // penalties enter x and are not rewritten from the registers at the end: 1 a later pass over them
                                // applies decay and one-hot add; 2 the streaming pass writes the decayed values itself and notes
                                // the old non-zero ones, the finish patches the sampled token (see stream_pen_kernel)
@@ -348,7 +349,7 @@ __device__ __forceinline__ void report_end(const Params &p, const PrevCall &pc, 
     if (streaming) a_store(&p.hdr->last_call, 1u | (p.report << 8));
     else if (pc.meta) a_store(&p.hdr->last_call, 0u);
     if (p.host_words && pc.meta)
-        __hip_atomic_store(p.host_words + ((pc.meta >> 8) & 3u), pc.slow_rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(p.host_words + ((pc.meta >> 8) & 15u), pc.slow_rows ? 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 __device__ __forceinline__ void lds_hist_zero(Lds &s, int nb)

@@ -1111,7 +1111,7 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     // there and, the general kernel's time growing with the row, at about 4700 for rows of 100256): a
     // call that is only an attempt (no top_k bounds the kept set) says so to the caller's policy.
     const uint32_t long_list = max(2048u, (uint32_t)p.V / 20u);
-    if (!FUSED && p.report == 1u && total > long_list) tell_policy();
+    if (!FUSED && p.attempt && total > long_list) tell_policy();
 
     // gather the tokens, re-based to the row's frame
     if (!listed)

@@ -1166,6 +1166,41 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     smp.close()
 
 
+def test_routing_is_kept_per_kind_and_size_of_call(torch_cuda, oracle):
+    """Two workloads interleaved on one workspace and one policy, both without a bounding top_k: a lone
+    flat row (its kept set never fits the stashes) and a batch of peaked rows (always does).  The report
+    words are kept per kind and size class of call, so the flat row's reports do not send the batch to the
+    general kernel, and the batch's good reports do not send the flat row back to the streaming path: after
+    its probe, every call of the batch is finished from the stashes (diag.rounds == 0), and no call of the
+    flat row is ever done the slow way (diag.rounds == 8)."""
+    torch = torch_cuda
+    from tests import capi
+    Vf, Bp, Vp = 262144, 48, 152064
+    flat = (np.random.default_rng(95).random((1, Vf), dtype=np.float32) * np.float32(4.0)).astype(np.float32)
+    peaked = H.logits_normal(Bp, Vp, 3.0, seed=96)
+    uf_np, up_np = H.uniforms(1, 97), H.uniforms(Bp, 98)
+    rc, cf, kf, pf = capi.normalize(1.0, -1, 0.3, Vf, 1, 1)
+    rc, cp, kp, pp = capi.normalize(1.0, -1, 0.3, Vp, Bp, 1)
+    ref_f = oracle.sample_batch(flat, cf, kf, pf, injected_u=uf_np)
+    ref_p = oracle.sample_batch(peaked, cp, kp, pp, injected_u=up_np)
+    lg_f, lg_p = torch.from_numpy(flat).cuda(), torch.from_numpy(peaked).cuda()
+    uf, up = torch.from_numpy(uf_np).cuda(), torch.from_numpy(up_np).cuda()
+    smp = capi.Sampler(Bp, Vf, with_policy=True, init=True)           # one workspace large enough for both shapes
+    flat_rounds, peaked_rounds = [], []
+    for i in range(150):
+        res = smp.sample(lg_f, cf, kf, pf, uniforms=uf)
+        _check(res, *ref_f, "interleaved, flat row, call %d" % i)
+        flat_rounds.append(int(res["diag"]["rounds"][0]))
+        res = smp.sample(lg_p, cp, kp, pp, uniforms=up)
+        _check(res, *ref_p, "interleaved, peaked batch, call %d" % i)
+        peaked_rounds.append(sorted(set(res["diag"]["rounds"].tolist())))
+    assert peaked_rounds[0] == [7] and all(r == [0] for r in peaked_rounds[1:]), peaked_rounds[:5]
+    assert flat_rounds[0] == 7 and 8 not in flat_rounds, flat_rounds[:10]
+    assert sum(1 for r in flat_rounds if r == 7) <= 3                  # the probe, and one or two retries (64, 128 calls later)
+    assert smp.policy_state() == 1 and smp.status() == 0
+    smp.close()
+
+
 def test_two_streams_two_workspaces_concurrently(torch_cuda, oracle):
     """Calls on two streams, each with its own workspace, state and outputs, issued alternately
     without any synchronisation in between, so that their kernels share the GPU: a cluster-path
