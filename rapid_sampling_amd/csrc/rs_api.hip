@@ -192,15 +192,24 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
     // Measured on MI355X: a cluster works best with at most ~64 workgroups (each exchange costs
     // more the more peers poll), slices of 32 float4 per thread only pay for rows of a quarter
     // million tokens and more (the variant spills), and a call wants a few hundred workgroups in
-    // flight -- 256 for small batches, where latency counts, 512 beyond.
+    // flight.
     int minR = maxR;
     for (int R = 1; R <= maxR; R *= 2)
         if (parts(R) <= 64u) { minR = R; break; }
     const int topR = (V4 >= 65536u || minR > 16) ? maxR : (maxR < 16 ? maxR : 16);
-    const uint64_t want = B <= 16 ? 256 : 512;
     int pick = minR;
-    for (int R = topR; R >= minR; R /= 2)
-        if ((uint64_t)B * parts(R) >= want) { pick = R; break; }
+    if (B <= 16) {
+        // a handful of rows: the shortest slices that keep the call within 256 workgroups (measured for 8 and
+        // 16 rows of 32768 to 100256 tokens: 128-256 workgroups 20-24 us, 400-800 workgroups 25-37 us; one to
+        // four rows are as fast with any length up to 8192 tokens)
+        for (int R = minR; R <= topR; R *= 2) {
+            pick = R;
+            if ((uint64_t)B * parts(R) <= 256u) break;
+        }
+    } else {
+        for (int R = topR; R >= minR; R /= 2)
+            if ((uint64_t)B * parts(R) >= 512u) { pick = R; break; }
+    }
     // A launch the device holds at once (256 CUs x the workgroups per CU of the variant, see
     // min_waves) draws no tickets, and tickets cost the first workgroups of a larger launch 10-15 us:
     // if a longer slice brings the launch within that, take it (measured on flat rows, 128-512 of
@@ -394,7 +403,11 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
     if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
     if (force == RS_PATH_WIDE) return keep_all ? kPathKeep : kPathWide;
-    if ((uint64_t)B * (uint64_t)V < (1ull << 17)) return kPathCluster;
+    // Small calls: rows of fewer than 8192 tokens are one or two workgroups of the general kernel each, with
+    // few or no exchanges (8.5 us for a row of 256 tokens); from 8192 tokens per row on the streaming
+    // path's two launches are faster whatever the batch (one row of 8192 to 100256 tokens: 13.6-14.7
+    // against 16.1-17.9 us, 16 rows: 14.5-15.8 against 16.8-21.3; measured per call between events).
+    if ((uint64_t)B * (uint64_t)V < (1ull << 17) && V < 8192) return kPathCluster;
     if (keep_all && V >= 32768) return kPathKeep;              // shorter rows: one workgroup of the general kernel does a row in one go
     // kept sets the stashes cannot hold: the wide path from kWideMin tokens on, unless its rows have been
     // going the slow way (slices that are no fair samples of their rows, ties of thousands of tokens)

@@ -1358,6 +1358,15 @@ def test_python_module_calls_captured_into_a_graph(torch_cuda, oracle):
     assert np.array_equal(pen.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32))
     with torch.cuda.stream(side):
         assert sample.workspace_status() == 0
+        # reset_routing replaces the policy object; the graph's kernels still hold the old one's pinned
+        # words, which therefore must stay allocated: replays after the reset work as before
+        sample._sample.reset_routing()
+    for i in range(2):
+        ref_a, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref)
+        ref_b, _ = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref, penalties=pen_ref, presence=0.1, repetition=0.2, decay=0.9)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(a.cpu().numpy(), ref_a) and np.array_equal(b.cpu().numpy(), ref_b), ("after reset_routing", i)
     # a stream without a workspace: the first call would have to allocate while capturing
     other = torch.cuda.Stream()
     with torch.cuda.stream(other):
