@@ -8,16 +8,20 @@ constexpr int kStreamNT = 256;
 hipError_t launch_stream(int slice_r, int32_t dtype, bool keep, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p,
                          const StreamView &v)
 {
-    const dim3 sgrid(B * v.G), sblock(kStreamNT);
-    // keep: the call keeps every live token; its kernels neither fill nor read stashes, and the finish needs no list
-#define RS_STREAM(Rv, Lv, KEEPv) do {                                                                                              \
-        if (dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<Rv, kStreamNT, RS_DTYPE_F32, KEEPv>), sgrid, sblock, 0, st, p, v);       \
-        else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<Rv, kStreamNT, RS_DTYPE_BF16, KEEPv>), sgrid, sblock, 0, st, p, v); \
-        else hipLaunchKernelGGL((stream_kernel<Rv, kStreamNT, RS_DTYPE_F16, KEEPv>), sgrid, sblock, 0, st, p, v);                             \
+    const dim3 sgrid(B * v.G);
+    // keep: the call keeps every live token; its kernels neither fill nor read stashes, and the finish needs no list.
+    // NTv threads with Rv groups of four tokens each: a slice of 4 Rv NTv tokens
+#ifndef RS_LONG_NT
+#define RS_LONG_NT 256
+#endif
+#define RS_STREAM(Rv, NTv, Lv, KEEPv) do {                                                                                         \
+        if (dtype == RS_DTYPE_F32) hipLaunchKernelGGL((stream_kernel<Rv, NTv, RS_DTYPE_F32, KEEPv>), sgrid, dim3(NTv), 0, st, p, v);       \
+        else if (dtype == RS_DTYPE_BF16) hipLaunchKernelGGL((stream_kernel<Rv, NTv, RS_DTYPE_BF16, KEEPv>), sgrid, dim3(NTv), 0, st, p, v); \
+        else hipLaunchKernelGGL((stream_kernel<Rv, NTv, RS_DTYPE_F16, KEEPv>), sgrid, dim3(NTv), 0, st, p, v);                             \
         hipLaunchKernelGGL((finish_kernel<Lv, KEEPv>), dim3(B), dim3(kThreads), KEEPv ? 0 : finish_lds_bytes, st, p, v); } while (0)
-    if (slice_r == 4) { if (keep) RS_STREAM(4, 12, true); else RS_STREAM(4, 12, false); }
-    else if (slice_r == 8) { if (keep) RS_STREAM(8, 13, true); else RS_STREAM(8, 13, false); }
-    else { if (keep) RS_STREAM(kStreamLongR, kStreamLongLog2, true); else RS_STREAM(kStreamLongR, kStreamLongLog2, false); }
+    if (slice_r == 4) { if (keep) RS_STREAM(4, 256, 12, true); else RS_STREAM(4, 256, 12, false); }
+    else if (slice_r == 8) { if (keep) RS_STREAM(8, 256, 13, true); else RS_STREAM(8, 256, 13, false); }
+    else { if (keep) RS_STREAM((kStreamLongR * 256 / RS_LONG_NT), RS_LONG_NT, kStreamLongLog2, true); else RS_STREAM((kStreamLongR * 256 / RS_LONG_NT), RS_LONG_NT, kStreamLongLog2, false); }
 #undef RS_STREAM
     return hipGetLastError();
 }

@@ -507,6 +507,37 @@ def test_cluster_levels_with_slices_that_hold_no_boundary_tokens(torch_cuda, ora
             _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="contiguous ties k=%s p=%s T=%s #%d" % (k, p, t, rep))
 
 
+def test_cluster_bins_posted_ahead_when_frames_lie_far_apart(torch_cuda, oracle):
+    """The general kernel's workgroups post the next digit of the bin in which they expect the row's
+    boundary ahead of the first exchange.  Rows whose slices lie in frames too far apart (whole slices
+    masked) make no use of that, redo level 1 and clear everything early: the bins posted ahead must be
+    complete, and read by nobody any more, before a workgroup clears its share of them (a workgroup that
+    cleared while others were still adding them up left those waiting until they gave up, now and then).
+    Flat rows, whose slices all post and agree, and sorted rows, whose slices post different bins, beside
+    them; every call against the oracle, a dozen calls on one workspace."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 12, 266240
+    rng = np.random.default_rng(321)
+    lg = (rng.standard_normal((B, V)) * 15).astype(np.float32)
+    lg[1, : V // 2] = -np.inf
+    lg[3, :] = -np.inf; lg[3, V - 7:] = rng.standard_normal(7)
+    lg[5] = rng.random(V, dtype=np.float32)
+    lg[6] = np.sort(rng.random(V, dtype=np.float32))
+    lg[7, 40000:200000] = -np.inf
+    lg[8] = rng.random(V, dtype=np.float32) * 4
+    u_np = H.uniforms(B, 322)
+    smp = capi.Sampler(B, V)
+    L, U = torch.from_numpy(lg).cuda(), torch.from_numpy(u_np).cuda()
+    for (t, k, p) in [(1.0, -1, 0.5), (0.7, 3000, 1.0), (1.0, 50, 0.9)]:
+        rc, c, kk, pp = capi.normalize(t, k, p, V, B, 1)
+        ref_out, ref_diag = oracle.sample_batch(lg, c, kk, pp, injected_u=u_np)
+        for it in range(4):
+            res = smp.sample(L, c, kk, pp, uniforms=U, path="cluster")
+            _check(res, ref_out, ref_diag, "posted ahead, T=%g k=%d p=%g call %d" % (t, k, p, it))
+            assert smp.status() == 0
+
+
 @pytest.mark.parametrize("fmt", ["float32", "bfloat16", "float16"])
 def test_streaming_path_middle_slices(torch_cuda, oracle, fmt):
     """Calls whose 4096-token slices no longer fit the device at once but whose 8192-token slices do
