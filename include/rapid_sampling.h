@@ -85,11 +85,11 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
 /*
  * Size of the workspace rs_sample needs for a batch of B rows of V tokens.
  * Replaces the reference's per-call `probs` scratch tensor of B*V floats
- * (sampling.cu:488,1014): a fixed record per row (about 38 KB) plus, for the
- * streaming path, about 0.8 bytes per token (stashes of the largest tokens,
- * counts and bins of each slice; up to 3.2 bytes per token for the first 4M
- * tokens, where slices are shorter); a fifth of the reference's scratch for
- * large V.
+ * (sampling.cu:488,1014): a fixed record per row (about 39 KB) plus, for the
+ * streaming paths, about 1.05 bytes per token (per slice of 16384 tokens the
+ * stash of its largest tokens, its counts and bins, and 4 KB for its note of
+ * the non-zero penalties; up to 3.2 bytes per token for the first 6M tokens,
+ * where slices are shorter); a quarter of the reference's scratch for large V.
  * It does not grow with T.
  *
  * One workspace may serve calls of different shapes if it is at least
@@ -125,14 +125,15 @@ int rs_workspace_status(const void *workspace_device, int32_t *status, void *str
  * Where the first wait that gave up was (synchronises `stream`; no counterpart
  * in the reference).  where[0] = the wait (0 none; 1 a histogram level,
  * 2 the first level's totals, 3 the candidates of a level, 4 the masses,
- * 5 the index, 6 the verdict of the one-launch kernel), where[1] =
+ * 5 the index, 6 the verdict of the one-launch kernel, 7 the slots and bins
+ * the workgroups of a row post ahead of the first exchange), where[1] =
  * row << 16 | slice of the workgroup that gave up, where[2] and where[3] = what
  * it had seen and what it waited for.  Cleared by rs_workspace_init.
  */
 int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *stream);
 
 /*
- * Routing state of the streaming path and an asynchronous error report, owned
+ * Routing state of the streaming paths and an asynchronous error report, owned
  * by the caller (optional; one per workspace).  No counterpart in the
  * reference.
  *
@@ -146,25 +147,37 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * the general kernel is faster for such calls; a call of fewer than 2^24
  * tokens with a bounding top_k counts a row as slow when its stashes hold
  * more tokens than the finishing workgroup's list and have to be gone through
- * twice more -- flat rows cut into many slices -- for the same reason).  Calls
- * that are given a policy report "a row went the slow
- * way: yes/no" to a word of pinned host memory inside it (yes at once, no by
- * the next call on the workspace), and rs_sample_ex reads that word, without
- * waiting, before it routes the next call: while it is set, calls of that
- * kind go to the general kernel; after 64 of them the streaming path is tried
- * again, each try that fails doubles that number (up to 1024), and a run of
- * good streaming calls as long as the last stay away puts it back to 64.
- * Without a policy, calls with a bounding top_k always stream and calls
- * without never do.  Results do not depend on the routing.
+ * twice more -- flat rows cut into many slices -- for the same reason).  The
+ * wide path (kept sets of any size, two passes over the logits) does a row the
+ * slow way when its slices are no fair samples of the row.  Calls that are
+ * given a policy report "a row went the slow way: yes/no" to a word of pinned
+ * host memory inside it (yes at once, no by the next call on the workspace),
+ * and rs_sample_ex reads that word, without waiting, before it routes the
+ * next call: while it is set, calls of that kind go to the general kernel (a
+ * call without a bounding top_k to the wide path when it is large enough);
+ * after 64 of them the path is tried again, each try that fails doubles that
+ * number (up to 1024), and a run of good calls as long as the last stay away
+ * puts it back to 64.  There is a word per KIND of call -- streaming with a
+ * bounding top_k, streaming without, wide -- and per SIZE CLASS (tokens per
+ * call below 2^20, below 2^24, from 2^24 on), so that workloads that share a
+ * policy do not flip each other's route.  The first call without a bounding
+ * top_k of a size class, and every such call that tries again after a stay
+ * away, runs as a PROBE: on the wide path, whose time does not depend on the
+ * kept set, with the finishing workgroups reporting whether the rows' kept sets
+ * (more than 512 tokens?) would have fitted the streaming path's stashes --
+ * so a workload of flat rows never pays for a row done the slow way.  Without
+ * a policy, calls with a bounding top_k always stream and calls without never
+ * do.  Results do not depend on the routing.
  *
  * A kernel that gives up waiting (RS_ERR_DEVICE) also writes the code into a
- * third pinned word, which rs_policy_error reads without synchronising.
+ * pinned word, which rs_policy_error reads without synchronising.
  *
  * rs_policy_create allocates (a small host object and 64 bytes of pinned host
  * memory); rs_policy_destroy frees them -- only after the last call that was
  * given the policy has completed on the device.
- * rs_policy_state: bit 0 set: calls without a bounding top_k currently go to
- * the general kernel, bit 1 set: so do calls with one.
+ * rs_policy_state (over all size classes): bit 0 set: calls without a bounding
+ * top_k currently leave the streaming path, bit 1 set: so do calls with one,
+ * bit 2 set: calls that would take the wide path take the general kernel.
  * rs_policy_error: *error = RS_OK or RS_ERR_DEVICE as last reported; with
  * clear != 0 the word is reset.
  */
@@ -207,17 +220,24 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  *
  * Calls that share a workspace must be ordered on one stream.
  *
- * The call is one kernel launch (the general kernel; with penalties and
- * top_k <= 1024 the one-launch streaming kernel while the call fits the GPU at
- * once), two for calls of at least 2^17 tokens without penalties whose kept
+ * The call is one kernel launch (the general kernel: rows of fewer than 8192
+ * tokens in calls of fewer than 2^17, and whatever the other paths do not
+ * take; with penalties and top_k <= 1024 the one-launch streaming kernel while
+ * the call fits the GPU at once), two for calls without penalties whose kept
  * set is expected to be small (a wait-free pass over the logits and a per-row
  * finish; see rs_policy; plain temperature sampling -- top_k = V, top_p = 1,
  * every token kept -- takes these two launches as well: the pass only counts,
- * and the finish reads one slice of the row again), or three for calls of at
- * least 2^23 tokens with
- * penalties and top_k <= 1024 (the same two and a pass that rewrites the
- * penalties); results are identical either way.  No environment variable is
- * read.
+ * and the finish reads one slice of the row again), four for kept sets of
+ * thousands of tokens in calls of at least 2^25 tokens (the wide path: the
+ * counting pass, a one-workgroup-per-row plan, a second pass over the logits
+ * that counts the boundary bin's next digit and sets the tokens around the
+ * expected threshold aside, a per-row finish), or three for calls of at least
+ * 2^23 tokens with penalties and top_k <= 1024 (a pass over logits and
+ * penalties that also writes the decayed penalties, the finish, which patches
+ * the sampled tokens' penalties, and a fix-up kernel for slices the pass left
+ * alone); results are identical either way.  No environment variable is read.
+ * A device that is not a whole MI355X (256 compute units) is refused with
+ * RS_ERR_UNSUPPORTED: the kernels' waits are only known to end on one.
  */
 int rs_sample(const float *logits_device, int64_t row_stride,
               float *penalties_device, int32_t *out_device,
@@ -260,7 +280,9 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
  * RS_PATH_ATTEMPT the streaming path whatever top_k is (penalties take the
  * general kernel on these three), RS_PATH_FUSED the streaming pass and the
  * finish in one launch (any call whose rows span at least two slices, with or
- * without penalties; else the general kernel).  `slice_r` forces the float4 groups per thread of the
+ * without penalties; else the general kernel), RS_PATH_WIDE the wide path (any
+ * call without penalties; a call that keeps every token takes the counting-only
+ * streaming variant).  `slice_r` forces the float4 groups per thread of the
  * general kernel (1, 2, 4, 8, 16 or 32; 0 = chosen by the library).
  * `policy` see rs_policy.  No counterpart in the reference.
  */

@@ -284,7 +284,11 @@ __device__ __forceinline__ bool slice_level1(const Params &p, Lds &s, Slice<R, P
             }
             __syncthreads();
             const uint32_t guess = s.bc32[3], nguess = s.bc32[4];
-            const bool post = guess != 0u && (uint64_t)nguess * G > (uint64_t)kCap;
+            // (a bin that is one tie of the slice's largest token -- rows of equal logits -- is not posted: the
+            // row is recognised as one tie without another level, and counting it would queue every token
+            // of the slice up at one address)
+            const bool post = guess != 0u && (uint64_t)nguess * G > (uint64_t)kCap &&
+                              !bin_is_one_tie(s.hm[(guess + pos0) & 511u], guess, e_bits_of(fkey_inv(kmax_row), Mloc));
             if (post) {
                 if (tid < 128) s.cand[tid] = 0;
                 __syncthreads();
