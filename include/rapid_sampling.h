@@ -85,7 +85,7 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
 /*
  * Size of the workspace rs_sample needs for a batch of B rows of V tokens.
  * Replaces the reference's per-call `probs` scratch tensor of B*V floats
- * (sampling.cu:488,1014): a fixed record per row (about 39 KB) plus, for the
+ * (sampling.cu:488,1014): a fixed record per row (about 38 KB) plus, for the
  * streaming paths, about 1.05 bytes per token (per slice of 16384 tokens the
  * stash of its largest tokens, its counts and bins, and 4 KB for its note of
  * the non-zero penalties; up to 3.2 bytes per token for the first 6M tokens,
@@ -165,7 +165,11 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * away, runs as a PROBE: on the wide path, whose time does not depend on the
  * kept set, with the finishing workgroups reporting whether the rows' kept sets
  * (more than 512 tokens?) would have fitted the streaming path's stashes --
- * so a workload of flat rows never pays for a row done the slow way.  Without
+ * so a workload of flat rows never pays for a row done the slow way.  A probe
+ * reports on itself when it has run; until then its word is pending and calls
+ * of its kind and size class are probes too (at most 64 of them), so a caller
+ * that issues many calls without synchronising does not run attempts on rows
+ * nobody has looked at yet.  Without
  * a policy, calls with a bounding top_k always stream and calls without never
  * do.  Results do not depend on the routing.
  *
@@ -228,7 +232,7 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  * finish; see rs_policy; plain temperature sampling -- top_k = V, top_p = 1,
  * every token kept -- takes these two launches as well: the pass only counts,
  * and the finish reads one slice of the row again), four for kept sets of
- * thousands of tokens in calls of at least 2^25 tokens (the wide path: the
+ * thousands of tokens in calls of at least 3 * 2^23 tokens (the wide path: the
  * counting pass, a one-workgroup-per-row plan, a second pass over the logits
  * that counts the boundary bin's next digit and sets the tokens around the
  * expected threshold aside, a per-row finish), or three for calls of at least

@@ -289,12 +289,18 @@ static size_t stream_bytes(int32_t B, int32_t V)
 // stream) do not flip each other's route.  word[2]: RS_ERR_DEVICE once a kernel gave up a wait.  away[]:
 // calls routed away since the word was last seen set and the path tried; period[]: how many of them
 // before it is tried again; good[]: calls in a row that found the word clear.
-constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u;
+// A probe's word is "pending" (kWordPending, set by the host with the call) until the probe has run: calls of
+// its kind issued in the meantime -- a caller that does not synchronise between calls issues many -- are
+// probes too, not attempts that may have to do their rows the slow way; after kPendingMost of them the
+// word is taken to be clear.
+constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u, kPendingMost = 64u;
+constexpr int32_t kWordPending = 2;
 constexpr int kKinds = 3, kClasses = 3;
 struct rs_policy {
     int32_t *word;
     uint32_t away[kKinds * kClasses], period[kKinds * kClasses], good[kKinds * kClasses];
     uint32_t probed[kClasses];                           // calls without a bounding top_k of this class have been tried once (as a probe)
+    uint32_t pending[kClasses];                          // calls issued since a probe of this class whose word is still pending
 };
 static inline int size_class(int32_t B, int32_t V)
 {
@@ -326,11 +332,12 @@ namespace rs {
 enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5, kPathProbe = 6 };
 // The wide path (four launches, two reads of the logits) against the general kernel (one launch, its
 // exchanges), measured on flat rows (U[0,1), top_p 0.9) and on N(0,1.5) with top_k 10000: the wide path
-// wins from about 2^25 tokens per call on in rows of 50304 tokens and more (256 x 131072: 104 against
-// 108 us and 85 against 99; 128 x 262144: 102 against 119; 32 x 1048576: 106 against 133; 512 x 262144:
-// 280 against 395), loses below that (128 x 131072: 74 against 66) and in short rows (2048 x 32768:
-// 225 against 193).
-constexpr uint64_t kWideMin = 1ull << 25;
+// wins from about 25 million tokens per call on in rows of 50304 tokens and more (96 x 262144: 88 against
+// 102 us and 69 against 93; 256 x 100256: 92 against 96 and 75 against 88; 512 x 50304: 105 against 107
+// and 86 against 97; 256 x 131072: 104 against 108 and 85 against 99; 32 x 1048576: 106 against 133;
+// 512 x 262144: 280 against 395), loses below that (128 x 131072: 72 against 64 and 58 against 61) and
+// in short rows (2048 x 32768: 225 against 193).
+constexpr uint64_t kWideMin = 3ull << 23;
 constexpr int32_t kWideMinV = 49152;
 constexpr uint64_t kPenStreamMin = 1ull << 23;
 // Plain temperature sampling (top_k = V, top_p = 1: every live token is kept) has no kept set to
@@ -377,10 +384,16 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     const int cls = size_class(B, V);
     // after a call of this kind with a slow row: the general kernel for a while, then another try
     bool retry = false;                                       // routed_away() let this call through after a stay away
+    bool pending = false;                                     // a probe of this class has been issued and has not run yet
     auto routed_away = [&](int kind) {
         if (!pol) return false;
         const int slot = policy_slot(kind, cls);
-        if (*(volatile int32_t *)(pol->word + policy_word(kind, cls)) == 0) {
+        volatile int32_t *word = pol->word + policy_word(kind, cls);
+        if (*word == kWordPending) {
+            if (++pol->pending[cls] <= kPendingMost) { pending = true; return false; }
+            *word = 0;
+        }
+        if (*word == 0) {
             if (pol->period[slot] > kAwayFirst && ++pol->good[slot] >= pol->period[slot]) pol->period[slot] = kAwayFirst;
             pol->away[slot] = 0;
             return false;
@@ -421,7 +434,11 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         // the wide path -- whose time does not depend on the kept set -- and its finishing workgroups report
         // whether the rows' kept sets would have fitted the stashes.  An attempt that fails costs a pass
         // of one workgroup over the row (hundreds of microseconds); a probe that says no costs nothing extra.
-        if (!pol->probed[cls] || retry) { pol->probed[cls] = 1u; return kPathProbe; }
+        if (!pol->probed[cls] || retry || pending) {
+            if (!pending) { pol->word[policy_word(1, cls)] = kWordPending; pol->pending[cls] = 0u; }
+            pol->probed[cls] = 1u;
+            return kPathProbe;
+        }
         return kPathAttempt;
     }
     return bounded ? kPathCluster : wide_or_general();
@@ -442,7 +459,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 411; }
+int rs_version(void) { return 412; }
 
 const char *rs_error_string(int code)
 {
@@ -535,7 +552,7 @@ int rs_policy_create(rs_policy **out)
     if (!pol) return RS_ERR_LAUNCH;
     pol->word = nullptr;
     for (int i = 0; i < kKinds * kClasses; ++i) { pol->away[i] = 0; pol->good[i] = 0; pol->period[i] = kAwayFirst; }
-    for (int i = 0; i < kClasses; ++i) pol->probed[i] = 0;
+    for (int i = 0; i < kClasses; ++i) { pol->probed[i] = 0; pol->pending[i] = 0; }
     if (hipHostMalloc((void **)&pol->word, 64, hipHostMallocDefault) != hipSuccess || !pol->word) {
         delete pol;
         return RS_ERR_LAUNCH;
@@ -556,7 +573,8 @@ int rs_policy_state(const rs_policy *pol, int32_t *state)
 {
     if (!pol || !state) return RS_ERR_NULL;
     const volatile int32_t *w = pol->word;
-    auto any = [&](int kind) { return w[policy_word(kind, 0)] != 0 || w[policy_word(kind, 1)] != 0 || w[policy_word(kind, 2)] != 0; };
+    auto set = [&](int kind, int cls) { const int32_t x = w[policy_word(kind, cls)]; return x != 0 && x != kWordPending; };
+    auto any = [&](int kind) { return set(kind, 0) || set(kind, 1) || set(kind, 2); };
     *state = (any(1) ? 1 : 0) | (any(0) ? 2 : 0) | (any(2) ? 4 : 0);
     return RS_OK;
 }

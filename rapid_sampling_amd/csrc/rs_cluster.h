@@ -18,10 +18,7 @@ struct Slice {
     uint32_t    base4;           // float4 slots of this thread: base4 + j*256, valid while < V4 (a prefix of j)
     int         nv;              // how many of them are inside the row
     uint32_t    kmax_row;        // fkey(max x): of the slice at first, of the row once it is known
-    uint32_t    h_used;          // cluster histograms this row has used and not yet cleared (bit i: rc->h[i]; bit 5: the
-                                 // bins posted ahead, h[1][256..383])
-    uint32_t    guess_t;         // thread t < G: what workgroup t posted in its guess slot (RowCtl::gs)
-    bool        ahead;           // this row's workgroups may have posted the boundary bin's next digit ahead (slice_level1 ran)
+    uint32_t    h_used;          // cluster histograms this row has used and not yet cleared (bit i: rc->h[i])
     bool        mx_posted;       // my slot of the slice maxima is still to be cleared
 };
 
@@ -35,7 +32,7 @@ __device__ __forceinline__ void slice_setup(const Params &p, Slice<R, PEN> &sl, 
     sl.nv = sl.base4 >= V4 ? 0 : (int)min((uint32_t)R, (V4 - sl.base4 + kThreads - 1) / kThreads);
     sl.lrow = logits_row(p, row);
     sl.pn4 = PEN ? reinterpret_cast<float4 *>(p.penalties + (int64_t)row * p.V) : nullptr;
-    sl.h_used = 0u; sl.mx_posted = false; sl.kmax_row = 0u; sl.guess_t = 0u; sl.ahead = false;
+    sl.h_used = 0u; sl.mx_posted = false; sl.kmax_row = 0u;
 }
 
 // This call's 64 random bits of a row, into s.bc64[5] (one thread; the state is advanced once, at
@@ -144,33 +141,6 @@ __device__ __forceinline__ float slice_load(const Params &p, Slice<R, PEN> &sl)
     return lmax;
 }
 
-// The guess slots of a row (RowCtl::gs), read until every workgroup of the row has written its own: thread
-// t < G keeps slot t in sl.guess_t.  posters: how many workgroups posted the next digit of a bin ahead;
-// posted: how many tokens they posted between them -- the count those bins must add up to before anyone
-// reads or clears them.  Returns false when the wait gave up.
-template <int R, bool PEN>
-__device__ __forceinline__ bool read_guesses(const Params &p, Lds &s, Slice<R, PEN> &sl, uint32_t &posters, uint32_t &posted)
-{
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const uint32_t G = sl.G;
-    uint32_t g = 0;
-    SpinGuard guard;
-    guard.start();
-    for (;;) {
-        uint32_t missing = 0;
-        if ((uint32_t)tid < G) { g = a_load(&sl.rc->gs[tid]); missing = g == 0u ? 1u : 0u; }
-        guard.tick(s, p.hdr, 7u);
-        const uint32_t m = block_sum_u32(s, missing, lane, wave);
-        if (m == 0u) break;
-        if (s.abort) return false;
-        if (tid == 0) { s.seen = G - m; s.want = G; }
-    }
-    sl.guess_t = g;
-    const uint32_t both = block_sum_u32(s, (uint32_t)tid < G && g >= 2u ? (1u << 24) + (g >> 12) : 0u, lane, wave);   // at most 64 posters, 2^20 tokens
-    posters = both >> 24; posted = both & 0xFFFFFFu;
-    return true;
-}
-
 // Steps 1b-2 of the cluster path: slice maximum, e in the slice's frame, the level-1 histogram
 // summed over the cluster and brought into the row's frame (s.g the row's, s.hm this slice's),
 // the tokens in the registers re-based to it.  Returns false when a bounded wait gave up.
@@ -234,81 +204,14 @@ __device__ __forceinline__ bool slice_level1(const Params &p, Lds &s, Slice<R, P
     auto clear_used = [&]() {
         for (uint32_t i = 0; i <= (uint32_t)kLevels; ++i)
             if (h_used >> i & 1u) zero_slice(rc->h[i], (i == 0u || i == (uint32_t)kLevels) ? (uint32_t)kNB : 128u, part, G);
-        if (h_used >> 5 & 1u) zero_slice(rc->h[1] + 256, 128u, part, G);
         h_used = 0u;
-        if (mx_posted && tid == 0) { a_store(&rc->mx[part], 0u); a_store(&rc->gs[part], 0u); }
+        if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
         mx_posted = false;
     };
     if (G == 1) {
         if (!hist_combine(s, p.hdr, G, rc->h[0], kNB, (uint32_t)p.V, lane, wave)) return false;
     } else {
-        // This slice's level 1 and its maximum go out first; what follows runs while they travel.
-        __syncthreads();
-        {
-            const uint64_t h0 = s.hm[tid], h1 = s.hm[tid + kThreads];
-            if (h0) a_add(&rc->h[0][tid], h0);
-            if (h1) a_add(&rc->h[0][tid + kThreads], h1);
-        }
-        // Ahead of the next exchange: a flat row's boundary bin holds thousands of tokens, which costs the
-        // cluster a further histogram level -- one more round trip.  A slice that is a fair sample of its
-        // row can tell where the row's boundary will be from its own bins (its share of top_k, top_p of
-        // its own mass); if the bin it finds is too full to be gathered, it posts the next 7 bits of its
-        // tokens in that bin right away, into bins of their own, and says in its slot which bin it meant
-        // and how many tokens it posted.  When the row's boundary is known and every slice meant that bin,
-        // the next level is already there.
-        {
-            if (wave == 0) {
-                uint32_t c3[3]; u128 m3[3];
-                uint32_t cs = 0; u128 ms = 0;
-#pragma unroll
-                for (int i = 0; i < 3; ++i) {
-                    const int idx = (int)kTop1 - 3 * lane - i;
-                    const uint64_t w = idx >= (int)kBin0 ? s.hm[((uint32_t)idx + pos0) & 511u] : 0ull;
-                    c3[i] = pack_count(w);
-                    m3[i] = w ? pack_mass(w, (uint32_t)idx >> 2) : (u128)0;
-                    cs += c3[i]; ms += m3[i];
-                }
-                const u128 mi = wave_inclusive_scan(ms);
-                const uint32_t ci = wave_inclusive_scan(cs);
-                const u128 Ploc = ceil_mul(p.top_p, lane63(mi));
-                const uint64_t kloc = ((uint64_t)p.top_k + G - 1u) / G;
-                uint64_t rcnt = (uint64_t)ci - cs;
-                u128 rm = mi - ms;
-                if (lane == 0) { s.bc32[3] = 0u; s.bc32[4] = 0u; }
-#pragma unroll
-                for (int i = 0; i < 3; ++i) {
-                    const bool before = rcnt >= kloc || rm >= Ploc;
-                    rcnt += c3[i]; rm += m3[i];
-                    if (!before && (rcnt >= kloc || rm >= Ploc)) { s.bc32[3] = kTop1 - (uint32_t)(3 * lane + i); s.bc32[4] = c3[i]; }
-                }
-            }
-            __syncthreads();
-            const uint32_t guess = s.bc32[3], nguess = s.bc32[4];
-            // (a bin that is one tie of the slice's largest token -- rows of equal logits -- is not posted: the
-            // row is recognised as one tie without another level, and counting it would queue every token
-            // of the slice up at one address)
-            const bool post = guess != 0u && (uint64_t)nguess * G > (uint64_t)kCap &&
-                              !bin_is_one_tie(s.hm[(guess + pos0) & 511u], guess, e_bits_of(fkey_inv(kmax_row), Mloc));
-            if (post) {
-                if (tid < 128) s.cand[tid] = 0;
-                __syncthreads();
-#pragma unroll
-                for (int j = 0; j < R; ++j)
-                    if (j < nv) {
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            const uint32_t b = opaque(eb[j * 4 + k]);
-                            if ((b >> 21) == guess)
-                                atomicAdd(reinterpret_cast<unsigned long long *>(&s.cand[(b >> 14) & 127u]), (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
-                        }
-                    }
-                __syncthreads();
-                if (tid < 128) { const uint64_t w = s.cand[tid]; if (w) a_add(&rc->h[1][256 + tid], w); }
-            }
-            if (tid == 0) a_store(&rc->gs[part], post ? (2u + ((guess + pos0) & 511u)) | nguess << 12 : 1u);
-            sl.ahead = true;
-        }
-        const int st = combine_level1(s, p.hdr, G, rc->h[0], rc->mx, (uint32_t)p.V, kmax_row, lane, wave, true);
+        const int st = combine_level1(s, p.hdr, G, rc->h[0], rc->mx, (uint32_t)p.V, kmax_row, lane, wave);
         if (st < 0) return false;
         // the row's frame, and this slice's distance from it
         const float dd = __builtin_floorf(fkey_inv(kmax_row)) - Mloc;
@@ -321,27 +224,7 @@ __device__ __forceinline__ bool slice_level1(const Params &p, Lds &s, Slice<R, P
         }
         if (st == 1) {
             // maxima too far apart for the shared octave positions: level 1 again, in the row's
-            // frame, through the spare histogram.  What was posted ahead is of no use then; the slots
-            // are read before this workgroup publishes again (nobody clears a slot before it has seen
-            // everybody publish again), and the bins posted ahead are complete before they are cleared.
-            uint32_t posters = 0, posted = 0;
-            if (!read_guesses(p, s, sl, posters, posted)) return false;
-            sl.ahead = false;
-            if (posters) {
-                // (before this workgroup publishes again: whoever clears its share of these bins has seen
-                // everybody publish again, hence everybody past this point)
-                SpinGuard guard;
-                guard.start();
-                for (;;) {
-                    const uint32_t c = tid < 128 ? pack_count(a_load(&rc->h[1][256 + tid])) : 0u;
-                    guard.tick(s, p.hdr, 7u);
-                    const uint32_t total = block_sum_u32(s, c, lane, wave);
-                    if (total == posted) break;
-                    if (s.abort) return false;
-                    if (tid == 0) { s.seen = total; s.want = posted; }
-                }
-                h_used |= 1u << 5;
-            }
+            // frame, through the spare histogram
             __syncthreads();
             lds_hist_zero(s, kNB);
             __syncthreads();
@@ -388,9 +271,8 @@ __device__ __forceinline__ bool slice_finish(const Params &p, Lds &s, Slice<R, P
     auto clear_used = [&]() {
         for (uint32_t i = 0; i <= (uint32_t)kLevels; ++i)
             if (h_used >> i & 1u) zero_slice(rc->h[i], (i == 0u || i == (uint32_t)kLevels) ? (uint32_t)kNB : 128u, part, G);
-        if (h_used >> 5 & 1u) zero_slice(rc->h[1] + 256, 128u, part, G);
         h_used = 0u;
-        if (mx_posted && tid == 0) { a_store(&rc->mx[part], 0u); a_store(&rc->gs[part], 0u); }
+        if (mx_posted && tid == 0) a_store(&rc->mx[part], 0u);
         mx_posted = false;
     };
     if (p.e_bits) {
@@ -424,34 +306,6 @@ __device__ __forceinline__ bool slice_finish(const Params &p, Lds &s, Slice<R, P
         const uint32_t emax = e_bits_of(xmax, __builtin_floorf(xmax));
         one_tie = bin_is_one_tie(s.g[f.bin], f.bin, emax);
         if (one_tie) { lo = emax; span = 0u; }
-    }
-    if (G > 1 && sl.ahead) {
-        uint32_t posters = 0, posted = 0;
-        if (!read_guesses(p, s, sl, posters, posted)) return false;
-        if (posters) {
-            h_used |= 1u << 5;                           // those bins are to be cleared with the others
-            // did every workgroup of the row post the next digit of THIS bin?  (position of the bin among
-            // the absolute octaves, as the slices named it)
-            const float Mrow = __builtin_floorf(xmax);
-            const uint32_t m4 = (uint32_t)(int)(Mrow - 128.0f * __builtin_floorf(Mrow * 0.0078125f)) * 4u;
-            const uint32_t want = 2u + ((f.bin - kBin0 + 352u + m4) & 511u);      // 352 = 512 - 160
-            const uint32_t others = block_sum_u32(s, (uint32_t)tid < G && (sl.guess_t & 0xFFFu) != want ? 1u : 0u, lane, wave);
-            const bool use = others == 0u && !one_tie && f.cnt_bin > (uint32_t)kCap && posted == f.cnt_bin;
-            // complete before anyone reads them, and before anyone clears them (the totals go to s.g[0..127],
-            // below the level-1 bins kept there)
-            __syncthreads();
-            if (use && tid < 128) s.hm[tid] = s.cand[tid];       // this slice's own share, counted when it was posted
-            if (!hist_poll(s, p.hdr, rc->h[1] + 256, 128, posted, lane, wave)) return false;
-            if (use) {
-                levels = 2;
-                const uint32_t dsh = level_shift(2u);
-                f = hist_find128(s, s.g, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
-                amass += local_mass_above(s, f.bin, exb, lane, wave);
-                mycnt = pack_count(s.hm[f.bin]);
-                lo |= f.bin << dsh;
-                span = (1u << dsh) - 1u;
-            }
-        }
     }
     while (!one_tie && f.cnt_bin > (uint32_t)kCap && levels < (uint32_t)kLevels) {
         ++levels;

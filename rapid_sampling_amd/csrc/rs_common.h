@@ -64,9 +64,6 @@ struct alignas(256) RowCtl {
     uint32_t verdict;     // one-launch path: 0 pending, sampled token + 1, or kVerdictFallback
     uint32_t pad[3];
     uint32_t mx[kMaxParts];     // per workgroup: fkey(max x of its slice), 0 = not yet written
-    uint32_t gs[kMaxParts];     // per workgroup: 0 not yet written, 1 nothing posted ahead, (2 + p) | n << 12: it posted the next
-                                // digit of its n tokens in the bin at absolute position p, where it expects the row's
-                                // boundary, into h[1][256..383]
     uint64_t A[2 * kMaxParts];  // per workgroup: a 124-bit mass as two words of 62 bits, each | kValid
     uint64_t cand[kCap];        // gathered tokens: bits << 32 | index
     uint64_t h[kLevels + 1][kNB];   // cluster histograms, packed (see kPackOne); one spare for the re-framed level 1
@@ -372,27 +369,6 @@ __device__ __forceinline__ void zero_slice(uint64_t *gh, uint32_t nb, uint32_t p
     for (uint32_t b = lo + threadIdx.x; b < hi; b += kThreads) a_store(&gh[b], (uint64_t)0);
 }
 
-// Read the row's bins (gh) until their counts add up to `expected`; the totals end in s.g.  Returns false
-// when the wait gave up.
-__device__ __forceinline__ bool hist_poll(Lds &s, WsHeader *hdr, const uint64_t *gh, int nb, uint32_t expected, int lane, int wave)
-{
-    SpinGuard guard;
-    guard.start();
-    for (;;) {
-        uint32_t c = 0;
-        for (int b = threadIdx.x; b < nb; b += kThreads) {
-            const uint64_t w = a_load(&gh[b]);
-            s.g[b] = w;
-            c += pack_count(w);
-        }
-        guard.tick(s, hdr, 1u);
-        const uint32_t total = block_sum_u32(s, c, lane, wave);
-        if (total == expected) return true;
-        if (s.abort) return false;
-        if (threadIdx.x == 0) { s.seen = total; s.want = expected; }
-    }
-}
-
 // Sum the workgroup histograms of a cluster: add mine (s.hm, kept) into the
 // row's global bins with one 64-bit atomic per non-empty bin, then read the
 // bins back until their counts add up to `expected` -- count and value of a
@@ -412,7 +388,21 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
         const uint64_t v = s.hm[b];
         if (v) a_add(&gh[b], v);
     }
-    return hist_poll(s, hdr, gh, nb, expected, lane, wave);
+    SpinGuard guard;
+    guard.start();
+    for (;;) {
+        uint32_t c = 0;
+        for (int b = threadIdx.x; b < nb; b += kThreads) {
+            const uint64_t w = a_load(&gh[b]);
+            s.g[b] = w;
+            c += pack_count(w);
+        }
+        guard.tick(s, hdr, 1u);
+        const uint32_t total = block_sum_u32(s, c, lane, wave);
+        if (total == expected) return true;
+        if (s.abort) return false;
+        if (threadIdx.x == 0) { s.seen = total; s.want = expected; }
+    }
 }
 
 // Level 1 of a cluster of several workgroups.  s.hm holds this slice's bins by
@@ -427,17 +417,14 @@ __device__ __forceinline__ bool hist_combine(Lds &s, WsHeader *hdr, uint32_t G, 
 // the slices' maxima lie within 86 octaves of each other.  Returns 0 on
 // success, 1 when they do not (s.g and s.hm are then undefined), -1 when the
 // wait gave up.
-// (`posted`: the caller has already added s.hm to the row's bins, right after its last barrier)
 __device__ __forceinline__ int combine_level1(Lds &s, WsHeader *hdr, uint32_t G, uint64_t *gh, const uint32_t *slots,
-                                              uint32_t expected, uint32_t &kmax_out, int lane, int wave, const bool posted = false)
+                                              uint32_t expected, uint32_t &kmax_out, int lane, int wave)
 {
     const int tid = threadIdx.x;
     __syncthreads();
     const uint64_t h0 = s.hm[tid], h1 = s.hm[tid + kThreads];
-    if (!posted) {
-        if (h0) a_add(&gh[tid], h0);
-        if (h1) a_add(&gh[tid + kThreads], h1);
-    }
+    if (h0) a_add(&gh[tid], h0);
+    if (h1) a_add(&gh[tid + kThreads], h1);
     uint64_t g0, g1;
     uint32_t kmax, kmin;
     SpinGuard guard;

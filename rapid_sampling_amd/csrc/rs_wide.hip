@@ -7,6 +7,15 @@
 
 namespace rs {
 
+// A probe tells the caller's policy itself how it went: rows whose kept sets would not have fitted the
+// stashes set the report word as they are found (wide_finish_row); if there was none, this one thread,
+// behind the finish in stream order, clears the word, which the host set to "pending" with the call.
+__global__ void probe_done_kernel(const Params p)
+{
+    if (threadIdx.x == 0 && a_load(&p.hdr->n_need) == 0u)
+        __hip_atomic_store(p.host_words + p.report, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v)
 {
     const dim3 sgrid(B * v.G), sblock(kThreads);
@@ -24,6 +33,7 @@ hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds
     else RS_WIDE(kStreamLongR, kStreamLongLog2);
 #undef RS_WIDE
 #undef RS_WIDE_DT
+    if (p.probe && p.host_words) hipLaunchKernelGGL(probe_done_kernel, dim3(1), dim3(kWave), 0, st, p);
     return hipGetLastError();
 }
 

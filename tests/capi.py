@@ -201,6 +201,7 @@ class Sampler:
             return res
         if not sync:
             res["out_dev"] = out
+            res["diag_dev"] = diag
             return res
         torch.cuda.synchronize()
         res["out"] = out.cpu().numpy()

@@ -507,14 +507,12 @@ def test_cluster_levels_with_slices_that_hold_no_boundary_tokens(torch_cuda, ora
             _run_case(torch_cuda, oracle, capi, lg, t, k, p, u_np=u, what="contiguous ties k=%s p=%s T=%s #%d" % (k, p, t, rep))
 
 
-def test_cluster_bins_posted_ahead_when_frames_lie_far_apart(torch_cuda, oracle):
-    """The general kernel's workgroups post the next digit of the bin in which they expect the row's
-    boundary ahead of the first exchange.  Rows whose slices lie in frames too far apart (whole slices
-    masked) make no use of that, redo level 1 and clear everything early: the bins posted ahead must be
-    complete, and read by nobody any more, before a workgroup clears its share of them (a workgroup that
-    cleared while others were still adding them up left those waiting until they gave up, now and then).
-    Flat rows, whose slices all post and agree, and sorted rows, whose slices post different bins, beside
-    them; every call against the oracle, a dozen calls on one workspace."""
+def test_cluster_rows_whose_slices_lie_in_frames_far_apart_beside_flat_ones(torch_cuda, oracle):
+    """General kernel, a dozen calls on one workspace: rows whose slices lie in frames too far apart for
+    the shared octave positions (whole slices masked), which redo level 1 in the row's frame and clear
+    the first histogram early, beside flat rows, whose boundary bin takes a further level over the
+    cluster, and sorted rows, whose slices hold different bins.  Every call against the oracle; the
+    workspace must stay clean from call to call."""
     torch = torch_cuda
     from tests import capi
     B, V = 12, 266240
@@ -534,7 +532,7 @@ def test_cluster_bins_posted_ahead_when_frames_lie_far_apart(torch_cuda, oracle)
         ref_out, ref_diag = oracle.sample_batch(lg, c, kk, pp, injected_u=u_np)
         for it in range(4):
             res = smp.sample(L, c, kk, pp, uniforms=U, path="cluster")
-            _check(res, ref_out, ref_diag, "posted ahead, T=%g k=%d p=%g call %d" % (t, k, p, it))
+            _check(res, ref_out, ref_diag, "frames far apart, T=%g k=%d p=%g call %d" % (t, k, p, it))
             assert smp.status() == 0
 
 
@@ -1230,6 +1228,48 @@ def test_routing_is_kept_per_kind_and_size_of_call(torch_cuda, oracle):
     assert sum(1 for r in flat_rounds if r == 7) <= 3                  # the probe, and one or two retries (64, 128 calls later)
     assert smp.policy_state() == 1 and smp.status() == 0
     smp.close()
+
+
+def test_calls_issued_behind_a_probe_that_has_not_run_yet_are_probes_too(torch_cuda, oracle):
+    """A caller that does not synchronise between calls issues many before the first has run.  The first
+    call without a bounding top_k on a policy is a probe, and its report word is pending until it has run:
+    the calls issued in the meantime are probes as well (diag.rounds == 7), not attempts that would do
+    their flat rows the slow way (diag.rounds == 8).  Once the probe has run, its verdict routes the
+    calls: flat rows to the general kernel, peaked rows to the streaming path.  A dozen calls queued
+    behind a kernel that keeps the GPU busy while they are issued, flat rows and peaked ones."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 8, 131072
+    flat = H.logits_uniform(B, V, seed=190)
+    peaked = H.logits_normal(B, V, 3.0, seed=191)
+    u_np = H.uniforms(B, 192)
+    rc, c, k, p = capi.normalize(1.0, -1, 0.4, V, B, 1)
+    u = torch.from_numpy(u_np).cuda()
+    for name, rows in (("flat", flat), ("peaked", peaked)):
+        ref_out, ref_diag = oracle.sample_batch(rows, c, k, p, injected_u=u_np)
+        lg = torch.from_numpy(rows).cuda()
+        smp = capi.Sampler(B, V, with_policy=True, init=True)
+        torch.cuda.synchronize()
+        torch.cuda._sleep(40_000_000)                    # some 20 ms: the calls below are all issued before the first runs
+        calls = [smp.sample(lg, c, k, p, uniforms=u, sync=False) for _ in range(12)]
+        torch.cuda.synchronize()
+        rounds = []
+        for i, res in enumerate(calls):
+            assert res["rc"] == 0
+            out = res["out_dev"].cpu().numpy()
+            diag = res["diag_dev"].cpu().numpy().view(capi.DIAG_DTYPE).reshape(B)
+            _check({"rc": 0, "out": out, "diag": diag}, ref_out, ref_diag, "%s rows, queued call %d" % (name, i))
+            rounds.append(sorted(set(diag["rounds"].tolist())))
+        assert rounds[0] == [7] and all(r != [8] and 8 not in r for r in rounds), (name, rounds)
+        # the probe has run: its verdict stands
+        res = smp.sample(lg, c, k, p, uniforms=u)
+        _check(res, ref_out, ref_diag, "%s rows, after the queue" % name)
+        if name == "flat":
+            assert smp.policy_state() == 1 and (res["diag"]["rounds"] >= 1).all() and (res["diag"]["rounds"] < 7).all()
+        else:
+            assert smp.policy_state() == 0 and (res["diag"]["rounds"] == 0).all()
+        assert smp.status() == 0
+        smp.close()
 
 
 def test_two_streams_two_workspaces_concurrently(torch_cuda, oracle):
