@@ -296,6 +296,7 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
 #define RS_PATH_ATTEMPT 3
 #define RS_PATH_FUSED   4
 #define RS_PATH_WIDE    5
+#define RS_PATH_WIDE1   6
 typedef struct rs_options {
     int32_t    path;
     int32_t    slice_r;

@@ -295,7 +295,7 @@ static size_t stream_bytes(int32_t B, int32_t V)
 // word is taken to be clear.
 constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u, kPendingMost = 64u;
 constexpr int32_t kWordPending = 2;
-constexpr int kKinds = 3, kClasses = 3;
+constexpr int kKinds = 4, kClasses = 3;
 struct rs_policy {
     int32_t *word;
     uint32_t away[kKinds * kClasses], period[kKinds * kClasses], good[kKinds * kClasses];
@@ -329,7 +329,7 @@ namespace rs {
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
-enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5, kPathProbe = 6 };
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5, kPathProbe = 6, kPathWide1 = 7 };
 // The wide path (four launches, two reads of the logits) against the general kernel (one launch, its
 // exchanges), measured on flat rows (U[0,1), top_p 0.9) and on N(0,1.5) with top_k 10000: the wide path
 // wins from about 25 million tokens per call on in rows of 50304 tokens and more (96 x 262144: 88 against
@@ -339,6 +339,13 @@ enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPat
 // in short rows (2048 x 32768: 225 against 193).
 constexpr uint64_t kWideMin = 3ull << 23;
 constexpr int32_t kWideMinV = 49152;
+// The one-pass wide path (a sample of the row, then one pass over all of it) against the two-pass one,
+// same rows: up to about 2^26 tokens per call the second pass of the two-pass path comes out of the
+// Infinity Cache and the two are level (256 x 131072: 91 against 101 us and 87 against 84; 512 x 65536: 105
+// against 106 and 103 against 91); from there on the one pass wins (256 x 262144: 134 against 154 and 123
+// against 129; 512 x 262144: 228 against 290 and 211 against 231; 128 x 1048576: 233 against 263 and 192
+// against 226).
+constexpr uint64_t kWide1Min = 1ull << 26;
 constexpr uint64_t kPenStreamMin = 1ull << 23;
 // Plain temperature sampling (top_k = V, top_p = 1: every live token is kept) has no kept set to
 // stash, but the streaming pass's bins alone say which slice holds the target: one pass at
@@ -416,6 +423,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (force == RS_PATH_STREAM) return bounded ? kPathStream : kPathCluster;
     if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
     if (force == RS_PATH_WIDE) return keep_all ? kPathKeep : kPathWide;
+    if (force == RS_PATH_WIDE1) return keep_all ? kPathKeep : kPathWide1;
     // Small calls: rows of fewer than 8192 tokens are one or two workgroups of the general kernel each, with
     // few or no exchanges (8.5 us for a row of 256 tokens); from 8192 tokens per row on the streaming
     // path's two launches are faster whatever the batch (one row of 8192 to 100256 tokens: 13.6-14.7
@@ -424,7 +432,14 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (keep_all && V >= 32768) return kPathKeep;              // shorter rows: one workgroup of the general kernel does a row in one go
     // kept sets the stashes cannot hold: the wide path from kWideMin tokens on, unless its rows have been
     // going the slow way (slices that are no fair samples of their rows, ties of thousands of tokens)
-    auto wide_or_general = [&]() { return (uint64_t)B * (uint64_t)V >= kWideMin && V >= kWideMinV && !routed_away(2) ? kPathWide : kPathCluster; };
+    // (the one-pass wide path first; when its rows have been going the slow way -- samples that are no fair
+    // picture of their rows -- the two-pass one, which counts everything; then the general kernel)
+    auto wide_or_general = [&]() {
+        const uint64_t tokens = (uint64_t)B * (uint64_t)V;
+        if (tokens >= kWide1Min && V >= kWideMinV && !routed_away(2)) return (int)kPathWide1;
+        if (tokens >= kWideMin && V >= kWideMinV && !routed_away(3)) return (int)kPathWide;
+        return (int)kPathCluster;
+    };
     if (!bounded && !(top_p < 1.0f)) return wide_or_general(); // a top_k of thousands and no nucleus: more than the stashes hold
     if (!pol) return bounded ? kPathStream : wide_or_general();
     if (!routed_away(bounded ? 0 : 1)) {
@@ -575,7 +590,7 @@ int rs_policy_state(const rs_policy *pol, int32_t *state)
     const volatile int32_t *w = pol->word;
     auto set = [&](int kind, int cls) { const int32_t x = w[policy_word(kind, cls)]; return x != 0 && x != kWordPending; };
     auto any = [&](int kind) { return set(kind, 0) || set(kind, 1) || set(kind, 2); };
-    *state = (any(1) ? 1 : 0) | (any(0) ? 2 : 0) | (any(2) ? 4 : 0);
+    *state = (any(1) ? 1 : 0) | (any(0) ? 2 : 0) | (any(2) ? 4 : 0) | (any(3) ? 8 : 0);
     return RS_OK;
 }
 
@@ -631,7 +646,7 @@ static int check_call(const void *logits, int32_t logits_dtype, int64_t row_stri
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
     if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
-    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_WIDE || opt->slice_r < 0)) return RS_ERR_ARG;
+    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_WIDE1 || opt->slice_r < 0)) return RS_ERR_ARG;
     if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
         return RS_ERR_ALIGN;
     return RS_OK;
@@ -719,7 +734,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
         // with static LDS alone -- with a 64 KB list in dynamic LDS it was 32 x 1, and rows of 33 and
         // more slices could, rarely, starve until their waits gave up.
         if (path == kPathFused) v.list_cap = 2048u;
-        const int kind = path == kPathAttempt || path == kPathProbe ? 1 : path == kPathWide ? 2 : 0;
+        const int kind = path == kPathAttempt || path == kPathProbe ? 1 : path == kPathWide1 ? 2 : path == kPathWide ? 3 : 0;
         p.report = path == kPathKeep ? 0u : (uint32_t)policy_word(kind, size_class(B, V));
         p.attempt = path == kPathAttempt ? 1u : 0u;
         p.probe = path == kPathProbe ? 1u : 0u;
@@ -728,6 +743,10 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
             // the list holds the tokens of ONE sub-bin of the boundary bin: 1/128 of it for a smooth distribution
             p.stash_k = 1u; v.list_cap = 4096u;
             return launch_wide(sr, logits_dtype, (uint32_t)B, (size_t)v.list_cap * sizeof(uint64_t), st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
+        }
+        if (path == kPathWide1) {
+            p.stash_k = 1u; v.list_cap = 4096u;
+            return launch_wide1(sr, logits_dtype, (uint32_t)B, (size_t)v.list_cap * sizeof(uint64_t), st, p, v) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
         }
         const size_t dyn = (size_t)v.list_cap * sizeof(uint64_t);
         if (path == kPathFused)

@@ -680,5 +680,6 @@ hipError_t launch_stream(int slice_r, int32_t dtype, bool keep, uint32_t B, size
                          const StreamView &v);
 hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v);
 hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
+hipError_t launch_wide1(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
 
 }  // namespace rs

@@ -394,7 +394,8 @@ void force_path(const std::string &name)
     else if (name == "attempt") g_forced_path = RS_PATH_ATTEMPT;
     else if (name == "fused") g_forced_path = RS_PATH_FUSED;
     else if (name == "wide") g_forced_path = RS_PATH_WIDE;
-    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused | wide");
+    else if (name == "wide1") g_forced_path = RS_PATH_WIDE1;
+    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused | wide | wide1");
 }
 
 // The workspace tensor of the current stream (tests poison it to force the error path).

@@ -74,11 +74,11 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     # Every way through the library on this one workspace: the general kernel alone, the wait-free
     # streaming path (taken for top_k <= 1024; rows it cannot finish go on to the general kernel), the
     # same attempted whatever top_k is, the one-launch path (streaming pass and finish in one kernel,
-    # falling back inside the kernel), the wide path (two passes over the logits and a finish, for kept
-    # sets of any size), then the general kernel again on the workspace these leave
+    # falling back inside the kernel), the wide paths (two passes over the logits and a finish, for kept
+    # sets of any size; one pass behind a sample of the row), then the general kernel again on the workspace these leave
     # behind.  All but the general kernel also return the e of every token: the kept set on that path.
     # With penalties: the one-launch path and the general kernel.
-    paths = ("cluster", "stream", "optimistic", "fused", "wide", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
+    paths = ("cluster", "stream", "optimistic", "fused", "wide", "wide1", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
     for path in paths:
         pen3 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
         res3 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen3, presence=presence, repetition=repetition, decay=decay,
@@ -306,8 +306,9 @@ def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
     0.9 on flat generators, /root/reference/bench.py:34-35, :66-72; its search costs the same whatever the
     kept set, sampling.cu:261-329): 512 flat rows of 262144 tokens under top_p 0.9, the bandwidth
     configuration's 128 rows of a million tokens with top_k 10000, 768 flat rows of 50304 tokens.  The
-    library takes the wide path for them by itself (diag.rounds == 7 for every row: none done the slow
-    way); every row goes through the oracle, and the general kernel must agree in every field."""
+    library takes a wide path for them by itself -- the one-pass one from 2^26 tokens per call on
+    (diag.rounds == 9), the two-pass one below (7), every row: none done the slow way; every row goes
+    through the oracle, and the general kernel and both wide paths must agree in every field."""
     torch = torch_cuda
     from tests import capi
     g = torch.Generator(device="cuda")
@@ -319,17 +320,20 @@ def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
     u = torch.from_numpy(u_np).cuda()
     smp = capi.Sampler(B, V)
     res = {}
-    for path in ("auto", "cluster", "wide"):
+    for path in ("auto", "cluster", "wide", "wide1"):
         print("wide at scale", B, T, V, path, flush=True)
         r = smp.sample(lg, c, k, p, uniforms=u, path=path)
         assert r["rc"] == 0 and smp.status() == 0
         res[path] = r
-    assert (res["auto"]["diag"]["rounds"] == 7).all(), np.unique(res["auto"]["diag"]["rounds"], return_counts=True)
+    auto_rounds = 9 if B * V >= 2 ** 26 else 7
+    assert (res["auto"]["diag"]["rounds"] == auto_rounds).all(), np.unique(res["auto"]["diag"]["rounds"], return_counts=True)
     assert (res["wide"]["diag"]["rounds"] == 7).all()
+    assert (res["wide1"]["diag"]["rounds"] == 9).all(), np.unique(res["wide1"]["diag"]["rounds"], return_counts=True)
     assert (res["cluster"]["diag"]["rounds"] < 7).all()
     for f in FIELDS:
         assert np.array_equal(res["auto"]["diag"][f], res["cluster"]["diag"][f]), f
         assert np.array_equal(res["auto"]["diag"][f], res["wide"]["diag"][f]), f
+        assert np.array_equal(res["auto"]["diag"][f], res["wide1"]["diag"][f]), f
     assert np.array_equal(res["auto"]["out"], res["cluster"]["out"])
     d = res["auto"]["diag"]
     step = 64 if V <= 262144 else 32
@@ -368,12 +372,19 @@ def test_wide_path_unusual_rows(torch_cuda, oracle):
     assert rounds[0] == 7 and rounds[4] == 7 and rounds[6] == 7 and rounds[7] == 7, rounds
     assert rounds[1] == 8 and rounds[2] == 8, rounds                # sorted rows: the slow way
     assert rounds[5] == 0, rounds                                   # one tie of all tokens: finished from the row's bins
+    # The one-pass wide path: its sample is taken from all over the row and its window is a range of values,
+    # so a sorted row is finished there when the one slice that holds the tokens around the threshold
+    # can set all of them aside; rows of a few distinct values put thousands of ties into one sub-bin.
+    res = capi.Sampler(8, V).sample(torch.from_numpy(lg).cuda(), c, k, p, path="wide1", uniforms=torch.from_numpy(H.uniforms(8, 61)).cuda())
+    rounds = res["diag"]["rounds"]
+    assert rounds[0] == 9 and rounds[4] == 9 and rounds[6] == 9 and rounds[7] == 9, rounds
+    assert rounds[1] in (8, 9) and rounds[2] in (8, 9) and rounds[3] == 8 and rounds[5] == 0, rounds
 
 
 def test_wide_path_reports_slow_rows(torch_cuda, oracle):
-    """Calls on the wide path that are given a policy report rows done the slow way in a word of their own
-    (rs_policy_state bit 2): the next calls of that kind take the general kernel, the wide path is tried
-    again after 64 of them, and a call that goes well clears the word through the call after it."""
+    """Calls on the two-pass wide path that are given a policy report rows done the slow way in a word of
+    their own (rs_policy_state bit 3): the next calls of that kind take the general kernel, the wide path is
+    tried again after 64 of them, and a call that goes well clears the word through the call after it."""
     torch = torch_cuda
     from tests import capi
     B, V = 300, 131072
@@ -394,17 +405,64 @@ def test_wide_path_reports_slow_rows(torch_cuda, oracle):
     assert (res["diag"]["rounds"] == 7).all() and smp.policy_state() == 0
     res = smp.sample(lg_bad, c, k, p, uniforms=u)
     _check(res, *ref_bad, "wide, one sorted row")
-    assert res["diag"]["rounds"][11] == 8 and (np.delete(res["diag"]["rounds"], 11) == 7).all() and smp.policy_state() == 4
+    assert res["diag"]["rounds"][11] == 8 and (np.delete(res["diag"]["rounds"], 11) == 7).all() and smp.policy_state() == 8
     for i in range(3):
         res = smp.sample(lg_good, c, k, p, uniforms=u)
         _check(res, *ref_good, "after a slow row %d" % i)
-        assert (res["diag"]["rounds"] < 7).all() and smp.policy_state() == 4       # general kernel
+        assert (res["diag"]["rounds"] < 7).all() and smp.policy_state() == 8       # general kernel
     for i in range(64):
         res = smp.sample(lg_good, c, k, p, uniforms=u, want_diag=False)
         assert res["rc"] == 0 and np.array_equal(res["out"], ref_good[0])
     assert smp.policy_state() == 0
     res = smp.sample(lg_good, c, k, p, uniforms=u)
     assert (res["diag"]["rounds"] == 7).all() and smp.policy_state() == 0 and smp.status() == 0
+    smp.close()
+
+
+def test_one_pass_wide_path_hands_over_to_the_two_pass_one(torch_cuda, oracle):
+    """From 2^26 tokens per call on, kept sets of thousands of tokens take the one-pass wide path (a sample of
+    each row decides what the one pass over it counts finely and sets aside; diag.rounds == 9).  A row of
+    which the sample is no fair picture (its 30000 largest tokens all lie in stretches the sample does not
+    look at, so the threshold is nowhere near where the sample expects it) is done the slow way (8) and
+    reported in a word of that path's own (rs_policy_state bit 2); the next calls take the two-pass wide
+    path (7), which counts everything, the one-pass path is tried again after 64 of them, and a call
+    that goes well clears the word through the call after it.  Every result equals the oracle's."""
+    torch = torch_cuda
+    from tests import capi
+    B, V = 72, 1048576
+    rng = np.random.default_rng(171)
+    good = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
+    rc, c, k, p = capi.normalize(1.0, 20000, 1.0, V, B, 1)
+    u_np = H.uniforms(B, 172)
+    u = torch.from_numpy(u_np).cuda()
+    ref_good = oracle.sample_batch(good, c, k, p, injected_u=u_np)
+    # the sample of a row of 2^20 tokens: 256 tokens out of every 8192, from the middle of the stretch
+    odd_row = good[11].copy()
+    odd_row.reshape(-1, 8192)[:, :256] += np.float32(8.0)
+    ref_odd = oracle.sample_batch(odd_row[None, :], c, k, p, injected_u=u_np[11:12])
+    ref_bad = (ref_good[0].copy(), ref_good[1].copy())
+    ref_bad[0][11] = ref_odd[0][0]
+    ref_bad[1][11] = ref_odd[1][0]
+    lg_good = torch.from_numpy(good).cuda()
+    lg_bad = lg_good.clone()
+    lg_bad[11] = torch.from_numpy(odd_row).cuda()
+    smp = capi.Sampler(B, V, with_policy=True, init=True)
+    res = smp.sample(lg_good, c, k, p, uniforms=u)
+    _check(res, *ref_good, "one pass, fair rows")
+    assert (res["diag"]["rounds"] == 9).all() and smp.policy_state() == 0
+    res = smp.sample(lg_bad, c, k, p, uniforms=u)
+    _check(res, *ref_bad, "one pass, one row the sample misjudges")
+    assert res["diag"]["rounds"][11] == 8 and (np.delete(res["diag"]["rounds"], 11) == 9).all() and smp.policy_state() == 4
+    for i in range(3):
+        res = smp.sample(lg_good, c, k, p, uniforms=u)
+        _check(res, *ref_good, "after a slow row %d" % i)
+        assert (res["diag"]["rounds"] == 7).all() and smp.policy_state() == 4      # the two-pass wide path
+    for i in range(64):
+        res = smp.sample(lg_good, c, k, p, uniforms=u, want_diag=False)
+        assert res["rc"] == 0 and np.array_equal(res["out"], ref_good[0])
+    assert smp.policy_state() == 0
+    res = smp.sample(lg_good, c, k, p, uniforms=u)
+    assert (res["diag"]["rounds"] == 9).all() and smp.policy_state() == 0 and smp.status() == 0
     smp.close()
 
 
