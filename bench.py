@@ -338,9 +338,10 @@ def main():
                     "rs::stream_pen_kernel (reads both, writes the decayed penalties), rs::finish_kernel (patches the sampled "
                     "tokens), rs::penalty_fix_kernel (slices the pass deferred: none here); algorithmic bytes 12*V per row"}
         del pen_b, last
-        # kept sets of thousands of tokens (the wide path: counting pass, plan, second pass around the
-        # boundary bin, finish -- the logits are read twice): the same rows with top_k 10000, and 512 flat
-        # rows of 262144 tokens with a nucleus of 0.9
+        # kept sets of thousands of tokens (calls of this size take the one-pass wide path: a look at a sample of
+        # each row, one pass over the logits, a finish per row): the same rows with top_k 10000, and 512 flat
+        # rows of 262144 tokens with a nucleus of 0.9; beside them the two-pass wide path (counting pass, plan,
+        # second pass around the boundary bin, finish) and the general kernel
         def call_wide_k():
             return sample.batch_sampling_temperature_topk_topp(big, st_b, 1.0, 10000, 1.0)
 
@@ -348,6 +349,8 @@ def main():
         sample._sample.force_path("cluster")
         try:
             t_wk_cluster = block_time_us(torch, call_wide_k, 2, 1)
+            sample._sample.force_path("wide")
+            t_wk_two = block_time_us(torch, call_wide_k, max(2, args.bandwidth_steps // 2), 2)
         finally:
             sample._sample.force_path("auto")
         flat_rows = torch.rand((512, 262144), generator=g, device=dev)
@@ -357,16 +360,24 @@ def main():
             return sample.batch_sampling_temperature_topk_topp(flat_rows, st_w, 1.0, -1, 0.9)
 
         t_wp = block_time_us(torch, call_wide_p, max(2, args.bandwidth_steps // 2), 3)
+        sample._sample.force_path("wide")
+        try:
+            t_wp_two = block_time_us(torch, call_wide_p, max(2, args.bandwidth_steps // 2), 2)
+        finally:
+            sample._sample.force_path("auto")
         result["roofline"]["wide_kept_sets"] = {
             "top_k_10000": {"us_per_call": round(t_wk, 2), "achieved": round(bytes_btv / (t_wk * 1e-6) / 1e9, 1),
                             "frac": round(bytes_btv / (t_wk * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                            "two_pass_us_per_call": round(t_wk_two, 2),
                             "cluster_path_us_per_call": round(t_wk_cluster, 2)},
             "flat_512x262144_top_p_0.9": {"us_per_call": round(t_wp, 2),
                                           "achieved": round(512 * 262144 * 4 / (t_wp * 1e-6) / 1e9, 1),
-                                          "frac": round(512 * 262144 * 4 / (t_wp * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
-            "note": "four launches: rs::stream_kernel (counting only), rs::wide_plan_kernel, rs::wide_kernel (reads the "
-                    "logits a second time), rs::wide_finish_kernel; achieved = algorithmic bytes 4*V per row / time of the "
-                    "whole call, although the path reads 8*V per row"}
+                                          "frac": round(512 * 262144 * 4 / (t_wp * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                          "two_pass_us_per_call": round(t_wp_two, 2)},
+            "note": "one-pass wide path, three launches: rs::wide_sample_kernel (a sample of each row, 32768 tokens at "
+                    "most), rs::wide1_kernel (the pass over the logits), rs::wide1_finish_kernel; two_pass: "
+                    "rs::stream_kernel (counting only), rs::wide_plan_kernel, rs::wide_kernel (reads the logits a second "
+                    "time), rs::wide_finish_kernel; achieved = algorithmic bytes 4*V per row / time of the whole call"}
         del flat_rows
         if args.traffic_probe:
             src = big.view(-1)[: Bb * Vb]

@@ -148,17 +148,22 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * tokens with a bounding top_k counts a row as slow when its stashes hold
  * more tokens than the finishing workgroup's list and have to be gone through
  * twice more -- flat rows cut into many slices -- for the same reason).  The
- * wide path (kept sets of any size, two passes over the logits) does a row the
- * slow way when its slices are no fair samples of the row.  Calls that are
+ * two-pass wide path (kept sets of any size, two passes over the logits) does a
+ * row the slow way when its slices are no fair samples of the row; the one-pass
+ * wide path (a sample of the row, then one pass over all of it; calls of at
+ * least 2^26 tokens) when the sample is no fair picture of the row (a few
+ * tokens that carry most of the mass under top_p).  Calls that are
  * given a policy report "a row went the slow way: yes/no" to a word of pinned
  * host memory inside it (yes at once, no by the next call on the workspace),
  * and rs_sample_ex reads that word, without waiting, before it routes the
  * next call: while it is set, calls of that kind go to the general kernel (a
- * call without a bounding top_k to the wide path when it is large enough);
+ * call without a bounding top_k to a wide path when it is large enough, a call
+ * that would take the one-pass wide path to the two-pass one);
  * after 64 of them the path is tried again, each try that fails doubles that
  * number (up to 1024), and a run of good calls as long as the last stay away
  * puts it back to 64.  There is a word per KIND of call -- streaming with a
- * bounding top_k, streaming without, wide -- and per SIZE CLASS (tokens per
+ * bounding top_k, streaming without, one-pass wide, two-pass wide -- and per
+ * SIZE CLASS (tokens per
  * call below 2^20, below 2^24, from 2^24 on), so that workloads that share a
  * policy do not flip each other's route.  The first call without a bounding
  * top_k of a size class, and every such call that tries again after a stay
@@ -181,7 +186,9 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * given the policy has completed on the device.
  * rs_policy_state (over all size classes): bit 0 set: calls without a bounding
  * top_k currently leave the streaming path, bit 1 set: so do calls with one,
- * bit 2 set: calls that would take the wide path take the general kernel.
+ * bit 2 set: calls that would take the one-pass wide path take the two-pass
+ * one, bit 3 set: calls that would take the two-pass wide path take the
+ * general kernel.
  * rs_policy_error: *error = RS_OK or RS_ERR_DEVICE as last reported; with
  * clear != 0 the word is reset.
  */
@@ -232,10 +239,15 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  * finish; see rs_policy; plain temperature sampling -- top_k = V, top_p = 1,
  * every token kept -- takes these two launches as well: the pass only counts,
  * and the finish reads one slice of the row again), four for kept sets of
- * thousands of tokens in calls of at least 3 * 2^23 tokens (the wide path: the
- * counting pass, a one-workgroup-per-row plan, a second pass over the logits
- * that counts the boundary bin's next digit and sets the tokens around the
- * expected threshold aside, a per-row finish), or three for calls of at least
+ * thousands of tokens in calls of at least 3 * 2^23 tokens (the two-pass wide
+ * path: the counting pass, a one-workgroup-per-row plan, a second pass over
+ * the logits that counts the boundary bin's next digit and sets the tokens
+ * around the expected threshold aside, a per-row finish), three for the same
+ * from 2^26 tokens on (the one-pass wide path: a one-workgroup-per-row look at
+ * a sample of the row, an eighth of it at most, one pass over the logits that
+ * counts the row's bins and, finely, the range in which the sample expects the
+ * threshold, and sets the tokens around it aside, a per-row finish that checks
+ * the guess against the exact counts), or three for calls of at least
  * 2^23 tokens with penalties and top_k <= 1024 (a pass over logits and
  * penalties that also writes the decayed penalties, the finish, which patches
  * the sampled tokens' penalties, and a fix-up kernel for slices the pass left
@@ -284,9 +296,9 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
  * RS_PATH_ATTEMPT the streaming path whatever top_k is (penalties take the
  * general kernel on these three), RS_PATH_FUSED the streaming pass and the
  * finish in one launch (any call whose rows span at least two slices, with or
- * without penalties; else the general kernel), RS_PATH_WIDE the wide path (any
- * call without penalties; a call that keeps every token takes the counting-only
- * streaming variant).  `slice_r` forces the float4 groups per thread of the
+ * without penalties; else the general kernel), RS_PATH_WIDE the two-pass wide
+ * path and RS_PATH_WIDE1 the one-pass wide path (any call without penalties; a
+ * call that keeps every token takes the counting-only streaming variant).  `slice_r` forces the float4 groups per thread of the
  * general kernel (1, 2, 4, 8, 16 or 32; 0 = chosen by the library).
  * `policy` see rs_policy.  No counterpart in the reference.
  */

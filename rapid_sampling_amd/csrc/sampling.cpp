@@ -334,8 +334,9 @@ int64_t workspace_status(std::optional<int64_t> device)
 }
 
 // Routing state of the current stream's workspace (rs_policy_state): bit 0 set: calls without a
-// bounding top_k currently take the general kernel (or the wide path), bit 1 set: calls with one take the
-// general kernel, bit 2 set: calls that would take the wide path take the general kernel.  -1: no workspace yet.
+// bounding top_k currently take the general kernel (or a wide path), bit 1 set: calls with one take the
+// general kernel, bit 2 set: calls that would take the one-pass wide path take the two-pass one, bit 3 set:
+// calls that would take the two-pass wide path take the general kernel.  -1: no workspace yet.
 int64_t policy_state(std::optional<int64_t> device)
 {
     const auto dev = at::Device(at::kCUDA, (c10::DeviceIndex)(device ? *device : c10::hip::current_device()));
