@@ -438,17 +438,16 @@ __global__ void __launch_bounds__(kThreads, (R <= 8 ? 5 : RS_STREAM_WAVES)) wide
     const uint32_t win_lo = s.win_lo, win_hi = s.win_hi, n = s.n;
     if (n != 0u) {
         const uint32_t rel = (127u - exb_top) << 23;     // bit patterns as if the range's top octave were [1, 2)
+        // the window as bit patterns: one comparison per token
+        const uint32_t w_lo = max(lo_bits + (win_lo << sh), lo_live), w_width = lo_bits + ((win_hi + 1u) << sh) - w_lo;
 #pragma unroll
         for (int j = 0; j < R; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const uint32_t b = eb[j * 4 + q];
-                if (b - lo_live < width) {
-                    const uint32_t sb = (b - lo_bits) >> sh;
-                    if (sb >= win_lo && sb <= win_hi) {
-                        const uint32_t slot = atomicAdd(&s.off[sb], 1u);
-                        if (slot < (uint32_t)kW1Cap) s.stage[slot] = ((uint64_t)(b + rel) << 32) | ((base4 + (uint32_t)j * NT) * 4u + (uint32_t)q);
-                    }
+                if (b - w_lo < w_width) {
+                    const uint32_t slot = atomicAdd(&s.off[(b - lo_bits) >> sh], 1u);
+                    if (slot < (uint32_t)kW1Cap) s.stage[slot] = ((uint64_t)(b + rel) << 32) | ((base4 + (uint32_t)j * NT) * 4u + (uint32_t)q);
                 }
             }
     }
