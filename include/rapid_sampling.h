@@ -172,7 +172,8 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * (more than 512 tokens?) would have fitted the streaming path's stashes --
  * so a workload of flat rows never pays for a row done the slow way.  A probe
  * reports on itself when it has run; until then its word is pending and calls
- * of its kind and size class are probes too (at most 64 of them), so a caller
+ * of its kind and size class are probes too (at most 64 of them, then they stay
+ * away as after a slow row), so a caller
  * that issues many calls without synchronising does not run attempts on rows
  * nobody has looked at yet.  Without
  * a policy, calls with a bounding top_k always stream and calls without never

@@ -292,7 +292,8 @@ static size_t stream_bytes(int32_t B, int32_t V)
 // A probe's word is "pending" (kWordPending, set by the host with the call) until the probe has run: calls of
 // its kind issued in the meantime -- a caller that does not synchronise between calls issues many -- are
 // probes too, not attempts that may have to do their rows the slow way; after kPendingMost of them the
-// word is taken to be clear.
+// calls stay away as after a slow row, and the try after that is a probe again (which leaves the word set
+// until it has run).
 constexpr uint32_t kAwayFirst = 64u, kAwayMost = 1024u, kPendingMost = 64u;
 constexpr int32_t kWordPending = 2;
 constexpr int kKinds = 4, kClasses = 3;
@@ -398,7 +399,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         volatile int32_t *word = pol->word + policy_word(kind, cls);
         if (*word == kWordPending) {
             if (++pol->pending[cls] <= kPendingMost) { pending = true; return false; }
-            *word = 0;
+            *word = 1;                                        // no word of the probe yet: away for now, the retry is a probe again
         }
         if (*word == 0) {
             if (pol->period[slot] > kAwayFirst && ++pol->good[slot] >= pol->period[slot]) pol->period[slot] = kAwayFirst;
@@ -449,8 +450,9 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         // the wide path -- whose time does not depend on the kept set -- and its finishing workgroups report
         // whether the rows' kept sets would have fitted the stashes.  An attempt that fails costs a pass
         // of one workgroup over the row (hundreds of microseconds); a probe that says no costs nothing extra.
+        // (a retry leaves the word set while its probe is under way: the calls behind it stay away)
         if (!pol->probed[cls] || retry || pending) {
-            if (!pending) { pol->word[policy_word(1, cls)] = kWordPending; pol->pending[cls] = 0u; }
+            if (!pending && !retry) { pol->word[policy_word(1, cls)] = kWordPending; pol->pending[cls] = 0u; }
             pol->probed[cls] = 1u;
             return kPathProbe;
         }
