@@ -44,7 +44,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, vendor figure
 # HBM bytes per call of the bandwidth configuration from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs
 # summarised in the file named here, valid for the library version they were taken with: a library
 # that has moved on reports traffic as null rather than a stale figure.
-TRAFFIC_PROFILE = {"file": "profiles/bench_kernels_hbm_traffic_pmc.md", "rs_version": 411, "bytes": 573757952}
+TRAFFIC_PROFILE = {"file": "profiles/bench_kernels_hbm_traffic_pmc.md", "rs_version": 413, "bytes": 573848064}
 
 
 def event_times_us(torch, fn, steps, warmup):
@@ -268,7 +268,7 @@ def main():
                        "plain loads, 64 KiB per workgroup", "non-temporal loads, 64 KiB per workgroup",
                        "persistent grid of 2048 workgroups, 4 loads in flight", "the same, an eighth of the data per XCD",
                        "256 KiB contiguous per workgroup, 16 loads in flight",
-                       "persistent grid of 1024 workgroups per XCD, 8 loads in flight",
+                       "persistent grid of 1024 workgroups, an eighth of the data per XCD, 8 loads in flight",
                        "persistent grid of 4096 workgroups, 2 loads in flight"]
         t_floors = [block_time_us(torch, floor_variant(n), args.bandwidth_steps, 3) for n in range(len(floor_names))]
         t_floor = min(t_floors)

@@ -476,7 +476,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 412; }
+int rs_version(void) { return 413; }
 
 const char *rs_error_string(int code)
 {
