@@ -318,8 +318,11 @@ __global__ void __launch_bounds__(kThreads, (R <= 8 ? 5 : RS_STREAM_WAVES)) wide
     const uint32_t width = ranged ? ((uint32_t)(bt + 1) << 21) - lo_live : 0u;          // no pattern is this far above lo_live when the range is off
     const uint32_t exb_top = (uint32_t)bt >> 2;
 
-    // e in the slice's frame (not clamped at 2^-40) and the level-1 histogram: the streaming pass's loop,
-    // without a branch in it; slots past the end of the row become 0
+    // e in the slice's frame (not clamped at 2^-40) and ONE histogram atomic per token, as in the streaming
+    // pass: a token of the range is counted in its sub-bin, every other token in its level-1 bin -- the
+    // address is selected, nothing is branched on (a conditional per token keeps the compiler from
+    // interleaving the tokens' polynomials and is issued whenever some lane of the wave takes it).  Slots
+    // past the end of the row become 0.
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         if (j < nv) {
@@ -327,25 +330,23 @@ __global__ void __launch_bounds__(kThreads, (R <= 8 ? 5 : RS_STREAM_WAVES)) wide
             for (int q = 0; q < 4; ++q) {
                 const uint32_t b = e_bits_raw(__uint_as_float(eb[j * 4 + q]), M);
                 eb[j * 4 + q] = b;
-                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) * kRep + (lane & (kRep - 1))]),
+                uint64_t *bin = &s.hm[(b >> 21) * kRep + (lane & (kRep - 1))];
+                uint64_t *sub = &s.sub[(((b - lo_bits) >> sh) & 127u) * kW1Rep + (lane & (kW1Rep - 1))];
+                atomicAdd(reinterpret_cast<unsigned long long *>(b - lo_live < width ? sub : bin),
                           (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
             }
         } else {
             eb[j * 4] = 0; eb[j * 4 + 1] = 0; eb[j * 4 + 2] = 0; eb[j * 4 + 3] = 0;
         }
     }
-    // the range's sub-bins, in a loop of its own (a conditional per token in the loop above keeps the
-    // compiler from interleaving the tokens' polynomials)
-    if (ranged) {
-#pragma unroll
-        for (int j = 0; j < R; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t b = eb[j * 4 + q];
-                if (b - lo_live < width)
-                    atomicAdd(reinterpret_cast<unsigned long long *>(&s.sub[((b - lo_bits) >> sh) * kW1Rep + (lane & (kW1Rep - 1))]),
-                              (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
-            }
+    __syncthreads();
+    // the range's level-1 bins: their sub-bins added up (everything behind this reads the bins as the
+    // streaming pass does)
+    if (ranged && tid < 128) {
+        const uint64_t w = s.sub[tid * kW1Rep] + s.sub[tid * kW1Rep + 1];
+        static_assert(kW1Rep == 2, "two copies");
+        if (w) atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[((lo_bits + ((uint32_t)tid << sh)) >> 21) * kRep + (tid & (kRep - 1))]),
+                         (unsigned long long)w);
     }
     if (p.e_bits) {
         // diagnostics: e of every token, still in the slice's frame; the finishing workgroup re-bases it
