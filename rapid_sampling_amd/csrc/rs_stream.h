@@ -1111,8 +1111,11 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     // there and, the general kernel's time growing with the row, at about 4700 for rows of 100256): a
     // call that is only an attempt (no top_k bounds the kept set) says so to the caller's policy, and so
     // does a call of moderate size with a bounding top_k (a lone flat row of 32768 tokens with top_k 1000:
-    // 26.7 us here against 17.5 on the general kernel).
-    const uint32_t long_list = max(2048u, (uint32_t)p.V / 20u);
+    // 26.7 us here against 17.5 on the general kernel).  Small calls in rows of up to 100256 tokens meet the
+    // general kernel earlier: a list of a thousand tokens takes one to sixteen such rows 21-27 us here
+    // against 18-21 there (lists of a few hundred: 12-14 us here).
+    const bool small_call = (uint64_t)p.B * (uint64_t)p.V < (1ull << 20) && p.V < 131072;
+    const uint32_t long_list = small_call ? 768u : max(2048u, (uint32_t)p.V / 20u);
     if (!FUSED && (p.attempt || (uint64_t)p.B * (uint64_t)p.V < (1ull << 24)) && total > long_list) tell_policy();
 
     // gather the tokens, re-based to the row's frame

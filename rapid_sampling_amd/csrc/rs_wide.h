@@ -432,20 +432,21 @@ __device__ __forceinline__ void wide_finish_row(const Params &p, const StreamVie
     PartHdr ph;
     ph.mkey = 0; ph.cov = 0; ph.n = 0; ph.cut = 0;
     if ((uint32_t)tid < G) ph = hdrs[tid];
-    // the row's level 2: thread j sums the slices' running sums at sub-bin j (a load instruction reads one
-    // slice's 129 consecutive words); the row's sub-bin j is the difference of two neighbours
+    // the row's level 2: a thread sums half of the slices' running sums at one of the 128 sub-bin edges (the
+    // 129th is zero by definition; a load instruction reads one slice's consecutive words, sixteen slices'
+    // loads in flight at a time); the row's sub-bin j is the difference of two neighbours
     uint64_t cpsum = 0;
-    if (tid < 129) {
-        const uint64_t *cp0 = v.stash + (size_t)row * G * kStashCap + 2 + tid;
-        uint32_t g = 0;
-        for (; g + 8u <= G; g += 8u) {
-            uint64_t w[8];
+    {
+        const uint32_t edge = (uint32_t)tid & 127u, upper = (uint32_t)tid >> 7;
+        const uint32_t g_mid = (G + 1u) >> 1, g_hi = upper ? G : g_mid;
+        const uint64_t *cp0 = v.stash + (size_t)row * G * kStashCap + 2 + edge;
+        for (uint32_t g0 = upper ? g_mid : 0u; g0 < g_hi; g0 += 16u) {
+            uint64_t w[16];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) w[u] = cp0[(size_t)(g + u) * kStashCap];
+            for (int u = 0; u < 16; ++u) w[u] = cp0[(size_t)min(g0 + (uint32_t)u, G - 1u) * kStashCap];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) cpsum += w[u];
+            for (int u = 0; u < 16; ++u) if (g0 + (uint32_t)u < g_hi) cpsum += w[u];
         }
-        for (; g < G; ++g) cpsum += cp0[(size_t)g * kStashCap];
     }
     WidePlan *plan = reinterpret_cast<WidePlan *>(rc->A);
     const WidePlan pl = *plan;
@@ -507,7 +508,11 @@ __device__ __forceinline__ void wide_finish_row(const Params &p, const StreamVie
 
     // level 2: the row's sub-bins of the boundary bin must add up to the bin
     const uint32_t b1 = f.bin;
-    if (tid < 129) s.g[tid] = cpsum;
+    if (tid >= 128) s.g[tid] = cpsum;                    // the upper half of the slices, beside the lower half's place
+    __syncthreads();
+    if (tid < 128) s.g[tid] = cpsum + s.g[tid + 128];
+    __syncthreads();
+    if (tid == 128) s.g[128] = 0;
     __syncthreads();
     if (tid < 128) s.hm[tid] = s.g[tid] - s.g[tid + 1];
     const uint32_t cnt2 = pack_count(s.g[0]);

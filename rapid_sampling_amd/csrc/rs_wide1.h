@@ -566,28 +566,42 @@ __device__ __forceinline__ void wide1_finish_row(const Params &p, const StreamVi
     const uint32_t cnt_ar = block_sum_u32(s, c_ab, lane, wave);
     const uint32_t cnt_in = block_sum_u32(s, c_in, lane, wave);
     const u128 mass_ar = block_sum_u128(s, m_ab, lane, wave);
-    // the row's running sums at the 129 sub-bin edges: the slices' added up
+    // The row's running sums at the sub-bin edges: the slices' added up (edge 128 is zero by definition).
+    // Every thread takes one edge and half of the slices, sixteen slices' loads in flight at a time; what a
+    // slice that said nothing left behind is not added.
+    if ((uint32_t)tid < G) t.take[tid] = ph.cov & kWideValid;
+    __syncthreads();
     uint32_t Rc = 0;
     u128 Rm = 0;
-    if (tid < 129) {
-        const uint32_t *cp0 = v.cum + (size_t)row * G * kSB + tid;
-        const uint64_t *mp0 = v.stash + (size_t)row * G * kStashCap + 2 + 2 * tid;
-        // (eight slices' loads in flight at a time; what a slice that said nothing left behind is not added)
-        for (uint32_t g0 = 0; g0 < G; g0 += 8u) {
-            uint32_t cv[8], c[8];
-            uint64_t m0[8], m1[8];
+    {
+        const uint32_t edge = (uint32_t)tid & 127u, upper = (uint32_t)tid >> 7;
+        const uint32_t g_mid = (G + 1u) >> 1, g_lo = upper ? g_mid : 0u, g_hi = upper ? G : g_mid;
+        const uint32_t *cp0 = v.cum + (size_t)row * G * kSB + edge;
+        const uint64_t *mp0 = v.stash + (size_t)row * G * kStashCap + 2 + 2 * edge;
+        for (uint32_t g0 = g_lo; g0 < g_hi; g0 += 16u) {
+            uint32_t c[16];
+            uint64_t m0[16], m1[16];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < 16; ++u) {
                 const size_t g = min(g0 + (uint32_t)u, G - 1u);
-                cv[u] = hdrs[g].cov; c[u] = cp0[g * kSB]; m0[u] = mp0[g * kStashCap]; m1[u] = mp0[g * kStashCap + 1];
+                c[u] = cp0[g * kSB]; m0[u] = mp0[g * kStashCap]; m1[u] = mp0[g * kStashCap + 1];
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (g0 + (uint32_t)u < G && (cv[u] & kWideValid)) { Rc += c[u]; Rm += (u128)m0[u] | ((u128)m1[u] << 64); }
+            for (int u = 0; u < 16; ++u)
+                if (g0 + (uint32_t)u < g_hi && t.take[g0 + (uint32_t)u]) { Rc += c[u]; Rm += (u128)m0[u] | ((u128)m1[u] << 64); }
         }
+        if (upper) { t.blo[edge] = (uint64_t)Rm; t.bhi[edge] = (uint64_t)(Rm >> 64); t.m4[edge] = Rc; }
     }
+    __syncthreads();
     uint64_t *Rlo = s.cand, *Rhi = s.cand + 256, *Rcn = s.cand + 512;
-    if (tid < 129) { Rlo[tid] = (uint64_t)Rm; Rhi[tid] = (uint64_t)(Rm >> 64); Rcn[tid] = Rc; }
+    if (tid < 128) {
+        Rm += (u128)t.blo[tid] | ((u128)t.bhi[tid] << 64);
+        Rc += t.m4[tid];
+        Rlo[tid] = (uint64_t)Rm; Rhi[tid] = (uint64_t)(Rm >> 64); Rcn[tid] = Rc;
+    } else {
+        Rc = 0; Rm = 0;
+        if (tid == 128) { Rlo[128] = 0; Rhi[128] = 0; Rcn[128] = 0; }
+    }
     const bool suff = tid < 129 && ((uint64_t)cnt_ar + Rc >= top_k || mass_ar + (Rm >> shr) >= P);
     {
         const uint64_t vote = __ballot(suff);
