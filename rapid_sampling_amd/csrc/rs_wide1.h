@@ -55,7 +55,7 @@ struct LdsS {                         // sampling kernel
     u128     D, P;
     Found    found;
     uint64_t g[kNB];                  // the sample's level-1 histogram, sample frame
-    uint64_t hm[kNB * 4];             // the same while it is counted: four copies of each bin
+    uint64_t hm[kNB * 8];             // the same while it is counted: eight copies of each bin (lane l adds to copy l % 8)
     uint32_t sub[128 * 4];            // the range's sub-bins, counts only, four copies
     uint32_t u32[16];
     uint32_t b32[8];
@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(kW1SampleT) wide_sample_kernel(const Params p,
         if (tid == 0) { none->state = 2u; none->M = 0.0f; none->bin_top = kTop1; none->n_log2 = 0u; none->j_lo = 1u; none->j_hi = 0u; none->j_est = 0u; none->pad = 0u; }
         return;
     }
-    for (int i = tid; i < kNB * 4; i += kThreads) s.hm[i] = 0;
+    for (int i = tid; i < kNB * 8; i += kThreads) s.hm[i] = 0;
     for (int i = tid; i < 128 * 4; i += kThreads) s.sub[i] = 0;
 
     uint32_t eb[kW1SampleR * 4];
@@ -125,13 +125,14 @@ __global__ void __launch_bounds__(kW1SampleT) wide_sample_kernel(const Params p,
             const uint32_t b = in ? e_bits_raw(__uint_as_float(eb[j * 4 + q]), M) : 0u;
             eb[j * 4 + q] = b;
             if (b >= kEMinBits)
-                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) * 4u + (uint32_t)(lane & 3)]),
+                atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[(b >> 21) * 8u + (uint32_t)(lane & 7)]),
                           (unsigned long long)(kPackOne | (b & 0x7FFFFFu)));
         }
     }
     __syncthreads();
     for (int b = tid; b < kNB; b += kThreads)
-        s.g[b] = b >= (int)kBin0 ? s.hm[b * 4] + s.hm[b * 4 + 1] + s.hm[b * 4 + 2] + s.hm[b * 4 + 3] : 0ull;
+        s.g[b] = b >= (int)kBin0 ? s.hm[b * 8] + s.hm[b * 8 + 1] + s.hm[b * 8 + 2] + s.hm[b * 8 + 3] +
+                                   s.hm[b * 8 + 4] + s.hm[b * 8 + 5] + s.hm[b * 8 + 6] + s.hm[b * 8 + 7] : 0ull;
     __syncthreads();
     // the sample's share of top_k
     const uint64_t k_s = p.top_k >= p.V ? (uint64_t)n_s : ((uint64_t)p.top_k * n_s + (uint64_t)p.V - 1u) / (uint64_t)p.V;
