@@ -33,7 +33,7 @@ namespace rs {
 
 constexpr int      kW1Head    = 260;                     // words at the head of a slice's stash region: mass above the range (2), running masses (129 x 2)
 constexpr int      kW1Cap     = kStashCap - kW1Head;     // tokens a slice can set aside
-constexpr int      kW1Rep     = 2;                       // copies of each sub-bin while it is counted
+constexpr int      kW1Rep     = 4;                       // copies of each sub-bin while it is counted
 constexpr int      kW1SampleT = 1024;                    // threads of the sampling kernel
 constexpr int      kW1SampleR = 8;                       // groups of four tokens per thread of the sampling kernel: 32768 tokens at most
 constexpr uint32_t kW1Rounds  = 9u;                      // DiagRow::rounds of a row finished here
@@ -137,6 +137,14 @@ __global__ void __launch_bounds__(kW1SampleT) wide_sample_kernel(const Params p,
     // the sample's share of top_k
     const uint64_t k_s = p.top_k >= p.V ? (uint64_t)n_s : ((uint64_t)p.top_k * n_s + (uint64_t)p.V - 1u) / (uint64_t)p.V;
     const Found f = hist_find_level1<false, false, LdsS>(s, max(k_s, (uint64_t)1), p.top_p, lane, wave);
+    // A sample that is one tie (rows of equal logits) says nothing about a threshold, and a range around it
+    // would queue every token of the row up at one sub-bin: no guess.  (A row that is one tie of all its
+    // tokens is recognised by the finishing workgroup from the row's bins alone.)
+    if (f.cnt_bin == n_s && bin_is_one_tie(s.g[f.bin], f.bin, e_bits_of(fkey_inv(kmax), M))) {
+        WideGuess *none = reinterpret_cast<WideGuess *>(rc->A);
+        if (tid == 0) { none->state = 2u; none->M = M; none->bin_top = kTop1; none->n_log2 = 0u; none->j_lo = 1u; none->j_hi = 0u; none->j_est = 0u; none->pad = 0u; }
+        return;
+    }
 
     // How many of the sample's tokens lie above its threshold, roughly (the position inside the boundary
     // bin by linear interpolation of count and mass), and how far off that rank may be for the row:
@@ -275,8 +283,7 @@ __global__ void __launch_bounds__(kThreads, (R <= 8 ? 5 : RS_STREAM_WAVES)) wide
 #pragma unroll
         for (int i = 0; i < kNB * kRep / 2 / NT; ++i) z[tid + i * NT] = make_uint4(0u, 0u, 0u, 0u);
         static_assert(kNB * kRep % (2 * NT) == 0, "whole stores");
-        if (tid < 128 * kW1Rep) s.sub[tid] = 0;
-        static_assert(128 * kW1Rep <= NT, "one store each");
+        for (int i = tid; i < 128 * kW1Rep; i += NT) s.sub[i] = 0;
     }
 #pragma unroll
     for (int j = 0; j < R; ++j) {
@@ -344,8 +351,9 @@ __global__ void __launch_bounds__(kThreads, (R <= 8 ? 5 : RS_STREAM_WAVES)) wide
     // the range's level-1 bins: their sub-bins added up (everything behind this reads the bins as the
     // streaming pass does)
     if (ranged && tid < 128) {
-        const uint64_t w = s.sub[tid * kW1Rep] + s.sub[tid * kW1Rep + 1];
-        static_assert(kW1Rep == 2, "two copies");
+        uint64_t w = 0;
+#pragma unroll
+        for (int c = 0; c < kW1Rep; ++c) w += s.sub[tid * kW1Rep + c];
         if (w) atomicAdd(reinterpret_cast<unsigned long long *>(&s.hm[((lo_bits + ((uint32_t)tid << sh)) >> 21) * kRep + (tid & (kRep - 1))]),
                          (unsigned long long)w);
     }
