@@ -248,7 +248,11 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  * a sample of the row, an eighth of it at most, one pass over the logits that
  * counts the row's bins and, finely, the range in which the sample expects the
  * threshold, and sets the tokens around it aside, a per-row finish that checks
- * the guess against the exact counts), or three for calls of at least
+ * the guess against the exact counts), one again for such kept sets in rows of
+ * 8192 to 65536 tokens when the call has 64 rows (128 from 32768 tokens on)
+ * or more (the row kernel: one workgroup of 1024 threads per row, the row in
+ * its registers; calls of more than 256 rows only from 32768 tokens per row
+ * on), or three for calls of at least
  * 2^23 tokens with penalties and top_k <= 1024 (a pass over logits and
  * penalties that also writes the decayed penalties, the finish, which patches
  * the sampled tokens' penalties, and a fix-up kernel for slices the pass left
@@ -299,7 +303,9 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
  * finish in one launch (any call whose rows span at least two slices, with or
  * without penalties; else the general kernel), RS_PATH_WIDE the two-pass wide
  * path and RS_PATH_WIDE1 the one-pass wide path (any call without penalties; a
- * call that keeps every token takes the counting-only streaming variant).  `slice_r` forces the float4 groups per thread of the
+ * call that keeps every token takes the counting-only streaming variant),
+ * RS_PATH_ROW the row kernel (any call without penalties in rows of up to
+ * 65536 tokens; else the general kernel).  `slice_r` forces the float4 groups per thread of the
  * general kernel (1, 2, 4, 8, 16 or 32; 0 = chosen by the library).
  * `policy` see rs_policy.  No counterpart in the reference.
  */
@@ -310,6 +316,7 @@ int rs_sample_dtype(const void *logits_device, int32_t logits_dtype, int64_t row
 #define RS_PATH_FUSED   4
 #define RS_PATH_WIDE    5
 #define RS_PATH_WIDE1   6
+#define RS_PATH_ROW     7
 typedef struct rs_options {
     int32_t    path;
     int32_t    slice_r;

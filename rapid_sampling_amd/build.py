@@ -36,7 +36,7 @@ def _run(cmd, verbose):
     subprocess.check_call(cmd)
 
 
-KERNEL_SOURCES = ["rs_api.hip", "rs_cluster.hip", "rs_stream.hip", "rs_wide.hip"]
+KERNEL_SOURCES = ["rs_api.hip", "rs_cluster.hip", "rs_stream.hip", "rs_wide.hip", "rs_row.hip"]
 
 
 def build_kernels(verbose=False):

@@ -42,6 +42,10 @@
 //     the boundary bin of the first known, counts the bin's next digit and sets
 //     aside the tokens around the place where each slice expects the threshold.
 //
+//   row kernel (row_kernel, one launch, no workspace, no waits): the same kept sets
+//     in rows of up to 65536 tokens when the call has rows enough to fill the GPU
+//     with one workgroup of 1024 threads per row, the row in its registers.
+//
 //   one-launch path (fused_kernel): the streaming pass and the finish in one
 //     grid, for calls with penalties that fit the device at once.
 //
@@ -330,7 +334,7 @@ namespace rs {
 // Measured on MI355X, back to back: with a bounding top_k the streaming path beats the cluster
 // kernel from 131072 tokens per call upwards (15-17 us for small calls against 16-31 us, 2-3
 // times faster for large ones); below that the single launch wins by up to a microsecond.
-enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5, kPathProbe = 6, kPathWide1 = 7 };
+enum { kPathCluster = 0, kPathStream = 1, kPathAttempt = 2, kPathFused = 3, kPathKeep = 4, kPathWide = 5, kPathProbe = 6, kPathWide1 = 7, kPathRow = 8 };
 // The wide path (four launches, two reads of the logits) against the general kernel (one launch, its
 // exchanges), measured on flat rows (U[0,1), top_p 0.9) and on N(0,1.5) with top_k 10000: the wide path
 // wins from about 25 million tokens per call on in rows of 50304 tokens and more (96 x 262144: 88 against
@@ -348,6 +352,29 @@ constexpr int32_t kWideMinV = 49152;
 // against 226).
 constexpr uint64_t kWide1Min = 1ull << 26;
 constexpr uint64_t kPenStreamMin = 1ull << 23;
+// The row kernel (one workgroup per row, the row in its registers, one launch; rows of up to 65536 tokens, no
+// penalties) against what else there is for kept sets the stashes cannot hold, same rows, us per call:
+//   rows x tokens   general/wide  row kernel        rows x tokens   general/wide  row kernel
+//    64 x  8192       19 / 15      18 / 14           96 x 50304       30 / 28      31 / 32
+//   256 x  8192       22 / 18      18 / 15          128 x 50304       39 / 36      32 / 32
+//   384 x  8192       24 / 19      32 / 25          256 x 50304       62 / 58      33 / 34
+//   256 x 16384       27 / 27      21 / 20          384 x 50304       81 / 77      62 / 63
+//   512 x 16384       32 / 33      39 / 36          512 x 50304      103 / 85      65 / 66
+//    96 x 32768       25 / 24      26 / 24         1024 x 50304      171 / 146    128 / 131
+//   256 x 32768       38 / 36      27 / 26         2048 x 50304      343 / 336    252 / 258
+//   384 x 32768       45 / 43      49 / 45          128 x 65536       38 / 36      37 / 39
+//   512 x 32768       58 / 55      52 / 47          256 x 65536       65 / 61      41 / 44
+//  2048 x 32768      193 / 185    197 / 181        1024 x 65536      186 / 184    159 / 167
+// Its time is that of one row (14 us for 8192 tokens, 20 for 16384, 26 for 32768, 33 for 50304, 42 for
+// 65536) times the rounds of 256 rows the call makes: it wins whenever one round does (from 64 rows on in
+// short rows, 128 in long ones), and in rows of 32768 tokens and more also over several rounds.
+static bool row_suits(int32_t B, int32_t V)
+{
+    if (V > kRowMaxV || V < 8192) return false;
+    if (B <= 256) return B >= (V < 32768 ? 64 : 128);
+    if (V < 32768) return false;
+    return B >= 512 || V >= 40000;                            // 257 to 511 rows: two rounds pay off in long rows only
+}
 // Plain temperature sampling (top_k = V, top_p = 1: every live token is kept) has no kept set to
 // stash, but the streaming pass's bins alone say which slice holds the target: one pass at
 // bandwidth that only counts, plus a second look at one slice per row, beats the general kernel's
@@ -425,6 +452,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (force == RS_PATH_ATTEMPT) return bounded ? kPathStream : kPathAttempt;
     if (force == RS_PATH_WIDE) return keep_all ? kPathKeep : kPathWide;
     if (force == RS_PATH_WIDE1) return keep_all ? kPathKeep : kPathWide1;
+    if (force == RS_PATH_ROW) return V <= kRowMaxV ? kPathRow : kPathCluster;
     // Small calls: rows of fewer than 8192 tokens are one or two workgroups of the general kernel each, with
     // few or no exchanges (8.5 us for a row of 256 tokens); from 8192 tokens per row on the streaming
     // path's two launches are faster whatever the batch (one row of 8192 to 100256 tokens: 13.6-14.7
@@ -433,10 +461,11 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     if (keep_all && V >= 32768) return kPathKeep;              // shorter rows: one workgroup of the general kernel does a row in one go
     // kept sets the stashes cannot hold: the wide path from kWideMin tokens on, unless its rows have been
     // going the slow way (slices that are no fair samples of their rows, ties of thousands of tokens)
-    // (the one-pass wide path first; when its rows have been going the slow way -- samples that are no fair
+    // (short rows in calls of many: the row kernel; else the one-pass wide path first; when its rows have been going the slow way -- samples that are no fair
     // picture of their rows -- the two-pass one, which counts everything; then the general kernel)
     auto wide_or_general = [&]() {
         const uint64_t tokens = (uint64_t)B * (uint64_t)V;
+        if (row_suits(B, V)) return (int)kPathRow;
         if (tokens >= kWide1Min && V >= kWideMinV && !routed_away(2)) return (int)kPathWide1;
         if (tokens >= kWideMin && V >= kWideMinV && !routed_away(3)) return (int)kPathWide;
         return (int)kPathCluster;
@@ -648,7 +677,7 @@ static int check_call(const void *logits, int32_t logits_dtype, int64_t row_stri
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
     if (!(top_k >= 1 && top_k <= V) || !(top_p > 0.0f && top_p <= 1.0f) || !(log2e_inv_temp > 0.0f)) return RS_ERR_ARG;
-    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_WIDE1 || opt->slice_r < 0)) return RS_ERR_ARG;
+    if (opt && (opt->path < RS_PATH_AUTO || opt->path > RS_PATH_ROW || opt->slice_r < 0)) return RS_ERR_ARG;
     if (((uintptr_t)logits & (logits_dtype == RS_DTYPE_F32 ? 15 : 7)) || (B > 1 && (row_stride & 3)) || ((uintptr_t)penalties & 15) || ((uintptr_t)e_bits & 15))
         return RS_ERR_ALIGN;
     return RS_OK;
@@ -705,6 +734,7 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.defer_pen = 0; p.probe = 0;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
+    if (path == kPathRow) return launch_row(logits_dtype, (uint32_t)B, (hipStream_t)stream, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
     if (path != kPathCluster) {
         const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V, pen);
         StreamView v;

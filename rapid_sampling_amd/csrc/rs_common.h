@@ -541,7 +541,8 @@ __device__ __forceinline__ bool bin_is_one_tie(uint64_t word, uint32_t bin, uint
 
 // The same for a 128-bin level (all tokens share the exponent ex): one wave,
 // lane l owns indices 127-2l and 126-2l, no LDS exchange inside the scan.
-__device__ __forceinline__ Found hist_find128(Lds &s, const uint64_t *arr, uint32_t cnt0, u128 mass0,
+template <typename L = Lds>
+__device__ __forceinline__ Found hist_find128(L &s, const uint64_t *arr, uint32_t cnt0, u128 mass0,
                                               uint64_t top_k, uint32_t ex, int lane, int wave)
 {
     if (wave == 0) {
@@ -681,5 +682,7 @@ hipError_t launch_stream(int slice_r, int32_t dtype, bool keep, uint32_t B, size
 hipError_t launch_fused(int slice_r, bool pen, uint32_t B, hipStream_t st, const Params &p, const StreamView &v);
 hipError_t launch_wide(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
 hipError_t launch_wide1(int slice_r, int32_t dtype, uint32_t B, size_t finish_lds_bytes, hipStream_t st, const Params &p, const StreamView &v);
+constexpr int32_t kRowMaxV = 65536;                      // the longest row the row kernel holds in its registers
+hipError_t launch_row(int32_t dtype, uint32_t B, hipStream_t st, const Params &p);
 
 }  // namespace rs

@@ -396,7 +396,8 @@ void force_path(const std::string &name)
     else if (name == "fused") g_forced_path = RS_PATH_FUSED;
     else if (name == "wide") g_forced_path = RS_PATH_WIDE;
     else if (name == "wide1") g_forced_path = RS_PATH_WIDE1;
-    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused | wide | wide1");
+    else if (name == "row") g_forced_path = RS_PATH_ROW;
+    else throw std::invalid_argument("force_path: auto | cluster | stream | attempt | fused | wide | wide1 | row");
 }
 
 // The workspace tensor of the current stream (tests poison it to force the error path).

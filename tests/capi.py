@@ -17,7 +17,7 @@ DIAG_DTYPE = np.dtype([
     ("S", "<u8", (2,)), ("r", "<u8", (2,)),
 ])
 
-PATHS = {None: 0, "auto": 0, "cluster": 1, "stream": 2, "optimistic": 3, "attempt": 3, "fused": 4, "wide": 5, "wide1": 6}
+PATHS = {None: 0, "auto": 0, "cluster": 1, "stream": 2, "optimistic": 3, "attempt": 3, "fused": 4, "wide": 5, "wide1": 6, "row": 7}
 
 
 class Options(C.Structure):

@@ -75,15 +75,20 @@ def _run_case(torch, oracle, capi, logits_np, temperature, top_k, top_p, *, pen_
     # streaming path (taken for top_k <= 1024; rows it cannot finish go on to the general kernel), the
     # same attempted whatever top_k is, the one-launch path (streaming pass and finish in one kernel,
     # falling back inside the kernel), the wide paths (two passes over the logits and a finish, for kept
-    # sets of any size; one pass behind a sample of the row), then the general kernel again on the workspace these leave
-    # behind.  All but the general kernel also return the e of every token: the kept set on that path.
+    # sets of any size; one pass behind a sample of the row), the row kernel (one workgroup per row, rows of
+    # up to 65536 tokens; longer ones take the general kernel), then the general kernel again on the workspace
+    # these leave behind.  All but the general kernel also return the e of every token: the kept set on that path.
     # With penalties: the one-launch path and the general kernel.
-    paths = ("cluster", "stream", "optimistic", "fused", "wide", "wide1", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
+    paths = ("cluster", "stream", "optimistic", "fused", "wide", "wide1", "row", "cluster") if pen_np is None else ("fused", "stream", "cluster", "fused")
     for path in paths:
         pen3 = None if pen_np is None else torch.from_numpy(pen_np.copy()).cuda()
+        with_e = path != "cluster" and not (path == "row" and V > 65536)
         res3 = smp.sample(lg, c, k, p, uniforms=u, penalties=pen3, presence=presence, repetition=repetition, decay=decay,
-                          path=path, force_r=force_r, want_e=path != "cluster")
-        _check(res3, ref_out, ref_diag, what + " (path %s)" % path, ref_e if path != "cluster" else None)
+                          path=path, force_r=force_r, want_e=with_e)
+        _check(res3, ref_out, ref_diag, what + " (path %s)" % path, ref_e if with_e else None)
+        if path == "row" and V <= 65536:
+            # (0: a row that is one tie of all its tokens, finished from the row's bins)
+            assert np.isin(res3["diag"]["rounds"], (0, 10)).all(), what + ": the row kernel finishes every row itself"
         assert smp.status() == 0
         if pen3 is not None:
             assert np.array_equal(pen3.cpu().numpy().view(np.uint32), pen_ref.view(np.uint32)), what + ": penalties, path " + path
@@ -306,9 +311,10 @@ def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
     0.9 on flat generators, /root/reference/bench.py:34-35, :66-72; its search costs the same whatever the
     kept set, sampling.cu:261-329): 512 flat rows of 262144 tokens under top_p 0.9, the bandwidth
     configuration's 128 rows of a million tokens with top_k 10000, 768 flat rows of 50304 tokens.  The
-    library takes a wide path for them by itself -- the one-pass one from 2^26 tokens per call on
-    (diag.rounds == 9), the two-pass one below (7), every row: none done the slow way; every row goes
-    through the oracle, and the general kernel and both wide paths must agree in every field."""
+    library takes a wide path for the long rows by itself -- the one-pass one from 2^26 tokens per call on
+    (diag.rounds == 9), the two-pass one below (7), every row: none done the slow way -- and the row kernel
+    for the rows of 50304 tokens (10); every row goes through the oracle, and the general kernel, both wide
+    paths and, where the rows fit it, the row kernel must agree in every field."""
     torch = torch_cuda
     from tests import capi
     g = torch.Generator(device="cuda")
@@ -320,12 +326,12 @@ def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
     u = torch.from_numpy(u_np).cuda()
     smp = capi.Sampler(B, V)
     res = {}
-    for path in ("auto", "cluster", "wide", "wide1"):
+    for path in ("auto", "cluster", "wide", "wide1") + (("row",) if V <= 65536 else ()):
         print("wide at scale", B, T, V, path, flush=True)
         r = smp.sample(lg, c, k, p, uniforms=u, path=path)
         assert r["rc"] == 0 and smp.status() == 0
         res[path] = r
-    auto_rounds = 9 if B * V >= 2 ** 26 else 7
+    auto_rounds = 10 if V <= 65536 else 9 if B * V >= 2 ** 26 else 7
     assert (res["auto"]["diag"]["rounds"] == auto_rounds).all(), np.unique(res["auto"]["diag"]["rounds"], return_counts=True)
     assert (res["wide"]["diag"]["rounds"] == 7).all()
     assert (res["wide1"]["diag"]["rounds"] == 9).all(), np.unique(res["wide1"]["diag"]["rounds"], return_counts=True)
@@ -334,6 +340,8 @@ def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
         assert np.array_equal(res["auto"]["diag"][f], res["cluster"]["diag"][f]), f
         assert np.array_equal(res["auto"]["diag"][f], res["wide"]["diag"][f]), f
         assert np.array_equal(res["auto"]["diag"][f], res["wide1"]["diag"][f]), f
+        if "row" in res:
+            assert np.array_equal(res["auto"]["diag"][f], res["row"]["diag"][f]), f
     assert np.array_equal(res["auto"]["out"], res["cluster"]["out"])
     d = res["auto"]["diag"]
     step = 64 if V <= 262144 else 32
@@ -379,6 +387,86 @@ def test_wide_path_unusual_rows(torch_cuda, oracle):
     rounds = res["diag"]["rounds"]
     assert rounds[0] == 9 and rounds[4] == 9 and rounds[6] == 9 and rounds[7] == 9, rounds
     assert rounds[1] in (8, 9) and rounds[2] in (8, 9) and rounds[3] == 8 and rounds[5] == 0, rounds
+
+
+def test_row_kernel_unusual_rows(torch_cuda, oracle):
+    """The row kernel (one workgroup per row, the row in its registers) on rows that take each of its ways:
+    a boundary bin of more tokens than its list holds (flat rows at a temperature of 2: every level counted
+    from the registers), sorted rows (a stretch per wave: the whole kept set in one wave's), rows of a few
+    distinct values (ties of thousands), masked stretches, a tie of all tokens, a row with one live token,
+    NaNs, few kept tokens (groups without one skipped); against the oracle on every path, in rows of every
+    length class the kernel is built for, float32, bfloat16 and half."""
+    torch = torch_cuda
+    from tests import capi
+    rng = np.random.default_rng(321)
+    for V in (65536, 50304, 20480, 12288, 4100, 64):
+        lg = rng.random((10, V), dtype=np.float32)
+        lg[1] = np.sort(lg[1])[::-1]
+        lg[2] = np.sort(lg[2])
+        lg[3] = np.round(lg[3] * 16) / 16
+        lg[4, V // 8:V // 8 * 5] = -np.inf
+        lg[5] = 0.5
+        lg[6] = (rng.standard_normal(V) * 1.5).astype(np.float32)
+        lg[7, ::3] += 0.5
+        lg[8] = -np.inf
+        lg[8, V - 3] = 1.0
+        lg[9, :V // 16] = np.nan
+        cases = [(2.0, -1, 0.9), (1.0, 10000, 1.0), (1.0, 40, 0.95)] if V >= 20480 else [(2.0, -1, 0.9), (1.0, 40, 0.95)]
+        for (temp, k, p) in cases:
+            _run_case(torch, oracle, capi, lg, temp, k, p, u_np=H.uniforms(10, 62), what="row kernel V=%d T=%g k=%d p=%g" % (V, temp, k, p))
+    for fmt in (torch.bfloat16, torch.float16):
+        lg = torch.from_numpy((rng.standard_normal((6, 50304)) * 3).astype(np.float32)).to(fmt).float().numpy()
+        _run_case(torch, oracle, capi, lg, 1.0, -1, 0.9, u_np=H.uniforms(6, 63), dtype=fmt, what="row kernel %s" % fmt)
+
+
+def test_row_kernel_takes_the_wide_kept_sets_of_calls_of_many_short_rows(torch_cuda, oracle):
+    """Calls of 128 rows and more (64 in rows of fewer than 32768 tokens) of 8192 to 65536 tokens whose kept
+    sets the stashes cannot hold go to the row kernel by themselves (diag.rounds == 10): a top_k of
+    thousands at once, a nucleus once the probe has reported its long lists; fewer rows, longer rows, 257
+    to 511 rows of fewer than 40000 tokens, more than 256 rows of fewer than 32768 and calls with a bounding
+    top_k do not.  Every call against the general kernel in every field, 64 rows of each against the oracle."""
+    torch = torch_cuda
+    from tests import capi
+    for (B, V, k, p, row) in [(128, 50304, 10000, 1.0, True), (300, 16384, 5000, 1.0, False), (200, 16384, 5000, 1.0, True),
+                              (127, 50304, 10000, 1.0, False), (160, 65540, 10000, 1.0, False), (256, 32768, 50, 0.9, False),
+                              (300, 32768, 5000, 1.0, False), (520, 32768, -1, 0.9, True), (64, 8192, 2000, 1.0, True)]:
+        lg_np = H.logits_uniform(B, V, seed=B)
+        lg = torch.from_numpy(lg_np).cuda()
+        rc, c, kk, pp = capi.normalize(1.0, k, p, V, B, 1)
+        u_np = H.uniforms(B, 64)
+        u = torch.from_numpy(u_np).cuda()
+        smp = capi.Sampler(B, V, with_policy=True, init=True)
+        print("row kernel routing", B, V, k, p, flush=True)
+        res = None
+        for call in range(3 if k == -1 else 1):                  # a nucleus: a probe first, then calls that know
+            res = smp.sample(lg, c, kk, pp, uniforms=u)
+            assert res["rc"] == 0 and smp.status() == 0
+        rounds = res["diag"]["rounds"]
+        assert ((rounds == 10).all() if row else (rounds != 10).all()), (B, V, k, p, np.unique(rounds, return_counts=True))
+        ref = smp.sample(lg, c, kk, pp, uniforms=u, path="cluster")
+        for f in FIELDS:
+            assert np.array_equal(res["diag"][f], ref["diag"][f]), f
+        assert np.array_equal(res["out"], ref["out"])
+        ref_out, ref_diag = oracle.sample_batch(lg_np[B - 64:], c, kk, pp, injected_u=u_np[B - 64:])
+        for f in FIELDS:
+            assert np.array_equal(res["diag"][f][B - 64:], ref_diag[f]), f
+        assert np.array_equal(res["out"][B - 64:], ref_out)
+        smp.close()
+    # the library's own random numbers: drawn as on every other path, the state left as the oracle leaves it
+    B, V = 130, 12288
+    lg_np = H.logits_normal(B, V, 0.5, seed=51)
+    rc, c, k, p = capi.normalize(1.0, 3000, 1.0, V, B, 1)
+    smp = capi.Sampler(B, V)
+    lg = torch.from_numpy(lg_np).cuda()
+    st = torch.empty(B * 64, dtype=torch.int8, device="cuda")
+    assert capi.lib().rs_philox_init(st.data_ptr(), 987654321, B, smp.stream()) == 0
+    rng_ref = oracle.rng_init(987654321, B)
+    for call in range(3):
+        ref_out, ref_diag = oracle.sample_batch(lg_np, c, k, p, rng=rng_ref)
+        res = smp.sample(lg, c, k, p, rng=st)
+        _check(res, ref_out, ref_diag, "row kernel, philox call %d" % call)
+        assert (res["diag"]["rounds"] == 10).all()
+    assert np.array_equal(st.cpu().numpy().view(np.uint32).reshape(B, 16), rng_ref)
 
 
 def test_wide_path_reports_slow_rows(torch_cuda, oracle):
@@ -1156,7 +1244,8 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     on the wide path that probes whether the rows' kept sets fit the stashes; peaked rows
     finish on it from the stashes (diag.rounds == 0).  A call with a row that had to be done the slow
     way (a flat row: the finishing workgroup goes through the logits again, diag.rounds == 8) says so in
-    the policy's report word at once, and the next calls go to the general kernel; streaming is tried
+    the policy's report word at once, and the next calls go to the general kernel (or, as these 600 rows of
+    65536 tokens once all of them are flat, to the row kernel, diag.rounds == 10); streaming is tried
     again after 64 of them, then 128, 256, ...; that a call went well is reported by the call after it,
     whichever kernel that is.  Without a policy no attempts are made.  Every result equals the
     oracle's whatever the route."""
@@ -1185,7 +1274,7 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     plain = capi.Sampler(B, V)                           # no policy: no report words
     res = plain.sample(lg_peaked, c, k, p, uniforms=u)
     _check(res, *ref_peaked, "no policy")
-    assert (res["diag"]["rounds"] >= 1).all()            # general kernel
+    assert (res["diag"]["rounds"] >= 1).all()            # no attempts without a policy: the row kernel for these 600 rows
 
     smp = capi.Sampler(B, V, with_policy=True, init=True)
     assert policy(smp) == 0
@@ -1208,7 +1297,7 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
     assert policy(smp) == 0
     res = smp.sample(lg_peaked, c, k, p, uniforms=u)
     assert (res["diag"]["rounds"] == 0).all() and policy(smp) == 0
-    # rows that are always too flat: the next try after 128 calls on the general kernel (a failed try doubles the stay)
+    # rows that are always too flat: the next try after 128 calls away (a failed try doubles the stay)
     streamed = []
     for i in range(135):
         res = smp.sample(lg_flat, c, k, p, uniforms=u)
@@ -1216,7 +1305,8 @@ def test_streaming_calls_are_routed_by_reports(torch_cuda, oracle):
         if (res["diag"]["rounds"] == 8).all():
             streamed.append(i)
         else:
-            assert (res["diag"]["rounds"] < 8).all() and (res["diag"]["rounds"] >= 1).all()
+            # 600 rows of 65536 tokens: the row kernel; the try after 128 calls away (call 129 here): a probe on the wide path
+            assert (res["diag"]["rounds"] == 10).all() or (i == 129 and (res["diag"]["rounds"] == 7).all()), (i, res["diag"]["rounds"][:4])
         assert policy(smp) == 1
     # (the try after 128 calls is a probe on the wide path, which says no without doing any row the slow way)
     assert streamed == [0], streamed
