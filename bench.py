@@ -365,6 +365,19 @@ def main():
             t_wp_two = block_time_us(torch, call_wide_p, max(2, args.bandwidth_steps // 2), 2)
         finally:
             sample._sample.force_path("auto")
+        # the same kind of kept set in many short rows: the row kernel (one workgroup per row, the row in registers)
+        short_rows = torch.rand((512, 50304), generator=g, device=dev)
+
+        def call_row():
+            return sample.batch_sampling_temperature_topk_topp(short_rows, st_w, 1.0, 10000, 1.0)
+
+        t_row = block_time_us(torch, call_row, 20, 3)
+        sample._sample.force_path("cluster")
+        try:
+            t_row_cluster = block_time_us(torch, call_row, 10, 2)
+        finally:
+            sample._sample.force_path("auto")
+        del short_rows
         result["roofline"]["wide_kept_sets"] = {
             "top_k_10000": {"us_per_call": round(t_wk, 2), "achieved": round(bytes_btv / (t_wk * 1e-6) / 1e9, 1),
                             "frac": round(bytes_btv / (t_wk * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
@@ -374,6 +387,12 @@ def main():
                                           "achieved": round(512 * 262144 * 4 / (t_wp * 1e-6) / 1e9, 1),
                                           "frac": round(512 * 262144 * 4 / (t_wp * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                                           "two_pass_us_per_call": round(t_wp_two, 2)},
+            "flat_512x50304_top_k_10000": {"us_per_call": round(t_row, 2),
+                                           "achieved": round(512 * 50304 * 4 / (t_row * 1e-6) / 1e9, 1),
+                                           "frac": round(512 * 50304 * 4 / (t_row * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                           "cluster_path_us_per_call": round(t_row_cluster, 2),
+                                           "note": "rs::row_kernel, one launch: a workgroup of 1024 threads per row, two rounds "
+                                                   "of 256 rows; bound by its vector instructions, not by the read"},
             "note": "one-pass wide path, three launches: rs::wide_sample_kernel (a sample of each row, 32768 tokens at "
                     "most), rs::wide1_kernel (the pass over the logits), rs::wide1_finish_kernel; two_pass: "
                     "rs::stream_kernel (counting only), rs::wide_plan_kernel, rs::wide_kernel (reads the logits a second "
