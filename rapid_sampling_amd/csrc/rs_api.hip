@@ -505,7 +505,7 @@ using namespace rs;
 
 extern "C" {
 
-int rs_version(void) { return 413; }
+int rs_version(void) { return 414; }
 
 const char *rs_error_string(int code)
 {

@@ -4,11 +4,15 @@
 // A row of up to 65536 tokens fits the registers of one compute unit (64 tokens per thread), and
 // then everything the other paths exchange between workgroups or kernels stays inside one
 // workgroup: the maximum, e, the level-1 histogram in LDS, the radix selection of the threshold
-// level by level on the registers, tie weight and target, and the pick by a scan of the kept
-// weights in index order.  Its time does not depend on the kept set (top_k 50 or a nucleus of a
-// hundred thousand tokens cost the same), only on the row: the vector instructions of e and of
-// three or four passes over the registers, about 13 us for a row of 50304 tokens; a call of B rows
-// takes ceil(B / 256) such times.  Same integers as every other path.
+// level by level (level 2 on the registers, the deeper ones on a list of the boundary bin's tokens
+// in LDS when they fit), tie weight and target, and the pick by sums and scans of the kept weights
+// in index order.  Its time hardly depends on the kept set, only on the row: it is the time of the
+// vector instructions of e and of three passes over the registers, 64 tokens per thread with four
+// waves per SIMD (measured, launch included: 14-18 us for 8192 tokens, 26 for 32768, 33 for 50304,
+// 42 for 65536); a call of B rows takes ceil(B / 256) such times.  For kept sets of thousands of
+// tokens in calls of 64 rows and more that is less than the general kernel's exchanges or the wide
+// paths' launches cost; small calls and small kept sets are better off elsewhere.  Same integers as
+// every other path.
 #pragma once
 
 #include "rs_common.h"
