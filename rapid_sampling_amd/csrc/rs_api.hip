@@ -487,7 +487,8 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
         }
         return kPathAttempt;
     }
-    return bounded ? kPathCluster : wide_or_general();
+    // (a bounding top_k whose rows have long lists all the same: flat rows with a top_k of a thousand)
+    return bounded ? (row_suits(B, V) ? kPathRow : kPathCluster) : wide_or_general();
 }
 
 static hipError_t fill_zero(void *dst, size_t bytes, hipStream_t st)
@@ -732,6 +733,10 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     p.stash_k = (uint32_t)top_k; p.report = 0; p.attempt = 0;
     p.host_words = opt && opt->policy ? opt->policy->word : nullptr;
     p.defer_pen = 0; p.probe = 0;
+    // Long lists on the streaming path are worth a report where another kernel does such rows faster: the
+    // general kernel in calls of fewer than 2^24 tokens, the row kernel (whose time does not depend on the
+    // kept set) in every call it suits
+    p.tell_lists = ((uint64_t)B * (uint64_t)V < (1ull << 24) || row_suits(B, V)) ? 1u : 0u;
     dim3 grid((uint32_t)B * g.G);
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path == kPathRow) return launch_row(logits_dtype, (uint32_t)B, (hipStream_t)stream, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;

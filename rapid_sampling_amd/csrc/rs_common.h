@@ -84,6 +84,7 @@ struct Params {
     int32_t      dtype;        // RS_DTYPE_* of the logits
     uint32_t     report;       // index of the report word of the caller's policy a streaming call writes (4..12: kind of call x size class), 0 none
     uint32_t     attempt;      // the call has no bounding top_k: its streaming pass is an attempt
+    uint32_t     tell_lists;   // streaming finish: a row whose list is long enough for another kernel to be faster says so to the policy
     uint32_t     probe;        // wide path as a probe for the streaming path: rows whose kept set the stashes would not hold are reported as slow
     int32_t     *host_words;   // the caller's rs_policy: pinned host memory, [2] error, [4..12] routing reports; or null
     int32_t      defer_pen;    // penalties enter x and are not rewritten from the registers at the end: 1 a later pass over them

@@ -23,7 +23,8 @@ constexpr int      kRowT      = 1024;                    // threads of the row k
 constexpr int      kRowW      = kRowT / kWave;
 constexpr int      kRowR      = 16;                      // groups of four tokens per thread at most: rows of up to 65536 tokens
 static_assert(kRowMaxV == kRowT * kRowR * 4, "the row kernel's registers hold kRowMaxV tokens");
-constexpr uint32_t kRowList   = (uint32_t)kNB * 8u * 2u; // tokens of the boundary bin listed for levels 3 and 4: what fits the bins' copies
+constexpr uint32_t kRowListW  = 768u;                    // tokens of the boundary bin a wave can list for levels 3 and 4
+constexpr uint32_t kRowList   = kRowListW * 12u;         // the row's boundary bin is listed when it holds no more than this (16 waves: room to spare for uneven shares)
 constexpr uint32_t kRowRounds = 10u;                     // DiagRow::rounds of a row finished here
 
 struct LdsRowS {                      // what the shared helpers work on
@@ -35,13 +36,15 @@ struct LdsRowS {                      // what the shared helpers work on
     uint64_t bc64[2];
     uint32_t bc32[8];
 };
+static_assert(kRowW * kRowListW / 2 >= (uint32_t)kNB * 8u, "the lists lie where the copies of the level-1 bins were");
 struct LdsRow {
     LdsRowS  s;
-    uint64_t hr8[kNB * 8];            // level 1 while it is counted: eight copies of each bin
+    uint64_t hr8[kRowW * kRowListW / 2];   // level 1 while it is counted: eight copies of each bin (the first kNB * 8
+                                      // words); later the waves' lists of the boundary bin's tokens (all of it)
     uint64_t lev[128 * 4];            // a deeper level while it is counted: four copies
     u128     wq[kRowW];               // per wave: kept weight of its stretch of the row
     u128     wq4[kRowW][4];           // the same, a quarter of the wave's groups at a time
-    uint32_t nlist;                   // entries of the list of the boundary bin's tokens
+    uint32_t nolist;                  // a wave's share of the boundary bin did not fit its list
     uint32_t wu[kRowW];
     uint64_t rand64;
 };
@@ -80,7 +83,7 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
     prev.slow_rows = 0; prev.meta = 0;
     if (reporter) prev = report_begin(p);
     for (int i = tid; i < kNB * 8; i += kRowT) L.hr8[i] = 0;
-    if (tid == 0) L.nlist = 0u;
+    if (tid == 0) L.nolist = 0u;
 
     // token (g0 + j * 64) * 4 + q sits in register j * 4 + q; slots past the end of the stretch read the
     // row's last group again (harmless for the maximum and the probe) and are set aside before anything is counted
@@ -208,11 +211,15 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
         if (one_tie) { lo = emax; span = 0u; }
     }
     // The tokens of the boundary bin are listed while level 2 counts them (where the bin's copies were: they
-    // are done with), if they fit; levels 3 and 4 then read the list, a few entries per thread, and not
-    // the registers again.
-    uint32_t *list = reinterpret_cast<uint32_t *>(L.hr8);
+    // are done with), every wave its own in a list of its own -- no counter to share, no wait: the place is
+    // the wave's running count plus the lane's rank among the wave's candidates of that instruction -- if
+    // the bin holds few enough for every wave's share to fit; levels 3 and 4 then read the lists, a few
+    // entries per thread, and not the registers again.  A wave whose share does not fit after all (a sorted
+    // row: the whole bin in one stretch) says so, and the levels go on from the registers.
+    uint32_t *list = reinterpret_cast<uint32_t *>(L.hr8) + (uint32_t)wave * kRowListW;
     const bool use_list = f.cnt_bin <= kRowList;
     bool have_list = false;
+    uint32_t nlist = 0u;                                 // wave-uniform
     for (uint32_t lv = 2; lv <= (uint32_t)kLevels && !one_tie && f.cnt_bin > 1u; ++lv) {
         const uint32_t dsh = level_shift(lv);
         if (tid < 128 * 4) L.lev[tid] = 0;
@@ -221,29 +228,35 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
         // kept in 128 registers across the levels
         uint32_t fmask = 0x7FFFFFu;
         asm volatile("" : "+v"(fmask));
-        if (!have_list) {
+        if (use_list && lv == 2u) {                      // count and list
 #pragma unroll
             for (int j = 0; j < kRowR; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const uint32_t b = eb[j * 4 + q];
-                    if (b - lo <= span) {
+                    const bool in = b - lo <= span;
+                    const uint64_t cand = __builtin_amdgcn_ballot_w64(in);
+                    if (in) {
                         atomicAdd(reinterpret_cast<unsigned long long *>(&L.lev[((b >> dsh) & 127u) * 4u + (uint32_t)(lane & 3)]),
                                   (unsigned long long)(kPackOne | (b & fmask)));
-                        if (use_list) {                  // one counter update per wave and instruction
-                            const uint64_t act = __builtin_amdgcn_ballot_w64(true);
-                            const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(act >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)act, 0u));
-                            uint32_t base = 0u;
-                            if (before == 0u) base = atomicAdd(&L.nlist, (uint32_t)__builtin_popcountll(act));
-                            base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
-                            list[base + before] = b;
-                        }
+                        const uint32_t at = nlist + __builtin_amdgcn_mbcnt_hi((uint32_t)(cand >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)cand, 0u));
+                        if (at < kRowListW) list[at] = b;
                     }
+                    nlist += (uint32_t)__builtin_popcountll(cand);
                 }
-            have_list = use_list;
+            if (nlist > kRowListW && lane == 0) L.nolist = 1u;
+        } else if (!have_list) {                         // count, from the registers
+#pragma unroll
+            for (int j = 0; j < kRowR; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t b = eb[j * 4 + q];
+                    if (b - lo <= span)
+                        atomicAdd(reinterpret_cast<unsigned long long *>(&L.lev[((b >> dsh) & 127u) * 4u + (uint32_t)(lane & 3)]),
+                                  (unsigned long long)(kPackOne | (b & fmask)));
+                }
         } else {
-            const uint32_t n = L.nlist;
-            for (uint32_t i = (uint32_t)tid; i < n; i += (uint32_t)kRowT) {
+            for (uint32_t i = (uint32_t)lane; i < nlist; i += (uint32_t)kWave) {
                 const uint32_t b = list[i];
                 if (b - lo <= span)
                     atomicAdd(reinterpret_cast<unsigned long long *>(&L.lev[((b >> dsh) & 127u) * 4u + (uint32_t)(lane & 3)]),
@@ -251,6 +264,7 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
             }
         }
         __syncthreads();
+        if (lv == 2u) have_list = use_list && L.nolist == 0u;
         if (tid < 128) s.hm[tid] = L.lev[tid * 4] + L.lev[tid * 4 + 1] + L.lev[tid * 4 + 2] + L.lev[tid * 4 + 3];
         __syncthreads();
         f = hist_find128(s, s.hm, f.cnt_above, f.mass_above, top_k, exb, lane, wave);
@@ -259,8 +273,7 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
     }
     if (span != 0u) {                                    // a single token left in the range: the threshold itself
         if (have_list) {
-            const uint32_t n = L.nlist;
-            for (uint32_t i = (uint32_t)tid; i < n; i += (uint32_t)kRowT)
+            for (uint32_t i = (uint32_t)lane; i < nlist; i += (uint32_t)kWave)
                 if (list[i] - lo <= span) s.bc32[6] = list[i];
         } else {
 #pragma unroll
@@ -285,12 +298,20 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
     // time; the wave whose stretch holds the target then finds it alone, in one quarter. ----
     constexpr int qb[5] = {0, (kRowR + 3) / 4, (2 * kRowR + 3) / 4, (3 * kRowR + 3) / 4, kRowR};
     // few kept tokens (f.cnt_above of them and f.cnt_bin ties): groups of four without one are skipped a wave at a time
-    const bool sparse = (uint64_t)(f.cnt_above + f.cnt_bin) * 8u < (uint64_t)(uint32_t)p.V;
-    auto weight = [=](uint32_t b) -> uint64_t { return (b > thr) ? w_of_bits(b) : (b == thr ? w_tie : 0ull); };
+    // (fewer than one kept token per wave and group on average: where most groups hold one the test only costs)
+    const bool sparse = (uint64_t)(f.cnt_above + f.cnt_bin) * 256u < (uint64_t)(uint32_t)p.V;
+    // (here a tie counts with the full weight of the threshold, and what the ties of the thread have too
+    // much, tie_less each, is taken off the sum: a select less per token)
+    auto weight = [=](uint32_t b) -> uint64_t {
+        const uint32_t x = b >= thr ? ((b & 0x7FFFFFu) | 0x800000u) : 0u;
+        return (uint64_t)x << (((b >> 23) - 87u) & 63u);
+    };
+    const uint64_t tie_less = w_of_bits(thr) - w_tie;    // w_tie <= the weight of the threshold
     u128 wtot = 0;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
         u128 mine = 0;
+        uint32_t ties = 0u;
 #pragma unroll
         for (int j = qb[q]; j < qb[q + 1]; ++j) {
             if (sparse) {
@@ -298,12 +319,14 @@ __global__ void __launch_bounds__(kRowT) row_kernel(const Params p)
                 if (__builtin_amdgcn_ballot_w64(m4 >= thr) == 0ull) continue;
             }
             mine += (u128)weight(eb[j * 4]) + weight(eb[j * 4 + 1]) + weight(eb[j * 4 + 2]) + weight(eb[j * 4 + 3]);
+            ties += (uint32_t)(eb[j * 4] == thr) + (uint32_t)(eb[j * 4 + 1] == thr) + (uint32_t)(eb[j * 4 + 2] == thr) + (uint32_t)(eb[j * 4 + 3] == thr);
             // four weights at a time: the running sum is made opaque, or all the weights are worked out first
             // (two registers each) and summed as a tree
             uint64_t lo64 = (uint64_t)mine, hi64 = (uint64_t)(mine >> 64);
             asm volatile("" : "+v"(lo64), "+v"(hi64));
             mine = ((u128)hi64 << 64) | lo64;
         }
+        mine -= (u128)ties * tie_less;
         const u128 t = wave_sum(mine);
         if (lane == 0) L.wq4[wave][q] = t;
         wtot += t;

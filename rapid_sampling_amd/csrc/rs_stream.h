@@ -1094,7 +1094,8 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
             // call while the call is of moderate size (measured: 64 flat rows of 131072 with top_k 1000,
             // 51 against 38 us; 128 rows of 262144, 77 against 117): such a call says so to the caller's
             // policy, as it did when these rows still went the slow way.
-            if ((uint64_t)p.B * (uint64_t)p.V < (1ull << 24)) tell_policy();
+            // (p.tell_lists: calls of fewer than 2^24 tokens, and calls whose rows the row kernel would take)
+            if (p.tell_lists) tell_policy();
         } else {
         if (total > v.list_cap || total == 0u) {
             // not resolvable from the stashes
@@ -1116,7 +1117,7 @@ __device__ __forceinline__ bool finish_row(const Params &p, const StreamView &v,
     // against 18-21 there (lists of a few hundred: 12-14 us here).
     const bool small_call = (uint64_t)p.B * (uint64_t)p.V < (1ull << 20) && p.V < 131072;
     const uint32_t long_list = small_call ? 768u : max(2048u, (uint32_t)p.V / 20u);
-    if (!FUSED && (p.attempt || (uint64_t)p.B * (uint64_t)p.V < (1ull << 24)) && total > long_list) tell_policy();
+    if (!FUSED && (p.attempt || p.tell_lists) && total > long_list) tell_policy();
 
     // gather the tokens, re-based to the row's frame
     if (!listed)

@@ -452,6 +452,26 @@ def test_row_kernel_takes_the_wide_kept_sets_of_calls_of_many_short_rows(torch_c
             assert np.array_equal(res["diag"][f][B - 64:], ref_diag[f]), f
         assert np.array_equal(res["out"][B - 64:], ref_out)
         smp.close()
+    # A bounding top_k whose rows have long lists all the same (flat rows, top_k 1000): the streaming finish
+    # says so to the policy in every call the row kernel suits, whatever its size (elsewhere only in calls of
+    # fewer than 2^24 tokens), and the calls after it go to the row kernel
+    B, V = 520, 50304
+    lg_np = H.logits_uniform(B, V, seed=77)
+    lg = torch.from_numpy(lg_np).cuda()
+    rc, c, kk, pp = capi.normalize(1.0, 1000, 1.0, V, B, 1)
+    u_np = H.uniforms(B, 65)
+    u = torch.from_numpy(u_np).cuda()
+    smp = capi.Sampler(B, V, with_policy=True, init=True)
+    first = smp.sample(lg, c, kk, pp, uniforms=u)
+    assert first["rc"] == 0 and (first["diag"]["rounds"] != 10).all() and smp.policy_state() == 2
+    res = smp.sample(lg, c, kk, pp, uniforms=u)
+    assert res["rc"] == 0 and (res["diag"]["rounds"] == 10).all() and smp.policy_state() == 2 and smp.status() == 0
+    ref_out, ref_diag = oracle.sample_batch(lg_np[:64], c, kk, pp, injected_u=u_np[:64])
+    for f in FIELDS:
+        assert np.array_equal(res["diag"][f], first["diag"][f]), f
+        assert np.array_equal(res["diag"][f][:64], ref_diag[f]), f
+    assert np.array_equal(res["out"], first["out"]) and np.array_equal(res["out"][:64], ref_out)
+    smp.close()
     # the library's own random numbers: drawn as on every other path, the state left as the oracle leaves it
     B, V = 130, 12288
     lg_np = H.logits_normal(B, V, 0.5, seed=51)
