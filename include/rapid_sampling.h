@@ -144,10 +144,12 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * rows (ties of thousands of tokens), without one (top_p < 1 alone) a flat
  * distribution (a call without a bounding top_k also counts a row as slow
  * when it is finished from a list of more than V/20, at least 2048, tokens:
- * the general kernel is faster for such calls; a call of fewer than 2^24
- * tokens with a bounding top_k counts a row as slow when its stashes hold
- * more tokens than the finishing workgroup's list and have to be gone through
- * twice more -- flat rows cut into many slices -- for the same reason).  The
+ * the general kernel is faster for such calls; a call with a bounding top_k
+ * does the same, and also counts a row as slow when its stashes hold more
+ * tokens than the finishing workgroup's list and have to be gone through
+ * twice more -- flat rows cut into many slices -- if it is of fewer than 2^24
+ * tokens or of a shape the row kernel takes, see rs_sample, which does such
+ * rows faster whatever the size of the call).  The
  * two-pass wide path (kept sets of any size, two passes over the logits) does a
  * row the slow way when its slices are no fair samples of the row; the one-pass
  * wide path (a sample of the row, then one pass over all of it; calls of at
@@ -158,7 +160,8 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * and rs_sample_ex reads that word, without waiting, before it routes the
  * next call: while it is set, calls of that kind go to the general kernel (a
  * call without a bounding top_k to a wide path when it is large enough, a call
- * that would take the one-pass wide path to the two-pass one);
+ * that would take the one-pass wide path to the two-pass one, calls of a
+ * shape the row kernel takes to the row kernel);
  * after 64 of them the path is tried again, each try that fails doubles that
  * number (up to 1024), and a run of good calls as long as the last stay away
  * puts it back to 64.  There is a word per KIND of call -- streaming with a
