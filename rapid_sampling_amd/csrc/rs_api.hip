@@ -235,6 +235,7 @@ static Geometry choose_geometry(int32_t B, int32_t V, bool pen, int force_r)
 // finishing workgroup handles quickly) unless the call is only a few of them.
 constexpr int kStreamNT = 256;
 constexpr uint32_t kStreamSmallParts = 1536;
+constexpr int32_t kMidMaxV = 262144;                          // rows up to here may be cut into slices of 8192 tokens whatever the call's size (wide_r)
 constexpr uint64_t kFusedSmall = 1ull << 22;
 static uint32_t stream_parts(int32_t V, int R) { return ((uint32_t)V / 4 + kStreamNT * R - 1) / (kStreamNT * R); }
 // `pen`: the pass that also reads penalties exists for the long slices only
@@ -272,7 +273,9 @@ static StreamLayout stream_layout(size_t parts, size_t base, bool with_pens = fa
 // path: at most kStreamSmallParts of them, of 4096 or of 8192 tokens; the one-launch path: calls of
 // at most kFusedSmall tokens, fewer than kFusedSmall / 4096 + B slices), so that the size grows
 // with B and with V and a workspace for the largest B and V serves every smaller call.
-static size_t stream_bytes(int32_t B, int32_t V)
+// (`least`: what every call needs; without it, also room for slices of 8192 tokens in rows of up to
+// 262144, which the one-pass wide path and the counting-only pass take when they are given it: see wide_r)
+static size_t stream_bytes(int32_t B, int32_t V, bool least)
 {
     const size_t longs = stream_layout((size_t)B * stream_parts(V, kStreamLongR), sizeof(WsHeader), true).end;
     size_t small_parts = (size_t)B * stream_parts(V, 4);
@@ -280,7 +283,26 @@ static size_t stream_bytes(int32_t B, int32_t V)
     static_assert(kStreamSmallParts >= kFusedSmall / 4096, "room for either kind of small call");
     if (small_parts > cap) small_parts = cap;
     const size_t shorts = stream_layout(small_parts, sizeof(WsHeader)).end;
-    return longs > shorts ? longs : shorts;
+    size_t bytes = longs > shorts ? longs : shorts;
+    if (!least) {
+        const size_t mids = stream_layout((size_t)B * stream_parts(V < kMidMaxV ? V : kMidMaxV, 8), sizeof(WsHeader)).end;
+        if (mids > bytes) bytes = mids;
+    }
+    return bytes;
+}
+// Slice length of the one-pass wide path and of the counting-only pass (plain temperature sampling): as
+// stream_r, but slices of 8192 tokens instead of 16384 in rows of up to 262144 tokens whenever the
+// workspace has room for them (a workspace of rs_workspace_bytes has).  Measured, us per call, 16384- against
+// 8192-token slices: one-pass wide path 128 x 100256 65 / 55, 128 x 262144 90 / 80, 256 x 131072 88 / 77,
+// 512 x 100256 128 / 110, 512 x 262144 210 / 191; counting-only pass with its finish 512 x 100256 60 / 51,
+// 512 x 131072 69 / 62, 512 x 262144 116 / 109.  (The pass with stashes gains nothing: 512 x 262144 110 / 117;
+// the two-pass wide path's counting pass 256 x 262144 161 / 168, 512 x 131072 159 / 153.)
+static int wide_r(int32_t B, int32_t V, size_t workspace_bytes)
+{
+    const int r = stream_r(B, V);
+    if (r != kStreamLongR || V > kMidMaxV) return r;
+    const size_t need = stream_layout((size_t)B * stream_parts(V, 8), sizeof(WsHeader)).end + (size_t)B * sizeof(RowCtl);
+    return need <= (workspace_bytes & ~(size_t)255) ? 8 : r;
 }
 
 }  // namespace rs
@@ -351,6 +373,12 @@ constexpr int32_t kWideMinV = 49152;
 // against 129; 512 x 262144: 228 against 290 and 211 against 231; 128 x 1048576: 233 against 263 and 192
 // against 226).
 constexpr uint64_t kWide1Min = 1ull << 26;
+// In rows of up to 262144 tokens the one-pass wide path works on slices of 8192 tokens (wide_r), which
+// moves its crossover with the general kernel down to about 12 million tokens per call (128 x 100256: 55
+// against 65 us; 128 x 131072: 60 against 66; 128 x 151936: 64 against 78; 64 x 262144: 62 against 65;
+// below: 64 x 131072 48 against 38, 32 x 262144 50 against 40) and puts it ahead of the two-pass path
+// everywhere above (256 x 131072: 77 against 94; 512 x 262144: 191 against 266).
+constexpr uint64_t kWide1MinMid = 12000000ull;
 constexpr uint64_t kPenStreamMin = 1ull << 23;
 // The row kernel (one workgroup per row, the row in its registers, one launch; rows of up to 65536 tokens, no
 // penalties) against what else there is for kept sets the stashes cannot hold, same rows, us per call:
@@ -466,7 +494,7 @@ static int choose_path(int32_t B, int32_t V, int32_t top_k, float top_p, bool pe
     auto wide_or_general = [&]() {
         const uint64_t tokens = (uint64_t)B * (uint64_t)V;
         if (row_suits(B, V)) return (int)kPathRow;
-        if (tokens >= kWide1Min && V >= kWideMinV && !routed_away(2)) return (int)kPathWide1;
+        if (tokens >= (V <= kMidMaxV ? kWide1MinMid : kWide1Min) && V >= kWideMinV && !routed_away(2)) return (int)kPathWide1;
         if (tokens >= kWideMin && V >= kWideMinV && !routed_away(3)) return (int)kPathWide;
         return (int)kPathCluster;
     };
@@ -549,7 +577,7 @@ int rs_workspace_bytes(int32_t B, int32_t V, size_t *bytes)
     if (!bytes) return RS_ERR_NULL;
     if (!(V > 0 && V <= 1048576 && V % 4 == 0)) return RS_ERR_VOCAB;
     if (B <= 0) return RS_ERR_BATCH;
-    *bytes = stream_bytes(B, V) + (size_t)B * sizeof(RowCtl);
+    *bytes = stream_bytes(B, V, false) + (size_t)B * sizeof(RowCtl);
     return RS_OK;
 }
 
@@ -714,8 +742,8 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     const int bad = check_call(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, log2e_inv_temp,
                                top_k, top_p, e_bits, opt);
     if (bad != RS_OK) return bad;
-    size_t need = 0;
-    rs_workspace_bytes(B, V, &need);
+    // (what the call cannot do without; rs_workspace_bytes asks for room for the shorter slices of wide_r on top)
+    const size_t need = stream_bytes(B, V, true) + (size_t)B * sizeof(RowCtl);
     if (workspace_bytes < need || ((uintptr_t)workspace & 255)) return RS_ERR_WORKSPACE;
     const int whole = device_is_whole();
     if (whole != RS_OK) return whole;
@@ -741,11 +769,15 @@ int rs_sample_ex(const void *logits, int32_t logits_dtype, int64_t row_stride, f
     const int path = choose_path(B, V, top_k, top_p, pen, opt);
     if (path == kPathRow) return launch_row(logits_dtype, (uint32_t)B, (hipStream_t)stream, p) == hipSuccess ? RS_OK : RS_ERR_LAUNCH;
     if (path != kPathCluster) {
-        const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED) : stream_r(B, V, pen);
+        const int sr = path == kPathFused ? fused_r(B, V, pen, opt && opt->path == RS_PATH_FUSED)
+                     : (path == kPathWide1 || path == kPathKeep) ? wide_r(B, V, workspace_bytes) : stream_r(B, V, pen);
         StreamView v;
         v.G = stream_parts(V, sr);
         const bool pen_stream = pen && path == kPathStream;                  // long slices: their layout has room for the notes
         const StreamLayout l = stream_layout((size_t)B * v.G, sizeof(WsHeader), pen_stream);
+        // (rs_workspace_bytes sets aside room for every slice length chosen above; checked all the same: a
+        // layout that ran into the rows' records would be written out of bounds by thousands of workgroups)
+        if (l.end + (size_t)B * sizeof(RowCtl) > (workspace_bytes & ~(size_t)255)) return RS_ERR_WORKSPACE;
         char *w = (char *)workspace;
         v.hdr = (PartHdr *)(w + l.hdr); v.stash = (uint64_t *)(w + l.stash); v.cum = (uint32_t *)(w + l.cum);
         v.shist = (uint64_t *)(w + l.shist);
@@ -855,9 +887,7 @@ int rs_sample_static(const void *logits, int32_t logits_dtype, int64_t row_strid
     const int bad = check_call(logits, logits_dtype, row_stride, penalties, out, rng_state, injected_u, B, V, log2e_inv_temp,
                                top_k, top_p, e_bits, opt);
     if (bad != RS_OK) return bad;
-    size_t need = 0;
-    const int rc = rs_workspace_bytes(B, V, &need);
-    if (rc != RS_OK) return rc;
+    const size_t need = stream_bytes(B, V, true) + (size_t)B * sizeof(RowCtl);  // what the call cannot do without
     if (need > (size_t)RS_STATIC_SCRATCH_BYTES) return RS_ERR_SCRATCH;
     const int whole = device_is_whole();
     if (whole != RS_OK) return whole;

@@ -89,7 +89,7 @@ def test_workspace_size_is_independent_of_t_monotone_and_bounded():
         for V in Vs:
             rc, n = capi.workspace_bytes(B, V)
             assert rc == 0 and n % 256 == 0
-            assert n <= 12 * 2 ** 20 + B * (65536 + 0.3 * 4 * V)
+            assert n <= 12 * 2 ** 20 + B * (65536 + 0.4 * 4 * V)
             sizes[B, V] = n
     for i, B in enumerate(Bs):
         for j, V in enumerate(Vs):

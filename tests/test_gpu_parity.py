@@ -305,14 +305,17 @@ def test_c5_full_size_paths_agree(torch_cuda, oracle):
 
 
 @pytest.mark.parametrize("B,T,V,top_k,top_p,gen", [(512, 1, 262144, -1, 0.9, "u1"), (128, 4, 1048576, 10000, 0.95, "n15"),
-                                                    (768, 1, 50304, 10000, 1.0, "u1")])
+                                                    (768, 1, 50304, 10000, 1.0, "u1"), (128, 1, 100256, 10000, 0.9, "u1"),
+                                                    (30, 1, 1048576, 10000, 1.0, "n15")])
 def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
     """Kept sets of thousands of tokens at scale (the reference's benchmark grid has top_k 10000 and top_p
     0.9 on flat generators, /root/reference/bench.py:34-35, :66-72; its search costs the same whatever the
     kept set, sampling.cu:261-329): 512 flat rows of 262144 tokens under top_p 0.9, the bandwidth
     configuration's 128 rows of a million tokens with top_k 10000, 768 flat rows of 50304 tokens.  The
     library takes a wide path for the long rows by itself -- the one-pass one from 2^26 tokens per call on
-    (diag.rounds == 9), the two-pass one below (7), every row: none done the slow way -- and the row kernel
+    and, in rows of up to 262144 tokens, which it cuts into slices of 8192 tokens, from 12 million
+    (diag.rounds == 9: 128 rows of 100256 tokens), the two-pass one below that in longer rows (7: 30 rows of a
+    million), every row: none done the slow way -- and the row kernel
     for the rows of 50304 tokens (10); every row goes through the oracle, and the general kernel, both wide
     paths and, where the rows fit it, the row kernel must agree in every field."""
     torch = torch_cuda
@@ -331,7 +334,7 @@ def test_wide_path_at_scale(torch_cuda, oracle, B, T, V, top_k, top_p, gen):
         r = smp.sample(lg, c, k, p, uniforms=u, path=path)
         assert r["rc"] == 0 and smp.status() == 0
         res[path] = r
-    auto_rounds = 10 if V <= 65536 else 9 if B * V >= 2 ** 26 else 7
+    auto_rounds = 10 if V <= 65536 else 9 if B * V >= (12000000 if V <= 262144 else 2 ** 26) else 7
     assert (res["auto"]["diag"]["rounds"] == auto_rounds).all(), np.unique(res["auto"]["diag"]["rounds"], return_counts=True)
     assert (res["wide"]["diag"]["rounds"] == 7).all()
     assert (res["wide1"]["diag"]["rounds"] == 9).all(), np.unique(res["wide1"]["diag"]["rounds"], return_counts=True)
@@ -495,7 +498,7 @@ def test_wide_path_reports_slow_rows(torch_cuda, oracle):
     tried again after 64 of them, and a call that goes well clears the word through the call after it."""
     torch = torch_cuda
     from tests import capi
-    B, V = 300, 131072
+    B, V = 30, 1048576                                   # (the two-pass path by itself: long rows, fewer than 2^26 tokens)
     good = H.logits_uniform(B, V, seed=71)
     bad = good.copy()
     bad[11] = np.sort(bad[11])

@@ -35,7 +35,10 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     # two calls in a row, the second smaller; then larger again, with penalties, and on the other paths
     shapes = [(8, 65536 + 4096, 50, 0.9, None, False), (3, 32768, 20, 0.8, None, False),
               (8, 65536 + 4096, 50, 0.9, None, False), (5, 131072, -1, 0.3, "attempt", False),
-              (6, 40960, 40, 0.95, None, True), (2, 8192, 5, 1.0, "cluster", False), (1, 262144, -1, 0.3, None, False)]
+              (6, 40960, 40, 0.95, None, True), (2, 8192, 5, 1.0, "cluster", False), (1, 262144, -1, 0.3, None, False),
+              # the one-pass wide path: in the static array, which has no room for this call's slices of 8192
+              # tokens, on slices of 16384; in a workspace of rs_workspace_bytes on the shorter ones -- same integers
+              (190, 100256, 10000, 1.0, None, False)]
     for n, (B, V, k_in, p_in, path, pen_on) in enumerate(shapes):
         lg_np = H.logits_normal(B, V, 2.5, seed=100 + n)
         u_np = H.uniforms(B, 200 + n)
