@@ -89,8 +89,12 @@ int rs_normalize_args(double temperature, int64_t top_k, double top_p,
  * streaming paths, about 1.05 bytes per token (per slice of 16384 tokens the
  * stash of its largest tokens, its counts and bins, and 4 KB for its note of
  * the non-zero penalties; up to 3.2 bytes per token for the first 6M tokens,
- * where slices are shorter); a quarter of the reference's scratch for large V.
- * It does not grow with T.
+ * where slices are shorter; 1.5 bytes per token in rows of up to 262144
+ * tokens, for the slices of 8192 tokens the one-pass wide path and the
+ * counting-only pass cut there); a quarter to two fifths of the reference's
+ * scratch.  It does not grow with T.  (A call is also accepted with a
+ * workspace that lacks the room for those slices of 8192 tokens -- the size
+ * versions before 414 asked for -- and then works on the long slices.)
  *
  * One workspace may serve calls of different shapes if it is at least
  * rs_workspace_bytes(largest B, largest V) of those calls and the same
@@ -153,7 +157,8 @@ int rs_workspace_where(const void *workspace_device, uint32_t where[4], void *st
  * two-pass wide path (kept sets of any size, two passes over the logits) does a
  * row the slow way when its slices are no fair samples of the row; the one-pass
  * wide path (a sample of the row, then one pass over all of it; calls of at
- * least 2^26 tokens) when the sample is no fair picture of the row (a few
+ * least 2^26 tokens, 12 million in rows of up to 262144) when the sample is
+ * no fair picture of the row (a few
  * tokens that carry most of the mass under top_p).  Calls that are
  * given a policy report "a row went the slow way: yes/no" to a word of pinned
  * host memory inside it (yes at once, no by the next call on the workspace),
@@ -243,11 +248,13 @@ int rs_philox_init(void *state_device, uint64_t seed, int32_t B, void *stream);
  * finish; see rs_policy; plain temperature sampling -- top_k = V, top_p = 1,
  * every token kept -- takes these two launches as well: the pass only counts,
  * and the finish reads one slice of the row again), four for kept sets of
- * thousands of tokens in calls of at least 3 * 2^23 tokens (the two-pass wide
+ * thousands of tokens in calls of at least 3 * 2^23 tokens in rows of more
+ * than 262144 tokens (the two-pass wide
  * path: the counting pass, a one-workgroup-per-row plan, a second pass over
  * the logits that counts the boundary bin's next digit and sets the tokens
  * around the expected threshold aside, a per-row finish), three for the same
- * from 2^26 tokens on (the one-pass wide path: a one-workgroup-per-row look at
+ * from 2^26 tokens on, and from 12 million tokens on in rows of 49152 to
+ * 262144 tokens (the one-pass wide path: a one-workgroup-per-row look at
  * a sample of the row, an eighth of it at most, one pass over the logits that
  * counts the row's bins and, finely, the range in which the sample expects the
  * threshold, and sets the tokens around it aside, a per-row finish that checks
@@ -343,8 +350,10 @@ int rs_sample_ex(const void *logits_device, int32_t logits_dtype, int64_t row_st
  *
  * The workspace is a static array in device memory inside the library,
  * RS_STATIC_SCRATCH_BYTES (32 MiB) on every GPU the library is used on, held
- * until the process ends.  A call whose rs_workspace_bytes(B, V) exceeds that
- * size is refused with RS_ERR_SCRATCH (64 rows of 152064 tokens need 16 MiB,
+ * until the process ends.  A call that cannot do with that much (what
+ * rs_workspace_bytes(B, V) asks for, less the room for slices of 8192 tokens
+ * in large calls, which such a call then does without)
+ * is refused with RS_ERR_SCRATCH (64 rows of 152064 tokens need 16 MiB,
  * 32 rows of 131072 tokens 14 MiB; 128 rows of 1048576 tokens, 105 MB, do not
  * fit).  Every check that can refuse a call -- arguments, alignment, size, the
  * device -- is made before anything is launched.  The call allocates nothing
