@@ -44,7 +44,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, vendor figure
 # HBM bytes per call of the bandwidth configuration from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs
 # summarised in the file named here, valid for the library version they were taken with: a library
 # that has moved on reports traffic as null rather than a stale figure.
-TRAFFIC_PROFILE = {"file": "profiles/bench_kernels_hbm_traffic_pmc.md", "rs_version": 414, "bytes": 573847962}
+TRAFFIC_PROFILE = {"file": "profiles/bench_kernels_hbm_traffic_pmc.md", "rs_version": 415, "bytes": 573847962}
 
 
 def event_times_us(torch, fn, steps, warmup):
