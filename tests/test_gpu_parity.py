@@ -392,6 +392,46 @@ def test_wide_path_unusual_rows(torch_cuda, oracle):
     assert rounds[1] in (8, 9) and rounds[2] in (8, 9) and rounds[3] == 8 and rounds[5] == 0, rounds
 
 
+def test_one_pass_wide_path_on_slices_of_8192_tokens_unusual_rows(torch_cuda, oracle):
+    """From 12 million tokens per call on, rows of up to 262144 tokens take the one-pass wide path on slices
+    of 8192 tokens (diag.rounds == 9) when the workspace has the room rs_workspace_bytes asks for.  The rows
+    of test_wide_path_unusual_rows twelve times over, 96 rows of 139264 tokens (17 slices each): sorted rows,
+    few distinct values, masked slices, one tie of all tokens, two populations; every row against the oracle,
+    the general kernel and the two-pass path equal in every field; rows the sample misjudges may go the slow
+    way (8), a tie of all tokens is finished from the row's bins (0)."""
+    torch = torch_cuda
+    from tests import capi
+    V, reps = 131072 + 8192, 12
+    rng = np.random.default_rng(124)
+    lg8 = rng.random((8, V), dtype=np.float32)
+    lg8[1] = np.sort(lg8[1])[::-1]
+    lg8[2] = np.sort(lg8[2])
+    lg8[3] = np.round(lg8[3] * 16) / 16
+    lg8[4, 16384:81920] = -np.inf
+    lg8[5] = 0.5
+    lg8[6] = (rng.standard_normal(V) * 1.5).astype(np.float32)
+    lg8[7, ::3] += 0.5
+    lg_np = np.tile(lg8, (reps, 1))
+    B = 8 * reps
+    lg = torch.from_numpy(lg_np).cuda()
+    u_np = H.uniforms(B, 66)
+    u = torch.from_numpy(u_np).cuda()
+    for (temp, k, p) in [(1.0, 10000, 1.0), (2.0, -1, 0.9)]:
+        rc, c, kk, pp = capi.normalize(temp, k, p, V, B, 1)
+        ref_out, ref_diag = oracle.sample_batch(lg_np, c, kk, pp, injected_u=u_np)
+        smp = capi.Sampler(B, V)
+        res = {}
+        for path in ("auto", "wide1", "wide", "cluster"):
+            print("short slices, unusual rows", temp, k, p, path, flush=True)
+            res[path] = smp.sample(lg, c, kk, pp, uniforms=u, path=path)
+            assert res[path]["rc"] == 0 and smp.status() == 0
+            _check(res[path], ref_out, ref_diag, "short slices T=%g k=%d p=%g path %s" % (temp, k, p, path))
+        rounds = res["auto"]["diag"]["rounds"]
+        assert np.isin(rounds, (0, 8, 9)).all() and (rounds == 9).sum() >= 4 * reps, np.unique(rounds, return_counts=True)
+        assert np.array_equal(rounds, res["wide1"]["diag"]["rounds"])
+        smp.close()
+
+
 def test_row_kernel_unusual_rows(torch_cuda, oracle):
     """The row kernel (one workgroup per row, the row in its registers) on rows that take each of its ways:
     a boundary bin of more tokens than its list holds (flat rows at a temperature of 2: every level counted
